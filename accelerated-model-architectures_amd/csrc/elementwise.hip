@@ -1,0 +1,229 @@
+// HBM-bound row kernels of the MoE path: top-k combine (forward and the router
+// weight gradient), the gather copy `group`, and stand-alone packed SwiGLU.
+// All move 16 bytes per lane per access and accumulate in fp32.
+#include "common.hpp"
+
+namespace {
+
+constexpr int EW_THREADS = 256;
+
+// y[t, c..c+7] = sum_j w[t, j] * in[t*k + j, c..c+7]
+template <typename ET>
+__global__ __launch_bounds__(EW_THREADS) void combine_kernel(const uint16_t *__restrict__ in, int64_t ld_in,
+                                                             const uint16_t *__restrict__ w, uint16_t *__restrict__ y,
+                                                             int64_t ldy, int64_t T, int k, int chunks_per_row) {
+    const int64_t g = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x;
+    if (g >= T * chunks_per_row) return;
+    const int64_t t = g / chunks_per_row;
+    const int c = (int)(g % chunks_per_row) * 8;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    for (int j = 0; j < k; ++j) {
+        const u32x4 v = *(const u32x4 *)(in + (t * k + j) * ld_in + c);
+        float s = 1.0f;
+        if (w) s = Elem<ET>::lo((uint32_t)w[t * k + j]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            acc[2 * q] += s * Elem<ET>::lo(v[q]);
+            acc[2 * q + 1] += s * Elem<ET>::hi(v[q]);
+        }
+    }
+    u32x4 o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) o[q] = Elem<ET>::pack(acc[2 * q], acc[2 * q + 1]);
+    *(u32x4 *)(y + t * ldy + c) = o;
+}
+
+// one wave per (t, j): d_w[t, j] = <in[t*k + j, :], dy[t, :]>
+template <typename ET>
+__global__ __launch_bounds__(EW_THREADS) void combine_bwd_kernel(const uint16_t *__restrict__ in, int64_t ld_in,
+                                                                 const uint16_t *__restrict__ dy, int64_t lddy,
+                                                                 uint16_t *__restrict__ d_w, int64_t Tk, int k, int H) {
+    const int lane = threadIdx.x % WAVE;
+    const int64_t row = (int64_t)blockIdx.x * (EW_THREADS / WAVE) + threadIdx.x / WAVE;
+    if (row >= Tk) return;
+    const int64_t t = row / k;
+    float acc = 0.f;
+    for (int c = lane * 8; c < H; c += WAVE * 8) {
+        const u32x4 a = *(const u32x4 *)(in + row * ld_in + c);
+        const u32x4 b = *(const u32x4 *)(dy + t * lddy + c);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            acc += Elem<ET>::lo(a[q]) * Elem<ET>::lo(b[q]);
+            acc += Elem<ET>::hi(a[q]) * Elem<ET>::hi(b[q]);
+        }
+    }
+#pragma unroll
+    for (int d = WAVE / 2; d > 0; d >>= 1) acc += __shfl_xor(acc, d);
+    if (lane == 0) d_w[row] = (uint16_t)(Elem<ET>::pack(acc, 0.f) & 0xffffu);
+}
+
+// out[n, :] = A[idx[n] / fan_out, :] * coeff[idx[n]]
+template <typename ET>
+__global__ __launch_bounds__(EW_THREADS) void group_kernel(const uint16_t *__restrict__ A, int64_t lda,
+                                                           const int64_t *__restrict__ idx, uint16_t *__restrict__ out,
+                                                           int64_t ldo, const uint16_t *__restrict__ coeff, int64_t M,
+                                                           int chunks_per_row, int fan_out) {
+    const int64_t g = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x;
+    if (g >= M * chunks_per_row) return;
+    const int64_t n = g / chunks_per_row;
+    const int c = (int)(g % chunks_per_row) * 8;
+    const int64_t s = idx[n];
+    u32x4 v = *(const u32x4 *)(A + (s / fan_out) * lda + c);
+    if (coeff) {
+        const float f = Elem<ET>::lo((uint32_t)coeff[s]);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] = Elem<ET>::pack(f * Elem<ET>::lo(v[q]), f * Elem<ET>::hi(v[q]));
+    }
+    *(u32x4 *)(out + n * ldo + c) = v;
+}
+
+// y[r, c..c+7] from x[r, 2c..2c+15]
+template <typename ET>
+__global__ __launch_bounds__(EW_THREADS) void swiglu_packed_fwd_kernel(const uint16_t *__restrict__ x, int64_t ldx,
+                                                                       uint16_t *__restrict__ y, int64_t ldy,
+                                                                       int64_t rows, int chunks_per_row) {
+    const int64_t g = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x;
+    if (g >= rows * chunks_per_row) return;
+    const int64_t r = g / chunks_per_row;
+    const int c = (int)(g % chunks_per_row) * 8;
+    const u32x4 a = *(const u32x4 *)(x + r * ldx + 2 * c);
+    const u32x4 b = *(const u32x4 *)(x + r * ldx + 2 * c + 8);
+    float h[8];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        float g0 = Elem<ET>::lo(a[q]), u0 = Elem<ET>::hi(a[q]);
+        float g1 = Elem<ET>::lo(b[q]), u1 = Elem<ET>::hi(b[q]);
+        h[q] = u0 * g0 * sigmoidf_fast(g0);
+        h[4 + q] = u1 * g1 * sigmoidf_fast(g1);
+    }
+    u32x4 o;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) o[q] = Elem<ET>::pack(h[2 * q], h[2 * q + 1]);
+    *(u32x4 *)(y + r * ldy + c) = o;
+}
+
+template <typename ET>
+__global__ __launch_bounds__(EW_THREADS) void swiglu_packed_bwd_kernel(const uint16_t *__restrict__ x, int64_t ldx,
+                                                                       const uint16_t *__restrict__ dy, int64_t lddy,
+                                                                       uint16_t *__restrict__ dx, int64_t lddx,
+                                                                       int64_t rows, int chunks_per_row) {
+    const int64_t g = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x;
+    if (g >= rows * chunks_per_row) return;
+    const int64_t r = g / chunks_per_row;
+    const int c = (int)(g % chunks_per_row) * 8;
+    const u32x4 d = *(const u32x4 *)(dy + r * lddy + c);
+    float dv[8];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        dv[2 * q] = Elem<ET>::lo(d[q]);
+        dv[2 * q + 1] = Elem<ET>::hi(d[q]);
+    }
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+        const u32x4 a = *(const u32x4 *)(x + r * ldx + 2 * c + 8 * half);
+        u32x4 o;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const float gg = Elem<ET>::lo(a[q]), uu = Elem<ET>::hi(a[q]), dd = dv[4 * half + q];
+            const float s = sigmoidf_fast(gg), silu = gg * s;
+            o[q] = Elem<ET>::pack(dd * uu * (s + silu * (1.f - s)), dd * silu);
+        }
+        *(u32x4 *)(dx + r * lddx + 2 * c + 8 * half) = o;
+    }
+}
+
+inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+inline int grid_for(int64_t work) { return (int)((work + EW_THREADS - 1) / EW_THREADS); }
+
+} // namespace
+
+#define DISPATCH_T(dtype, ...)                                      \
+    do {                                                            \
+        if ((dtype) == XMA_ROCM_BF16) {                             \
+            typedef __bf16 ET;                                       \
+            __VA_ARGS__;                                            \
+        } else {                                                    \
+            typedef _Float16 ET;                                     \
+            __VA_ARGS__;                                            \
+        }                                                           \
+    } while (0)
+
+extern "C" int xma_rocm_combine(const void *expert_out, int64_t ld_in, const void *w, void *y, int64_t ldy, int64_t T,
+                                int32_t k, int32_t H, int dtype, void *stream) {
+    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED, "combine: dtype %d", dtype);
+    XMA_REQUIRE(T >= 0 && k >= 1 && H >= 8 && H % 8 == 0 && ld_in % 8 == 0 && ldy % 8 == 0, XMA_ROCM_EINVAL,
+                "combine: T=%lld k=%d H=%d ld_in=%lld ldy=%lld (H, ld %% 8 == 0)", (long long)T, k, H, (long long)ld_in,
+                (long long)ldy);
+    XMA_REQUIRE(T == 0 || (expert_out && y && aligned16(expert_out) && aligned16(y)), XMA_ROCM_EINVAL,
+                "combine: null or misaligned pointer");
+    if (T == 0) return XMA_ROCM_OK;
+    const int cpr = H / 8;
+    XMA_REQUIRE(T * cpr < ((int64_t)1 << 31) * EW_THREADS, XMA_ROCM_EUNSUPPORTED, "combine: too large");
+    hipStream_t st = (hipStream_t)stream;
+    DISPATCH_T(dtype, (combine_kernel<ET><<<grid_for(T * cpr), EW_THREADS, 0, st>>>(
+                          (const uint16_t *)expert_out, ld_in, (const uint16_t *)w, (uint16_t *)y, ldy, T, k, cpr)));
+    return xma_check_launch("combine_kernel");
+}
+
+extern "C" int xma_rocm_combine_bwd(const void *expert_out, int64_t ld_in, const void *dy, int64_t lddy, void *d_w,
+                                    int64_t T, int32_t k, int32_t H, int dtype, void *stream) {
+    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED, "combine_bwd: dtype %d", dtype);
+    XMA_REQUIRE(T >= 0 && k >= 1 && H >= 8 && H % 8 == 0 && ld_in % 8 == 0 && lddy % 8 == 0, XMA_ROCM_EINVAL,
+                "combine_bwd: T=%lld k=%d H=%d", (long long)T, k, H);
+    XMA_REQUIRE(T == 0 || (expert_out && dy && d_w && aligned16(expert_out) && aligned16(dy)), XMA_ROCM_EINVAL,
+                "combine_bwd: null or misaligned pointer");
+    if (T == 0) return XMA_ROCM_OK;
+    const int64_t rows = T * k;
+    const int64_t blocks = (rows + (EW_THREADS / WAVE) - 1) / (EW_THREADS / WAVE);
+    XMA_REQUIRE(blocks < ((int64_t)1 << 31), XMA_ROCM_EUNSUPPORTED, "combine_bwd: too large");
+    hipStream_t st = (hipStream_t)stream;
+    DISPATCH_T(dtype, (combine_bwd_kernel<ET><<<(int)blocks, EW_THREADS, 0, st>>>(
+                          (const uint16_t *)expert_out, ld_in, (const uint16_t *)dy, lddy, (uint16_t *)d_w, rows, k, H)));
+    return xma_check_launch("combine_bwd_kernel");
+}
+
+extern "C" int xma_rocm_group(const void *A, int64_t lda, const int64_t *idx, void *out, int64_t ldo, const void *coeff,
+                              int64_t M, int32_t K, int32_t fan_out, int dtype, void *stream) {
+    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED, "group: dtype %d", dtype);
+    XMA_REQUIRE(M >= 0 && K >= 8 && K % 8 == 0 && lda % 8 == 0 && ldo % 8 == 0 && fan_out >= 1, XMA_ROCM_EINVAL,
+                "group: M=%lld K=%d fan_out=%d", (long long)M, K, fan_out);
+    XMA_REQUIRE(M == 0 || (A && idx && out && aligned16(A) && aligned16(out)), XMA_ROCM_EINVAL,
+                "group: null or misaligned pointer");
+    if (M == 0) return XMA_ROCM_OK;
+    const int cpr = K / 8;
+    hipStream_t st = (hipStream_t)stream;
+    DISPATCH_T(dtype, (group_kernel<ET><<<grid_for(M * cpr), EW_THREADS, 0, st>>>(
+                          (const uint16_t *)A, lda, idx, (uint16_t *)out, ldo, (const uint16_t *)coeff, M, cpr, fan_out)));
+    return xma_check_launch("group_kernel");
+}
+
+extern "C" int xma_rocm_swiglu_packed_forward(const void *x, int64_t ldx, void *y, int64_t ldy, int64_t rows,
+                                              int32_t cols_out, int dtype, void *stream) {
+    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED, "swiglu_packed: dtype %d", dtype);
+    XMA_REQUIRE(rows >= 0 && cols_out >= 8 && cols_out % 8 == 0 && ldx % 8 == 0 && ldy % 8 == 0, XMA_ROCM_EINVAL,
+                "swiglu_packed: rows=%lld cols_out=%d (cols_out %% 8 == 0)", (long long)rows, cols_out);
+    XMA_REQUIRE(rows == 0 || (x && y && aligned16(x) && aligned16(y)), XMA_ROCM_EINVAL,
+                "swiglu_packed: null or misaligned pointer");
+    if (rows == 0) return XMA_ROCM_OK;
+    const int cpr = cols_out / 8;
+    hipStream_t st = (hipStream_t)stream;
+    DISPATCH_T(dtype, (swiglu_packed_fwd_kernel<ET><<<grid_for(rows * cpr), EW_THREADS, 0, st>>>(
+                          (const uint16_t *)x, ldx, (uint16_t *)y, ldy, rows, cpr)));
+    return xma_check_launch("swiglu_packed_fwd_kernel");
+}
+
+extern "C" int xma_rocm_swiglu_packed_backward(const void *x, int64_t ldx, const void *dy, int64_t lddy, void *dx,
+                                               int64_t lddx, int64_t rows, int32_t cols_out, int dtype, void *stream) {
+    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED, "swiglu_packed_bwd: dtype %d",
+                dtype);
+    XMA_REQUIRE(rows >= 0 && cols_out >= 8 && cols_out % 8 == 0 && ldx % 8 == 0 && lddy % 8 == 0 && lddx % 8 == 0,
+                XMA_ROCM_EINVAL, "swiglu_packed_bwd: rows=%lld cols_out=%d", (long long)rows, cols_out);
+    XMA_REQUIRE(rows == 0 || (x && dy && dx && aligned16(x) && aligned16(dy) && aligned16(dx)), XMA_ROCM_EINVAL,
+                "swiglu_packed_bwd: null or misaligned pointer");
+    if (rows == 0) return XMA_ROCM_OK;
+    const int cpr = cols_out / 8;
+    hipStream_t st = (hipStream_t)stream;
+    DISPATCH_T(dtype, (swiglu_packed_bwd_kernel<ET><<<grid_for(rows * cpr), EW_THREADS, 0, st>>>(
+                          (const uint16_t *)x, ldx, (const uint16_t *)dy, lddy, (uint16_t *)dx, lddx, rows, cpr)));
+    return xma_check_launch("swiglu_packed_bwd_kernel");
+}

@@ -1,0 +1,43 @@
+"""continuous_count with the signature of the reference
+(xma/functional/continuous_count/__init__.py:15-51) and a ``rocm`` branch."""
+
+from __future__ import annotations
+
+import torch
+
+from ...accelerator import Accelerator, KernelBackend
+
+
+@torch.no_grad()
+def continuous_count(x: torch.Tensor, bins: int, *, kernel_backend: KernelBackend | None = None) -> torch.Tensor:
+    """Counts the occurrences of the values [0, bins) in ``x``; values outside
+    that range are the caller's responsibility (the rocm kernel ignores them,
+    ``bincount`` on the torch path does not).
+
+    :param x: 1-D int32 or int64 tensor
+    :param bins: number of bins
+    :param kernel_backend: KernelBackend.rocm | KernelBackend.torch | None (platform default)
+    :return: uint32 tensor of shape (bins,)
+    """
+    if bins == 1:
+        return torch.tensor([x.numel()], dtype=torch.uint32, device=x.device)
+
+    assert x.dim() == 1, "x should be 1-dimensional"
+    assert x.dtype in [torch.int32, torch.long]
+
+    if kernel_backend is None:
+        kernel_backend = Accelerator.get_kernel_backend()
+    else:
+        assert kernel_backend.verify_accelerator()
+
+    if kernel_backend == KernelBackend.rocm:
+        from ...rocm.ops import continuous_count_rocm
+
+        y = torch.zeros(bins, dtype=torch.uint32, device=x.device)
+        continuous_count_rocm(x=x.contiguous(), y=y)
+    elif kernel_backend == KernelBackend.torch:
+        y = x.bincount(minlength=bins).to(torch.uint32)
+    else:
+        raise ValueError(f"unexpected kernel_backend ({kernel_backend})")
+
+    return y

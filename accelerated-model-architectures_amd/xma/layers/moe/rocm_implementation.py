@@ -1,0 +1,215 @@
+"""KernelBackend.rocm implementation of the MoE expert computation.
+
+Mirrors the op-level interface of the reference's Triton implementation
+(xma/layers/moe/triton_implementation/__init__.py): ``scatter2scatter``,
+``group``, ``group_bwd_W`` and the two autograd Functions behind
+``up_projection_experts`` / ``down_projection_experts``; adds ``route`` (one op
+for sort + histogram + offsets) and ``fused_swiglu_experts`` (the whole expert
+computation with SwiGLU folded into the GEMM epilogues).
+
+Differences from the reference's data flow, all of which remove HBM passes:
+  * dW reads its gathered operand through the index instead of a materialised
+    ``grouped_x`` / ``grouped_grad_out`` copy, and writes every element of dW
+    (no zeros_like fill);
+  * the router-weight scaling of dy is applied inside the GEMMs;
+  * backward reuses the un-weighted expert outputs saved by forward instead of
+    recomputing them with another GEMM (triton_implementation/__init__.py:117-128);
+  * combine and its backward are dedicated coalesced kernels, not bmm.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from ...rocm import ops
+
+
+# ----------------------------------------------------------------------------------------- routing
+@torch.no_grad()
+def route(selected_experts: torch.Tensor, num_experts: int):
+    """(counts uint32 (E,), inclusive offsets int64 (E,), exclusive offsets int64 (E,),
+    sorted_expert_idxs, sorted_scattered_idxs int64) of the flattened (T, k) selection; stable order."""
+    ids = selected_experts.flatten().contiguous()
+    n, dev = ids.numel(), ids.device
+    counts = torch.empty(num_experts, dtype=torch.uint32, device=dev)
+    incl = torch.empty(num_experts, dtype=torch.int64, device=dev)
+    excl = torch.empty(num_experts, dtype=torch.int64, device=dev)
+    sorted_expert_idxs = torch.empty_like(ids)
+    sorted_scattered_idxs = torch.empty(n, dtype=torch.int64, device=dev)
+    workspace = torch.empty(ops.route_workspace_elements(n, num_experts), dtype=torch.int32, device=dev)
+    ops.route_rocm(ids, counts, incl, excl, sorted_expert_idxs, sorted_scattered_idxs, workspace)
+    return counts, incl, excl, sorted_expert_idxs, sorted_scattered_idxs
+
+
+# ----------------------------------------------------------------------------------------- op mirrors
+def scatter2scatter(
+    X: torch.Tensor,
+    W: torch.Tensor,
+    sorted_expert_idxs: torch.Tensor,
+    sorted_scattered_idxs: torch.Tensor,
+    out: torch.Tensor,
+    FAN_OUT: int,
+    x_grouped: bool = False,
+    y_grouped: bool = False,
+    expert_offsets: torch.Tensor | None = None,
+    row_scale: torch.Tensor | None = None,
+) -> None:
+    """Signature of the reference op (scatter_kernel.py:137-147) plus the inclusive ``expert_offsets`` the
+    expert-major tile schedule is derived from (computed from ``sorted_expert_idxs`` when not given)."""
+    assert sorted_scattered_idxs.size(0) == sorted_expert_idxs.size(0)
+    assert sorted_scattered_idxs.size(0) == X.size(0) * (1 if x_grouped else FAN_OUT)
+    assert out.size(0) == sorted_expert_idxs.size(0) and out.size(1) == W.size(-1)
+    if expert_offsets is None:
+        expert_offsets = torch.bincount(sorted_expert_idxs, minlength=W.size(0)).cumsum(-1)
+    ops.scatter2scatter_rocm(X, W, sorted_scattered_idxs, expert_offsets, out, row_scale, FAN_OUT, x_grouped, y_grouped)
+
+
+def group(
+    A: torch.Tensor,
+    sorted_expert_idxs: torch.Tensor,
+    out: torch.Tensor,
+    coeff: torch.Tensor | None = None,
+    fan_out: int = 1,
+) -> None:
+    """Signature of the reference op (group_kernel.py:69-76)."""
+    ops.group_rocm(A, sorted_expert_idxs, out, coeff, fan_out)
+
+
+def group_bwd_W(DY: torch.Tensor, X: torch.Tensor, expert_offsets: torch.Tensor, DW: torch.Tensor, E: int) -> None:
+    """Signature of the reference op (group_backward_kernel.py:102-103): both operands already grouped."""
+    assert DW.size(0) == E
+    idx = torch.empty(0, dtype=torch.int64, device=DY.device)
+    ops.group_bwd_W_rocm(DY, X, idx, expert_offsets, DW, None, 0, 0)
+
+
+def _empty_dw_like(expert_weights: torch.Tensor) -> torch.Tensor:
+    """Uninitialised gradient with the shape and strides of ``expert_weights`` ((E, in, out) view of
+    (E, out, in) storage); the dW kernel writes every element, so no zero fill is needed."""
+    return torch.empty_like(expert_weights)
+
+
+# ----------------------------------------------------------------------------------------- autograd
+class _UpProjectionExperts(torch.autograd.Function):
+    """x (T, H) -> grouped (T*k, out); counterpart of triton_implementation/__init__.py:12-72."""
+
+    @staticmethod
+    def forward(ctx, x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets):
+        output = torch.empty(sorted_expert_idxs.size(0), expert_weights.size(-1), device=x.device, dtype=x.dtype)
+        ops.scatter2scatter_rocm(x, expert_weights, sorted_scattered_idxs, expert_offsets, output, None, k, False, True)
+        ctx.save_for_backward(x, expert_weights, sorted_scattered_idxs, expert_offsets)
+        ctx.k = k
+        return output
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, expert_weights, sorted_scattered_idxs, expert_offsets = ctx.saved_tensors
+        k = ctx.k
+        grad_out = grad_out.contiguous()
+
+        d_weights = _empty_dw_like(expert_weights)
+        ops.group_bwd_W_rocm(grad_out, x, sorted_scattered_idxs, expert_offsets, d_weights, None, 0, k)
+
+        scattered = torch.empty(sorted_scattered_idxs.size(0), x.size(1), dtype=x.dtype, device=x.device)
+        ops.scatter2scatter_rocm(
+            grad_out, expert_weights.permute(0, 2, 1), sorted_scattered_idxs, expert_offsets, scattered, None, 1, True, False
+        )
+        d_input = torch.empty_like(x)
+        ops.combine_rocm(scattered, None, d_input, k)
+        return d_input, d_weights, None, None, None, None
+
+
+class _DownProjectionExperts(torch.autograd.Function):
+    """grouped h (T*k, I) -> y (T, H) = sum_j w[t, j] * expert_out[t*k + j]; counterpart of
+    triton_implementation/__init__.py:75-162 (there called with k = 1 and router_weights (T, top_k))."""
+
+    @staticmethod
+    def forward(ctx, x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, router_weights):
+        assert k == 1
+        T, top_k = router_weights.shape
+        expert_out = torch.empty(sorted_expert_idxs.size(0), expert_weights.size(-1), device=x.device, dtype=x.dtype)
+        ops.scatter2scatter_rocm(x, expert_weights, sorted_scattered_idxs, expert_offsets, expert_out, None, 1, True, False)
+        router_weights = router_weights.contiguous()
+        y = torch.empty(T, expert_out.size(1), device=x.device, dtype=x.dtype)
+        ops.combine_rocm(expert_out, router_weights, y, top_k)
+        ctx.save_for_backward(x, expert_weights, sorted_scattered_idxs, expert_offsets, router_weights, expert_out)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, expert_weights, sorted_scattered_idxs, expert_offsets, router_weights, expert_out = ctx.saved_tensors
+        top_k = router_weights.size(1)
+        grad_out = grad_out.contiguous()
+
+        d_router_weights = torch.empty_like(router_weights)
+        ops.combine_bwd_rocm(expert_out, grad_out, d_router_weights)
+
+        flat_w = router_weights.view(-1)
+        d_weights = _empty_dw_like(expert_weights)
+        ops.group_bwd_W_rocm(grad_out, x, sorted_scattered_idxs, expert_offsets, d_weights, flat_w, top_k, 0)
+
+        d_input = torch.empty_like(x)
+        ops.scatter2scatter_rocm(
+            grad_out, expert_weights.permute(0, 2, 1), sorted_scattered_idxs, expert_offsets, d_input, flat_w, top_k, False, True
+        )
+        return d_input, d_weights, None, None, None, None, d_router_weights
+
+
+class _FusedSwiGLUExperts(torch.autograd.Function):
+    """Whole expert computation with packed SwiGLU in the GEMM epilogues:
+    forward  up-projection (+ SwiGLU) -> down-projection (scattered) -> combine
+    backward combine' -> dX2 (+ SwiGLU') -> dW2, dW1 -> dX1 (scattered) -> k-way sum."""
+
+    @staticmethod
+    def forward(ctx, x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets):
+        # w_fc: (E, H, 2I) view, w_proj: (E, I, H) view (both permuted views of the parameters)
+        T, top_k = router_weights.shape
+        M = sorted_scattered_idxs.numel()
+        z = torch.empty(M, w_fc.size(-1), device=x.device, dtype=x.dtype)
+        h = torch.empty(M, w_fc.size(-1) // 2, device=x.device, dtype=x.dtype)
+        ops.up_projection_swiglu_rocm(x, w_fc, sorted_scattered_idxs, expert_offsets, z, h, top_k)
+        expert_out = torch.empty(M, w_proj.size(-1), device=x.device, dtype=x.dtype)
+        ops.scatter2scatter_rocm(h, w_proj, sorted_scattered_idxs, expert_offsets, expert_out, None, 1, True, False)
+        router_weights = router_weights.contiguous()
+        y = torch.empty(T, expert_out.size(1), device=x.device, dtype=x.dtype)
+        ops.combine_rocm(expert_out, router_weights, y, top_k)
+        ctx.save_for_backward(x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets, z, h, expert_out)
+        return y
+
+    @staticmethod
+    def backward(ctx, grad_out):
+        x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets, z, h, expert_out = ctx.saved_tensors
+        top_k = router_weights.size(1)
+        grad_out = grad_out.contiguous()
+        flat_w = router_weights.view(-1)
+
+        d_router_weights = torch.empty_like(router_weights)
+        ops.combine_bwd_rocm(expert_out, grad_out, d_router_weights)
+
+        dz = torch.empty_like(z)
+        ops.down_projection_dx_swiglu_rocm(
+            grad_out, w_proj.permute(0, 2, 1), sorted_scattered_idxs, expert_offsets, z, dz, flat_w, top_k
+        )
+        d_w_proj = _empty_dw_like(w_proj)
+        ops.group_bwd_W_rocm(grad_out, h, sorted_scattered_idxs, expert_offsets, d_w_proj, flat_w, top_k, 0)
+        d_w_fc = _empty_dw_like(w_fc)
+        ops.group_bwd_W_rocm(dz, x, sorted_scattered_idxs, expert_offsets, d_w_fc, None, 0, top_k)
+
+        scattered = expert_out.new_empty(expert_out.shape)
+        ops.scatter2scatter_rocm(dz, w_fc.permute(0, 2, 1), sorted_scattered_idxs, expert_offsets, scattered, None, 1, True, False)
+        d_x = torch.empty_like(x)
+        ops.combine_rocm(scattered, None, d_x, top_k)
+        return d_x, d_w_fc, d_w_proj, d_router_weights, None, None
+
+
+def up_projection_experts(x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets):
+    return _UpProjectionExperts.apply(x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets)
+
+
+def down_projection_experts(x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, router_weights):
+    return _DownProjectionExperts.apply(
+        x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, router_weights
+    )
+
+
+def fused_swiglu_experts(x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets):
+    return _FusedSwiGLUExperts.apply(x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets)

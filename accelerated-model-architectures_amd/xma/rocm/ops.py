@@ -1,0 +1,287 @@
+"""torch.library custom ops over the C ABI of libxma_rocm.so.
+
+Same shape as the reference's op boundary (xma/custom_op.py:72-108): every op
+is a ``torch.library.custom_op`` that mutates caller-allocated outputs and
+returns nothing, so autograd Functions and ``torch.compile`` see ordinary ops.
+The Python side validates shapes/dtypes/contiguity and raises like the
+reference (asserts), then hands raw device pointers, sizes, strides and the
+current HIP stream to the library.  The stream is looked up per call because
+backward runs on autograd's thread.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from .loader import check, get_library
+
+
+_DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1}
+
+EPI_STORE, EPI_SWIGLU, EPI_SWIGLU_BWD = 0, 1, 2
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _ptr(t: torch.Tensor | None) -> int | None:
+    return None if t is None else t.data_ptr()
+
+
+def _code(t: torch.Tensor) -> int:
+    if t.dtype not in _DTYPE_CODE:
+        raise NotImplementedError(f"KernelBackend.rocm covers bfloat16 and float16, got {t.dtype}")
+    return _DTYPE_CODE[t.dtype]
+
+
+def _rows(t: torch.Tensor, name: str) -> int:
+    """leading dimension of a 2-D row-major tensor"""
+    assert t.dim() == 2 and t.is_cuda, f"{name} should be a 2-D device tensor"
+    assert t.stride(1) == 1 or t.size(1) == 1, f"{name} should have contiguous rows"
+    return t.stride(0) if t.size(0) > 1 else max(t.size(1), t.stride(0))
+
+
+def _weight_layout(W: torch.Tensor) -> tuple[int, int, int]:
+    """W is logically (E, K, N) as in the reference's scatter2scatter.  Returns
+    (w_is_kn, expert stride, leading dimension) of its storage."""
+    assert W.dim() == 3 and W.is_cuda
+    E, K, N = W.shape
+    if W.stride(1) == 1 and (W.stride(2) >= K or N == 1):  # permuted view of (E, N, K): x @ W[e]^T form
+        return 0, W.stride(0), W.stride(2)
+    assert W.stride(2) == 1, "expert weights should be contiguous along K or along N"
+    return 1, W.stride(0), W.stride(1)
+
+
+# --------------------------------------------------------------------------- a1
+@torch.library.custom_op("xma_rocm::continuous_count", mutates_args={"y"})
+def continuous_count_rocm(x: torch.Tensor, y: torch.Tensor) -> None:
+    """y (uint32, zero-filled by the caller) += histogram of x
+    (reference op: _continuous_count_cuda, continuous_count/cuda_implementation.py:171-197)."""
+    assert x.is_cuda and y.is_cuda and x.dim() == 1 and x.is_contiguous() and y.is_contiguous()
+    assert x.dtype in (torch.int32, torch.int64) and y.dtype == torch.uint32
+    lib = get_library()
+    check(
+        lib.xma_rocm_continuous_count(_ptr(x), int(x.dtype == torch.int64), x.numel(), _ptr(y), y.numel(), _stream(x)),
+        "xma_rocm_continuous_count",
+    )
+
+
+# --------------------------------------------------------------------------- a2
+def route_workspace_elements(n: int, num_experts: int) -> int:
+    return (get_library().xma_rocm_route_workspace_bytes(n, num_experts) + 3) // 4
+
+
+@torch.library.custom_op(
+    "xma_rocm::route",
+    mutates_args={"counts", "offsets_inclusive", "offsets_exclusive", "sorted_expert_idxs", "sorted_scattered_idxs", "workspace"},
+)
+def route_rocm(
+    ids: torch.Tensor,
+    counts: torch.Tensor,
+    offsets_inclusive: torch.Tensor,
+    offsets_exclusive: torch.Tensor,
+    sorted_expert_idxs: torch.Tensor,
+    sorted_scattered_idxs: torch.Tensor,
+    workspace: torch.Tensor,
+) -> None:
+    """counts / offsets / stable expert-major permutation of ``ids`` in one op
+    (replaces sort + continuous_count + cumsum, moe/__init__.py:210-217)."""
+    E = counts.numel()
+    assert ids.is_cuda and ids.dim() == 1 and ids.is_contiguous() and ids.dtype in (torch.int32, torch.int64)
+    assert counts.dtype == torch.uint32 and offsets_inclusive.dtype == torch.int64 and offsets_exclusive.dtype == torch.int64
+    assert offsets_inclusive.numel() == E and offsets_exclusive.numel() == E
+    assert sorted_expert_idxs.dtype == ids.dtype and sorted_expert_idxs.numel() == ids.numel()
+    assert sorted_scattered_idxs.dtype == torch.int64 and sorted_scattered_idxs.numel() == ids.numel()
+    assert workspace.dtype == torch.int32 and workspace.is_contiguous()
+    lib = get_library()
+    check(
+        lib.xma_rocm_route(
+            _ptr(ids), int(ids.dtype == torch.int64), ids.numel(), E, _ptr(counts), _ptr(offsets_inclusive),
+            _ptr(offsets_exclusive), _ptr(sorted_expert_idxs), _ptr(sorted_scattered_idxs), _ptr(workspace),
+            workspace.numel() * 4, _stream(ids),
+        ),
+        "xma_rocm_route",
+    )
+
+
+# --------------------------------------------------------------------------- a5 a7 a8 a10
+def _scatter2scatter(X, W, idx, offs, out, aux, scale, fan_out, x_grouped, y_grouped, epilogue, M, N, K):
+    w_is_kn, w_es, ldw = _weight_layout(W)
+    assert W.dtype == X.dtype
+    assert idx.dtype == torch.int64 and idx.is_contiguous() and offs.dtype == torch.int64 and offs.is_contiguous()
+    assert offs.numel() == W.size(0)
+    if scale is not None:
+        assert scale.dtype == X.dtype and scale.is_contiguous()
+    lib = get_library()
+    check(
+        lib.xma_rocm_scatter2scatter(
+            _ptr(X), _rows(X, "X"), _ptr(W), w_es, ldw, w_is_kn, _ptr(idx), _ptr(offs),
+            _ptr(out), 0 if out is None else _rows(out, "out"), _ptr(aux), 0 if aux is None else _rows(aux, "aux"),
+            _ptr(scale), M, N, K, W.size(0), fan_out, int(x_grouped), int(y_grouped), epilogue, _code(X), _stream(X),
+        ),
+        "xma_rocm_scatter2scatter",
+    )
+
+
+@torch.library.custom_op("xma_rocm::scatter2scatter", mutates_args={"out"})
+def scatter2scatter_rocm(
+    X: torch.Tensor,
+    W: torch.Tensor,
+    sorted_scattered_idxs: torch.Tensor,
+    expert_offsets: torch.Tensor,
+    out: torch.Tensor,
+    row_scale: torch.Tensor | None,
+    FAN_OUT: int,
+    x_grouped: bool,
+    y_grouped: bool,
+) -> None:
+    """out[dst(n)] = X[src(n)] @ W[e(n)] (* row_scale[idx[n]]), W logically (E, K, N)."""
+    M = sorted_scattered_idxs.numel()
+    E, K, N = W.shape
+    assert X.size(1) == K and out.size(1) == N and out.size(0) == M
+    assert X.size(0) * (1 if x_grouped else FAN_OUT) == M
+    _scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, None, row_scale, FAN_OUT, x_grouped, y_grouped,
+                     EPI_STORE, M, N, K)
+
+
+@torch.library.custom_op("xma_rocm::up_projection_swiglu", mutates_args={"z", "h"})
+def up_projection_swiglu_rocm(
+    X: torch.Tensor,
+    W: torch.Tensor,
+    sorted_scattered_idxs: torch.Tensor,
+    expert_offsets: torch.Tensor,
+    z: torch.Tensor,
+    h: torch.Tensor,
+    FAN_OUT: int,
+) -> None:
+    """z (grouped pre-activations, (Tk, 2I)) and h = swiglu_packed(z) (Tk, I) in one GEMM."""
+    M = sorted_scattered_idxs.numel()
+    E, K, N = W.shape
+    assert X.size(1) == K and X.size(0) * FAN_OUT == M
+    assert z.shape == (M, N) and h.shape == (M, N // 2) and N % 2 == 0
+    _scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, z, h, None, FAN_OUT, False, True, EPI_SWIGLU, M, N, K)
+
+
+@torch.library.custom_op("xma_rocm::down_projection_dx_swiglu", mutates_args={"dz"})
+def down_projection_dx_swiglu_rocm(
+    dY: torch.Tensor,
+    W: torch.Tensor,
+    sorted_scattered_idxs: torch.Tensor,
+    expert_offsets: torch.Tensor,
+    z: torch.Tensor,
+    dz: torch.Tensor,
+    row_scale: torch.Tensor,
+    FAN_OUT: int,
+) -> None:
+    """dz = swiglu_packed'(z) * ((dY[idx // k] * w[idx]) @ W[e]); W logically (E, H, I), dY is (T, H)."""
+    M = sorted_scattered_idxs.numel()
+    E, K, N = W.shape
+    assert dY.size(1) == K and dY.size(0) * FAN_OUT == M
+    assert z.shape == (M, 2 * N) and dz.shape == (M, 2 * N)
+    _scatter2scatter(dY, W, sorted_scattered_idxs, expert_offsets, dz, z, row_scale, FAN_OUT, False, True,
+                     EPI_SWIGLU_BWD, M, N, K)
+
+
+@torch.library.custom_op("xma_rocm::group_bwd_W", mutates_args={"DW"})
+def group_bwd_W_rocm(
+    DY: torch.Tensor,
+    X: torch.Tensor,
+    sorted_scattered_idxs: torch.Tensor,
+    expert_offsets: torch.Tensor,
+    DW: torch.Tensor,
+    dy_scale: torch.Tensor | None,
+    dy_fan_out: int,
+    x_fan_out: int,
+) -> None:
+    """DW[e] = sum_n DY[dsrc(n)]^T X[xsrc(n)].  DW is logically (E, K_in, N_out) with the storage of the
+    parameter (E, N_out, K_in), as the reference's zeros_like(weight.permute(0, 2, 1)).  A fan_out of 0
+    marks an operand that is already in grouped order."""
+    E, K_in, N_out = DW.shape
+    assert DW.stride(1) == 1 and DW.is_cuda, "DW should be a permuted view of (E, N_out, K_in) storage"
+    assert DY.size(1) == N_out and X.size(1) == K_in and DY.dtype == X.dtype == DW.dtype
+    assert expert_offsets.numel() == E and expert_offsets.dtype == torch.int64
+    assert sorted_scattered_idxs.dtype == torch.int64 and sorted_scattered_idxs.is_contiguous()
+    if dy_scale is not None:
+        assert dy_scale.dtype == DY.dtype and dy_scale.is_contiguous()
+    lib = get_library()
+    check(
+        lib.xma_rocm_group_bwd_W(
+            _ptr(DY), _rows(DY, "DY"), int(dy_fan_out == 0), max(dy_fan_out, 1), _ptr(dy_scale),
+            _ptr(X), _rows(X, "X"), int(x_fan_out == 0), max(x_fan_out, 1),
+            _ptr(sorted_scattered_idxs), _ptr(expert_offsets), _ptr(DW), DW.stride(0), DW.stride(2),
+            N_out, K_in, E, _code(X), _stream(X),
+        ),
+        "xma_rocm_group_bwd_W",
+    )
+
+
+@torch.library.custom_op("xma_rocm::group", mutates_args={"out"})
+def group_rocm(A: torch.Tensor, sorted_expert_idxs: torch.Tensor, out: torch.Tensor, coeff: torch.Tensor | None, fan_out: int) -> None:
+    """out[n] = A[idx[n] // fan_out] * coeff[idx[n]] (reference: group_kernel.py:69-100; the index argument
+    keeps the reference's name although it receives sorted_scattered_idxs)."""
+    M, K = out.shape
+    assert A.size(1) == K and sorted_expert_idxs.numel() == M and sorted_expert_idxs.dtype == torch.int64
+    if coeff is not None:
+        assert coeff.dtype == A.dtype and coeff.is_contiguous()
+    lib = get_library()
+    check(
+        lib.xma_rocm_group(_ptr(A), _rows(A, "A"), _ptr(sorted_expert_idxs), _ptr(out), _rows(out, "out"), _ptr(coeff),
+                           M, K, fan_out, _code(A), _stream(A)),
+        "xma_rocm_group",
+    )
+
+
+# --------------------------------------------------------------------------- combine
+@torch.library.custom_op("xma_rocm::combine", mutates_args={"y"})
+def combine_rocm(expert_out: torch.Tensor, w: torch.Tensor | None, y: torch.Tensor, k: int) -> None:
+    """y[t] = sum_j w[t, j] * expert_out[t * k + j]  (w None: plain sum over the k slots)."""
+    T, H = y.shape
+    assert expert_out.shape == (T * k, H) and expert_out.dtype == y.dtype
+    if w is not None:
+        assert w.shape == (T, k) and w.is_contiguous() and w.dtype == y.dtype
+    lib = get_library()
+    check(
+        lib.xma_rocm_combine(_ptr(expert_out), _rows(expert_out, "expert_out"), _ptr(w), _ptr(y), _rows(y, "y"), T, k, H,
+                             _code(y), _stream(y)),
+        "xma_rocm_combine",
+    )
+
+
+@torch.library.custom_op("xma_rocm::combine_bwd", mutates_args={"d_w"})
+def combine_bwd_rocm(expert_out: torch.Tensor, dy: torch.Tensor, d_w: torch.Tensor) -> None:
+    """d_w[t, j] = <expert_out[t * k + j], dy[t]>."""
+    T, k = d_w.shape
+    H = dy.size(1)
+    assert expert_out.shape == (T * k, H) and dy.shape == (T, H) and d_w.is_contiguous()
+    assert expert_out.dtype == dy.dtype == d_w.dtype
+    lib = get_library()
+    check(
+        lib.xma_rocm_combine_bwd(_ptr(expert_out), _rows(expert_out, "expert_out"), _ptr(dy), _rows(dy, "dy"), _ptr(d_w),
+                                 T, k, H, _code(dy), _stream(dy)),
+        "xma_rocm_combine_bwd",
+    )
+
+
+# --------------------------------------------------------------------------- stand-alone packed SwiGLU
+@torch.library.custom_op("xma_rocm::swiglu_packed_forward", mutates_args={"y"})
+def swiglu_packed_forward_rocm(x: torch.Tensor, y: torch.Tensor) -> None:
+    rows, cols = y.shape
+    assert x.shape == (rows, 2 * cols) and x.dtype == y.dtype
+    lib = get_library()
+    check(
+        lib.xma_rocm_swiglu_packed_forward(_ptr(x), _rows(x, "x"), _ptr(y), _rows(y, "y"), rows, cols, _code(x), _stream(x)),
+        "xma_rocm_swiglu_packed_forward",
+    )
+
+
+@torch.library.custom_op("xma_rocm::swiglu_packed_backward", mutates_args={"dx"})
+def swiglu_packed_backward_rocm(x: torch.Tensor, dy: torch.Tensor, dx: torch.Tensor) -> None:
+    rows, cols = dy.shape
+    assert x.shape == (rows, 2 * cols) and dx.shape == x.shape and x.dtype == dy.dtype == dx.dtype
+    lib = get_library()
+    check(
+        lib.xma_rocm_swiglu_packed_backward(_ptr(x), _rows(x, "x"), _ptr(dy), _rows(dy, "dy"), _ptr(dx), _rows(dx, "dx"),
+                                            rows, cols, _code(x), _stream(x)),
+        "xma_rocm_swiglu_packed_backward",
+    )

@@ -1,0 +1,161 @@
+/*
+ * xma_rocm.h - C ABI of libxma_rocm.so: the MI355X (gfx950) kernels behind
+ * KernelBackend.rocm for XMA's MoE layer and continuous_count.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller (PyTorch's caching
+ *     allocator in the Python host); the library allocates nothing and keeps no
+ *     state between calls;
+ *   - `stream` is a hipStream_t passed as void*; all work is enqueued on it and
+ *     no entry point synchronises;
+ *   - return value 0 = enqueued, negative = XMA_ROCM_E* (argument errors are
+ *     detected before anything is launched; launch errors come from
+ *     hipGetLastError right after the launch); xma_rocm_last_error() gives the
+ *     message of the calling thread's last failure;
+ *   - `dtype` is XMA_ROCM_BF16 or XMA_ROCM_F16 (fp32 accumulation in both);
+ *   - leading dimensions (ld*) and expert strides are in ELEMENTS;
+ *   - "grouped" order = position n in the expert-sorted list; "scattered" order
+ *     = row sorted_scattered_idxs[n] of the flattened (T, k) selection.
+ *
+ * Citations are to the reference tree (xma/...), which each entry point replaces.
+ */
+#ifndef XMA_ROCM_H
+#define XMA_ROCM_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define XMA_ROCM_ABI_VERSION 1
+
+/* the library is built with hidden visibility; only these entry points are exported */
+#define XMA_API __attribute__((visibility("default")))
+
+#define XMA_ROCM_OK 0
+#define XMA_ROCM_EINVAL (-1)       /* bad argument (null pointer, size, alignment) */
+#define XMA_ROCM_EUNSUPPORTED (-2) /* shape or dtype the kernels do not cover */
+#define XMA_ROCM_EWORKSPACE (-3)   /* workspace smaller than *_workspace_bytes */
+#define XMA_ROCM_ELAUNCH (-4)      /* HIP reported an error at launch */
+
+#define XMA_ROCM_BF16 0
+#define XMA_ROCM_F16 1
+
+/* epilogues of xma_rocm_scatter2scatter */
+#define XMA_ROCM_EPI_STORE 0      /* out = acc (optionally * row_scale) */
+#define XMA_ROCM_EPI_SWIGLU 1     /* up-projection: out = z (pre-activation, may be NULL), aux = swiglu_packed(z) */
+#define XMA_ROCM_EPI_SWIGLU_BWD 2 /* down-projection dX: aux = saved z, out = dz = swiglu_packed'(z) * (acc * row_scale) */
+
+XMA_API int xma_rocm_abi_version(void);
+XMA_API const char *xma_rocm_last_error(void);
+
+/*
+ * Histogram of ids in [0, bins): counts[b] += #{i : ids[i] == b}.  ids outside
+ * the range are ignored.  Like the reference kernel the result is ACCUMULATED
+ * into `counts`, which the caller zero-fills first.
+ * Replaces _continuous_count_cuda, xma/functional/continuous_count/cuda_implementation.py:171-197
+ * (called from xma/functional/continuous_count/__init__.py:43-45).
+ */
+XMA_API int xma_rocm_continuous_count(const void *ids, int ids_are_int64, int64_t n, uint32_t *counts, int32_t bins,
+                              void *stream);
+
+/*
+ * Routing in one op: counts, inclusive/exclusive expert offsets and the STABLE
+ * expert-major permutation of the flattened top-k selection.
+ * Replaces `selected_experts.flatten().sort()` + continuous_count + cumsum,
+ * xma/layers/moe/__init__.py:210-217.
+ *   ids                    (n,)  int32|int64 expert id of each (token, slot)
+ *   counts                 (E,)  uint32, overwritten
+ *   offsets_inclusive      (E,)  int64, cumsum(counts)
+ *   offsets_exclusive      (E,)  int64, may be NULL
+ *   sorted_expert_idxs     (n,)  same dtype as ids, may be NULL
+ *   sorted_scattered_idxs  (n,)  int64
+ * ids must lie in [0, E); E <= 2048.
+ */
+XMA_API size_t xma_rocm_route_workspace_bytes(int64_t n, int32_t num_experts);
+XMA_API int xma_rocm_route(const void *ids, int ids_are_int64, int64_t n, int32_t num_experts, uint32_t *counts,
+                   int64_t *offsets_inclusive, int64_t *offsets_exclusive, void *sorted_expert_idxs,
+                   int64_t *sorted_scattered_idxs, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Grouped GEMM with fused row gather / scatter: for every expert e and every
+ * grouped position n in [offsets[e-1], offsets[e]):
+ *     acc[n, :] = X[src(n), :K] @ B_e            B_e = W[e]^T  if !w_is_kn   (W[e] is (N, K), K contiguous)
+ *                                                B_e = W[e]    if  w_is_kn   (W[e] is (K, N), N contiguous)
+ *     src(n)  = n                         if x_grouped else sorted_scattered_idxs[n] / fan_out
+ *     dst(n)  = n                         if y_grouped else sorted_scattered_idxs[n]
+ * followed by the epilogue (XMA_ROCM_EPI_*).  row_scale (may be NULL) is a
+ * vector indexed in scattered order (the flattened (T, k) router weights).
+ * Replaces scatter2scatter, xma/layers/moe/triton_implementation/scatter_kernel.py:137-183
+ * (kernel :58-134), the separate activation pass xma/layers/moe/__init__.py:226
+ * and its autograd backward, and the coefficient pass of `group`
+ * (xma/layers/moe/triton_implementation/__init__.py:134-140).
+ * Requirements: K % 8 == 0, N % 8 == 0, ld* % 8 == 0, 16-byte aligned bases.
+ *   EPI_STORE       out (M, N)
+ *   EPI_SWIGLU      out (M, N) = z or NULL;  aux (M, N/2) = h
+ *   EPI_SWIGLU_BWD  aux (M, 2N) = z (read, grouped order);  out (M, 2N) = dz;  requires y_grouped
+ */
+XMA_API int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *W, int64_t w_expert_stride, int64_t ldw,
+                             int w_is_kn, const int64_t *sorted_scattered_idxs, const int64_t *expert_offsets,
+                             void *out, int64_t ldo, void *aux, int64_t ldaux, const void *row_scale, int64_t M,
+                             int32_t N, int32_t K, int32_t num_experts, int32_t fan_out, int x_grouped,
+                             int y_grouped, int epilogue, int dtype, void *stream);
+
+/*
+ * Weight gradient of a grouped linear: for every expert e
+ *     DW[e] (N_out, K_in) = sum_{n in expert e} DY[dsrc(n), :N_out]^T  X[xsrc(n), :K_in]
+ *     dsrc(n) = n if dy_grouped else sorted_scattered_idxs[n] / dy_fan_out   (then scaled by dy_scale[idx[n]] if given)
+ *     xsrc(n) = n if x_grouped  else sorted_scattered_idxs[n] / x_fan_out
+ * Every element of DW is written exactly once (zeros for experts with no
+ * rows), fp32 accumulation over the expert's whole row range, no atomics.
+ * Replaces group_bwd_W, xma/layers/moe/triton_implementation/group_backward_kernel.py:102-128
+ * (kernel :21-99), the zeros_like fill (triton_implementation/__init__.py:49,142)
+ * and the `group` gather copies that feed it (:46-47, :134-140).
+ * DW has the storage layout of the parameter, (E, N_out, K_in) row-major.
+ */
+XMA_API int xma_rocm_group_bwd_W(const void *DY, int64_t lddy, int dy_grouped, int32_t dy_fan_out, const void *dy_scale,
+                         const void *X, int64_t ldx, int x_grouped, int32_t x_fan_out,
+                         const int64_t *sorted_scattered_idxs, const int64_t *expert_offsets, void *DW,
+                         int64_t dw_expert_stride, int64_t lddw, int32_t N_out, int32_t K_in, int32_t num_experts,
+                         int dtype, void *stream);
+
+/*
+ * Gather copy: out[n, :] = A[idx[n] / fan_out, :] * (coeff ? coeff[idx[n]] : 1), n < M.
+ * Replaces group, xma/layers/moe/triton_implementation/group_kernel.py:69-100.
+ */
+XMA_API int xma_rocm_group(const void *A, int64_t lda, const int64_t *idx, void *out, int64_t ldo, const void *coeff,
+                   int64_t M, int32_t K, int32_t fan_out, int dtype, void *stream);
+
+/*
+ * Top-k combine: y[t, :] = sum_j (w ? w[t, j] : 1) * expert_out[t * k + j, :], fp32 accumulation.
+ * Replaces the bmm of xma/layers/moe/triton_implementation/__init__.py:100-101
+ * and, with w == NULL, the `.sum(-2)` reductions of :70 and :160.
+ */
+XMA_API int xma_rocm_combine(const void *expert_out, int64_t ld_in, const void *w, void *y, int64_t ldy, int64_t T,
+                     int32_t k, int32_t H, int dtype, void *stream);
+
+/*
+ * Combine backward w.r.t. the router weights:
+ *     d_w[t, j] = <expert_out[t * k + j, :], dy[t, :]>
+ * Replaces the bmm of xma/layers/moe/triton_implementation/__init__.py:130-131.
+ */
+XMA_API int xma_rocm_combine_bwd(const void *expert_out, int64_t ld_in, const void *dy, int64_t lddy, void *d_w, int64_t T,
+                         int32_t k, int32_t H, int dtype, void *stream);
+
+/*
+ * Stand-alone packed SwiGLU (gate = even columns, up = odd columns), fp32 math:
+ *     y[r, c] = u * g * sigmoid(g),  g = x[r, 2c], u = x[r, 2c + 1]
+ * and its closed-form backward.  Replaces xma/functional/swiglu/torch_implementation.py:21-30
+ * and xma/functional/swiglu/triton_implementation/backward.py:14-23 for the packed layout.
+ */
+XMA_API int xma_rocm_swiglu_packed_forward(const void *x, int64_t ldx, void *y, int64_t ldy, int64_t rows, int32_t cols_out,
+                                   int dtype, void *stream);
+XMA_API int xma_rocm_swiglu_packed_backward(const void *x, int64_t ldx, const void *dy, int64_t lddy, void *dx,
+                                    int64_t lddx, int64_t rows, int32_t cols_out, int dtype, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XMA_ROCM_H */

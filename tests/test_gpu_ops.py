@@ -1,0 +1,146 @@
+"""GPU parity of the MoE ops (grouped GEMMs, dW, group, combine) through the C ABI against the
+op-level oracle.  Tolerance: max-abs-normalised error <= 1e-2 for bf16/fp16 results with fp32
+accumulation (the bar of the north star); operands are bit-identical on both sides."""
+
+import pytest
+import torch
+
+from oracle import moe as oracle
+from tests.utils import nerr
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+
+def _routing(T, E, k, seed, skew=0.0, empty=()):
+    g = torch.Generator().manual_seed(seed)
+    logits = torch.randn(T, E, generator=g) + skew * torch.randn(E, generator=g)
+    for e in empty:
+        logits[:, e] = -1e9
+    sel = logits.topk(k, dim=-1).indices
+    se, ss = sel.flatten().sort(stable=True)
+    offs = torch.bincount(se, minlength=E).cumsum(0)
+    return sel, se, ss, offs
+
+
+CASES = [
+    # T, E, k, K, N, skew, empty experts
+    (7, 4, 2, 64, 64, 0.0, ()),
+    (7, 8, 4, 128, 72, 0.0, ()),
+    (300, 3, 2, 192, 320, 0.0, ()),
+    (700, 8, 2, 256, 512, 1.5, (3,)),
+    (1024, 2, 1, 64, 264, 0.0, ()),
+    (513, 6, 4, 72, 40, 2.0, (0, 5)),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", CASES)
+@pytest.mark.parametrize("w_kn", [False, True])
+@pytest.mark.parametrize("x_grouped,y_grouped", [(False, True), (True, False), (True, True), (False, False)])
+def test_scatter2scatter(dtype, case, w_kn, x_grouped, y_grouped):
+    from xma.layers.moe import rocm_implementation as R
+
+    T, E, k, K, N, skew, empty = case
+    print(f"case T={T} E={E} k={k} K={K} N={N} w_kn={w_kn} xg={x_grouped} yg={y_grouped} {dtype}", flush=True)
+    sel, se, ss, offs = _routing(T, E, k, 0, skew, empty)
+    g = torch.Generator().manual_seed(1)
+    M = T * k
+    X = torch.randn(M if x_grouped else T, K, generator=g).to(dtype)
+    if w_kn:
+        W = (torch.randn(E, K, N, generator=g) * 0.1).to(dtype)  # contiguous (E, K, N)
+    else:
+        W = (torch.randn(E, N, K, generator=g) * 0.1).to(dtype).permute(0, 2, 1)  # view of (E, N, K)
+    scale = torch.rand(M, generator=g).to(dtype)
+    for rs in (None, scale):
+        want = oracle.scatter2scatter(X, W, se, ss, k, x_grouped, y_grouped, rs)
+        Wd = W.cuda() if w_kn else W.permute(0, 2, 1).contiguous().cuda().permute(0, 2, 1)
+        out = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+        R.scatter2scatter(X.cuda(), Wd, se.cuda(), ss.cuda(), out, k, x_grouped, y_grouped, offs.cuda(),
+                          None if rs is None else rs.cuda())
+        torch.cuda.synchronize()
+        assert torch.isfinite(out).all()
+        assert nerr(out, want) <= TOL
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", CASES)
+def test_group_bwd_W(dtype, case):
+    from xma.rocm import ops
+
+    T, E, k, K, N, skew, empty = case
+    print(f"case T={T} E={E} k={k} K={K} N={N} {dtype}", flush=True)
+    sel, se, ss, offs = _routing(T, E, k, 2, skew, empty)
+    g = torch.Generator().manual_seed(3)
+    M = T * k
+    x_tok = torch.randn(T, K, generator=g).to(dtype)
+    dy_tok = torch.randn(T, N, generator=g).to(dtype)
+    dy_grp = torch.randn(M, N, generator=g).to(dtype)
+    x_grp = torch.randn(M, K, generator=g).to(dtype)
+    scale = torch.rand(M, generator=g).to(dtype)
+
+    def run(DY, X, dy_scale, dy_fan, x_fan):
+        DW = torch.full((E, N, K), float("nan"), dtype=dtype, device="cuda").permute(0, 2, 1)
+        ops.group_bwd_W_rocm(DY.cuda(), X.cuda(), ss.cuda(), offs.cuda(), DW, None if dy_scale is None else dy_scale.cuda(),
+                             dy_fan, x_fan)
+        torch.cuda.synchronize()
+        assert torch.isfinite(DW).all()
+        return DW
+
+    # both grouped (the reference op), x gathered (dW1), dy gathered and scaled (dW2)
+    want = oracle.group_bwd_W(dy_grp, x_grp, offs, E)
+    assert nerr(run(dy_grp, x_grp, None, 0, 0), want) <= TOL
+    want = oracle.group_bwd_W(dy_grp, oracle.group(x_tok, ss, None, k), offs, E)
+    assert nerr(run(dy_grp, x_tok, None, 0, k), want) <= TOL
+    want = oracle.group_bwd_W(oracle.group(dy_tok, ss, scale, k), x_grp, offs, E)
+    assert nerr(run(dy_tok, x_grp, scale, k, 0), want) <= TOL
+    # experts without rows get an all-zero slice
+    got = run(dy_grp, x_grp, None, 0, 0)
+    for e in empty:
+        assert (got[e] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_group_and_combine(dtype):
+    from xma.layers.moe import rocm_implementation as R
+    from xma.rocm import ops
+
+    g = torch.Generator().manual_seed(5)
+    for T, k, H in [(7, 2, 64), (33, 4, 136), (1000, 8, 2048), (513, 1, 72)]:
+        E = 8
+        sel, se, ss, offs = _routing(T, E, k, 6)
+        A = torch.randn(T, H, generator=g).to(dtype)
+        coeff = torch.rand(T * k, generator=g).to(dtype)
+        for c in (None, coeff):
+            out = torch.empty(T * k, H, dtype=dtype, device="cuda")
+            R.group(A.cuda(), ss.cuda(), out, None if c is None else c.cuda(), k)
+            assert torch.equal(out.cpu(), oracle.group(A, ss, c, k))  # one rounding of an fp32 product: exact match
+        eo = torch.randn(T * k, H, generator=g).to(dtype)
+        w = torch.rand(T, k, generator=g).to(dtype)
+        dy = torch.randn(T, H, generator=g).to(dtype)
+        for ww in (None, w):
+            y = torch.empty(T, H, dtype=dtype, device="cuda")
+            ops.combine_rocm(eo.cuda(), None if ww is None else ww.cuda(), y, k)
+            assert nerr(y, oracle.combine(eo, ww, k)) <= TOL
+        d_w = torch.empty(T, k, dtype=dtype, device="cuda")
+        ops.combine_bwd_rocm(eo.cuda(), dy.cuda(), d_w)
+        assert nerr(d_w, oracle.combine_bwd(eo, dy, k)) <= TOL
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_swiglu_packed_standalone(dtype):
+    from xma import KernelBackend
+    from xma.functional import swiglu_packed
+
+    g = torch.Generator().manual_seed(7)
+    for rows, cols in [(1, 8), (7, 64), (300, 1408), (65, 4096)]:
+        x = (torch.randn(rows, 2 * cols, generator=g) * 2).to(dtype)
+        dy = torch.randn(rows, cols, generator=g).to(dtype)
+        xd = x.cuda().requires_grad_()
+        y = swiglu_packed(xd, kernel_backend=KernelBackend.rocm)
+        y.backward(dy.cuda())
+        assert nerr(y, oracle.swiglu_packed(x.float())) <= TOL
+        dg, du = oracle.swiglu_backward(x[..., 0::2].float(), x[..., 1::2].float(), dy.float())
+        want = torch.stack([dg, du], dim=-1).flatten(-2)
+        assert nerr(xd.grad, want) <= TOL
