@@ -1,0 +1,336 @@
+"""MoE hot-path benchmark on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c5|c2]
+
+Default workload: the Mixtral-shaped layer (T=8192, H=4096, I=14336, E=8, top-2, packed SwiGLU, bf16).
+A step is one forward + backward of the expert computation (routing histogram/sort, grouped
+up-projection + SwiGLU, grouped down-projection, combine, and all of their gradients) on synthetic
+inputs that are resident in HBM before the timed region.  Prints ONE JSON line:
+
+  value        tokens/s over the K timed steps (c2: routed ids/s)
+  roofline     the dominant kernel against its roofline; `achieved` = algorithmic FLOPs (or bytes)
+               of one launch / its average duration, timed live with events on the launch stream
+  cpu_baseline the CPU oracle (plain torch restatement of the reference's torch path) on a bounded
+               sample of the same workload, on this box's host cores
+  kernels      per-kernel duration / throughput table (extra, for the record)
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "accelerated-model-architectures_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+import torch  # noqa: E402
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0  # MI355X HBM3E
+
+WORKLOADS = {
+    # name: T, H, I, E, k, router bias std
+    "c3": dict(T=8192, H=4096, I=14336, E=8, k=2, bias=0.0, label="Mixtral-shaped MoE layer fwd+bwd"),
+    "c4": dict(T=16384, H=2048, I=1408, E=64, k=6, bias=1.5, label="fine-grained MoE fwd+bwd (skewed routing)"),
+    "c5": dict(T=32768, H=2048, I=768, E=128, k=8, bias=0.0, label="many-expert MoE fwd+bwd"),
+}
+
+
+def _time_gpu(fn, iters: int, warmup: int = 2) -> float:
+    """average milliseconds per call, events on the current (launch) stream"""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / iters
+
+
+def _make_moe_inputs(cfg, device, seed=0):
+    from xma.functional import swiglu_packed
+    from xma.layers import MoE
+
+    g = torch.Generator(device=device).manual_seed(seed)
+    T, H, I, E, k = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["k"]
+    with torch.device("meta"):
+        moe = MoE(E, k, H, I, swiglu_packed, True, add_bias=False, std=0.02)
+    moe = moe.to_empty(device=device).to(torch.bfloat16)
+    with torch.no_grad():
+        for p in (moe.c_fc.weight, moe.c_proj.weight, moe.gate.weight):
+            p.copy_((torch.randn(p.shape, generator=g, device=device, dtype=torch.float32) * 0.02).to(p.dtype))
+        moe.c_fc.N_array.fill_(2 * I), moe.c_fc.K_array.fill_(H)
+        moe.c_proj.N_array.fill_(H), moe.c_proj.K_array.fill_(I)
+    x = torch.randn(T, H, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    logits = torch.randn(T, E, generator=g, device=device, dtype=torch.float32)
+    if cfg["bias"]:
+        logits = logits + cfg["bias"] * torch.randn(E, generator=g, device=device, dtype=torch.float32)
+    vals, sel = logits.topk(k, dim=-1)
+    rw = torch.softmax(vals.float(), dim=-1).to(torch.bfloat16)
+    grad = torch.randn(T, H, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
+    return moe, x, rw, sel, grad
+
+
+def _kernel_table(moe, x, rw, sel, grad, cfg, iters):
+    """per-kernel timings of the ops of one step, each launched alone in a loop"""
+    from xma.layers.moe import rocm_implementation as R
+    from xma.rocm import ops
+
+    T, H, I, E, k = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["k"]
+    Tk = T * k
+    dev = x.device
+    counts, offs, excl, se, ss = R.route(sel, E)
+    w_fc, w_proj = moe.c_fc.weight.detach().permute(0, 2, 1), moe.c_proj.weight.detach().permute(0, 2, 1)
+    z = torch.empty(Tk, 2 * I, device=dev, dtype=x.dtype)
+    h = torch.empty(Tk, I, device=dev, dtype=x.dtype)
+    eo = torch.empty(Tk, H, device=dev, dtype=x.dtype)
+    y = torch.empty(T, H, device=dev, dtype=x.dtype)
+    dz = torch.empty_like(z)
+    d_rw = torch.empty_like(rw)
+    dw_fc, dw_proj = torch.empty_like(w_fc), torch.empty_like(w_proj)
+    flat_w = rw.view(-1)
+    ids = sel.flatten()
+
+    ops.up_projection_swiglu_rocm(x, w_fc, ss, offs, z, h, k)
+    ops.scatter2scatter_rocm(h, w_proj, ss, offs, eo, None, 1, True, False)
+    ops.down_projection_dx_swiglu_rocm(grad, w_proj.permute(0, 2, 1), ss, offs, z, dz, flat_w, k)
+
+    table = {}
+
+    def gemm(name, fn, flops):
+        ms = _time_gpu(fn, iters)
+        table[name] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "frac_mfma_peak": round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+                       "flops": flops}
+
+    def mem(name, fn, nbytes):
+        ms = _time_gpu(fn, iters)
+        table[name] = {"ms": round(ms, 4), "gbs": round(nbytes / ms / 1e6, 1), "frac_hbm_peak": round(nbytes / ms / 1e6 / PEAK_HBM_GBS, 4),
+                       "bytes": nbytes}
+
+    f = 2.0 * Tk * H * I
+    gemm("up_swiglu(grouped_gemm NT+SwiGLU)", lambda: ops.up_projection_swiglu_rocm(x, w_fc, ss, offs, z, h, k), 2 * f)
+    gemm("down(grouped_gemm NT)", lambda: ops.scatter2scatter_rocm(h, w_proj, ss, offs, eo, None, 1, True, False), f)
+    gemm("dx2_swiglu_bwd(grouped_gemm NN)",
+         lambda: ops.down_projection_dx_swiglu_rocm(grad, w_proj.permute(0, 2, 1), ss, offs, z, dz, flat_w, k), f)
+    gemm("dw2(grouped_gemm_dw)", lambda: ops.group_bwd_W_rocm(grad, h, ss, offs, dw_proj, flat_w, k, 0), f)
+    gemm("dw1(grouped_gemm_dw)", lambda: ops.group_bwd_W_rocm(dz, x, ss, offs, dw_fc, None, 0, k), 2 * f)
+    gemm("dx1(grouped_gemm NN)", lambda: ops.scatter2scatter_rocm(dz, w_fc.permute(0, 2, 1), ss, offs, eo, None, 1, True, False), 2 * f)
+    esz = 2
+    mem("combine", lambda: ops.combine_rocm(eo, rw, y, k), Tk * H * esz + T * k * esz + T * H * esz)
+    mem("combine_bwd", lambda: ops.combine_bwd_rocm(eo, grad, d_rw), Tk * H * esz + T * H * esz + T * k * esz)
+    mem("route", lambda: R.route(sel, E), Tk * 8 + Tk * 8 + Tk * 8 + E * 20)
+    return table
+
+
+def run_moe(args, cfg, name):
+    from oracle import moe as oracle_moe
+    from xma import KernelBackend
+
+    dev = torch.device("cuda:0")
+    moe, x, rw, sel, grad = _make_moe_inputs(cfg, dev)
+    T, H, I, E, k = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["k"]
+    xg = x.clone().requires_grad_()
+    rwg = rw.clone().requires_grad_()
+
+    def step():
+        for p in moe.parameters():
+            p.grad = None
+        xg.grad = None
+        rwg.grad = None
+        y = moe._compute_experts(xg, rwg, sel, kernel_backend=KernelBackend.rocm)
+        y.backward(grad)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    counts = torch.bincount(sel.flatten(), minlength=E)
+
+    table = _kernel_table(moe, x, rw, sel, grad, cfg, args.kernel_iters)
+    gemms = {n: v for n, v in table.items() if "tflops" in v}
+    dom = max(gemms, key=lambda n: gemms[n]["ms"])
+    total_flops = sum(v["flops"] for v in gemms.values())
+    total_ms = sum(v["ms"] for v in gemms.values())
+    roofline = {
+        "kernel": dom,
+        "bound": "mfma",
+        "achieved": gemms[dom]["tflops"],
+        "peak": PEAK_BF16_TFLOPS,
+        "unit": "TFLOP/s",
+        "frac": round(gemms[dom]["tflops"] / PEAK_BF16_TFLOPS, 4),
+        "traffic": None,
+        "all_gemms_tflops": round(total_flops / total_ms / 1e9, 1),
+        "all_gemms_frac": round(total_flops / total_ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+    }
+
+    # CPU baseline: the oracle, bf16 like the reference's torch path, on the first T/8 tokens with every other
+    # dimension unchanged (same weights, bit-identical)
+    cpu = None
+    if not args.no_cpu_baseline:
+        Ts = max(T // args.cpu_fraction, 1)
+        w1, w2 = moe.c_fc.weight.detach().cpu(), moe.c_proj.weight.detach().cpu()
+        xs, rws, sels, gs = x[:Ts].cpu(), rw[:Ts].cpu(), sel[:Ts].cpu(), grad[:Ts].cpu()
+        t1 = time.perf_counter()
+        oracle_moe.experts_forward_backward(xs, rws, sels, w1, w2, oracle_moe.swiglu_packed, gs)
+        dt = time.perf_counter() - t1
+        cpu = {
+            "value": round(Ts / dt, 1),
+            "unit": "tokens/s",
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"one fwd+bwd of the torch-path oracle in bf16 on the first {Ts} of {T} tokens (all other dimensions "
+                      f"and the weights unchanged), {dt:.1f} s",
+        }
+        del w1, w2
+
+    out = {
+        "metric": "moe_fwd_bwd_tokens_per_s",
+        "value": round(T / ms_per_step * 1e3, 1),
+        "unit": "tokens/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{name}: {cfg['label']}, T={T} H={H} I={I} E={E} top-{k} packed SwiGLU bf16, x~N(0,1) W~N(0,0.02) "
+                        f"logits~N(0,1){'+N(0,1.5) expert bias' if cfg['bias'] else ''}, upstream grad~N(0,1)",
+            "tokens": T,
+            "rows_per_expert_min_mean_max": [int(counts.min()), float(counts.float().mean()), int(counts.max())],
+            "step_tflops": round(18.0 * T * k * H * I / ms_per_step / 1e9, 1),
+        },
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "kernels": table,
+    }
+    print(json.dumps(out))
+
+
+def run_routing(args):
+    """configs[1]: continuous_count + routing on 4 Mi int32 ids over 64 experts (uniform; --zipf for the skewed run)"""
+    from oracle import routing as oracle_routing
+    from xma import KernelBackend
+    from xma.functional import continuous_count
+    from xma.layers.moe import rocm_implementation as R
+    from xma.rocm import ops
+
+    n, E = 4 * 1024 * 1024, 64
+    g = torch.Generator().manual_seed(0)
+    if args.zipf:
+        p = torch.arange(1, E + 1, dtype=torch.float64) ** (-1.1)
+        ids_cpu = torch.multinomial(p / p.sum(), n, replacement=True, generator=g).to(torch.int32)
+    else:
+        ids_cpu = torch.randint(0, E, (n,), generator=g, dtype=torch.int32)
+    # rotate over enough distinct buffers to exceed the 256 MB Infinity Cache
+    nbuf = 20
+    bufs = [ids_cpu.cuda() for _ in range(nbuf)]
+    it = [0]
+
+    def step():
+        it[0] += 1
+        R.route(bufs[it[0] % nbuf], E)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    y = torch.zeros(E, dtype=torch.uint32, device="cuda")
+
+    def hist():
+        it[0] += 1
+        ops.continuous_count_rocm(bufs[it[0] % nbuf], y)
+
+    hist_ms = _time_gpu(hist, args.kernel_iters * 10, warmup=5)
+    hist_warm_ms = _time_gpu(lambda: ops.continuous_count_rocm(bufs[0], y), args.kernel_iters * 10, warmup=5)
+    route_ms = _time_gpu(step, args.kernel_iters * 5, warmup=5)
+    hist_bytes = n * 4 + E * 4
+    route_bytes = n * 4 + n * 8 + n * 4 + E * 20
+    t1 = time.perf_counter()
+    reps = 3
+    for _ in range(reps):
+        oracle_routing.route(ids_cpu.numpy(), E)
+    dt = (time.perf_counter() - t1) / reps
+    out = {
+        "metric": "routing_ids_per_s",
+        "value": round(n / ms_per_step * 1e3, 1),
+        "unit": "ids/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int32",
+        "data": "synthetic",
+        "config": {"workload": f"c2: counts + offsets + stable permutation of {n} int32 ids over E={E}, "
+                               f"{'Zipf(s=1.1)' if args.zipf else 'uniform'}, {nbuf} rotating input buffers"},
+        "roofline": {
+            "kernel": "route (3 kernels: unit histogram, scan, stable scatter)",
+            "bound": "hbm",
+            "achieved": round(route_bytes / route_ms / 1e6, 1),
+            "peak": PEAK_HBM_GBS,
+            "unit": "GB/s",
+            "frac": round(route_bytes / route_ms / 1e6 / PEAK_HBM_GBS, 4),
+            "traffic": None,
+        },
+        "cpu_baseline": {"value": round(n / dt, 1), "unit": "ids/s", "cores": 1, "kind": "port",
+                         "sample": f"numpy stable argsort + bincount + cumsum of the same {n} ids, mean of {reps}"},
+        "kernels": {
+            "continuous_count_cold": {"ms": round(hist_ms, 5), "gbs": round(hist_bytes / hist_ms / 1e6, 1),
+                                      "frac_hbm_peak": round(hist_bytes / hist_ms / 1e6 / PEAK_HBM_GBS, 4), "bytes": hist_bytes},
+            "continuous_count_warm": {"ms": round(hist_warm_ms, 5), "gbs": round(hist_bytes / hist_warm_ms / 1e6, 1),
+                                      "frac_hbm_peak": round(hist_bytes / hist_warm_ms / 1e6 / PEAK_HBM_GBS, 4)},
+            "route": {"ms": round(route_ms, 5), "gbs": round(route_bytes / route_ms / 1e6, 1), "bytes": route_bytes},
+        },
+    }
+    print(json.dumps(out))
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--zipf", action="store_true", help="c2 only: Zipf(s=1.1) ids instead of uniform")
+    ap.add_argument("--kernel-iters", type=int, default=5)
+    ap.add_argument("--cpu-fraction", type=int, default=8, help="CPU baseline runs on T / this many tokens")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build measures one GPU; --gpus N with N > 1 is not supported (no collectives in the path)")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: needs a GPU")
+    from xma.rocm import get_library
+
+    get_library()
+    if args.workload == "c2":
+        run_routing(args)
+    else:
+        run_moe(args, WORKLOADS[args.workload], args.workload)
+
+
+if __name__ == "__main__":
+    main()
