@@ -1,0 +1,124 @@
+"""Host logic that needs no GPU: the C-ABI library loads and exports every symbol include/xma_rocm.h declares,
+backend selection and error behaviour mirror the reference, module layout matches its state-dict."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+import torch.nn as nn
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared_symbols():
+    text = open(os.path.join(ROOT, "include", "xma_rocm.h")).read()
+    return sorted(set(re.findall(r"\b(xma_rocm_[a-zA-Z0-9_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    from xma.rocm import LIBRARY_PATH, get_library
+    from xma.rocm.loader import SIGNATURES
+
+    assert os.path.isfile(LIBRARY_PATH), "build the library first: python __graft_entry__.py"
+    lib = ctypes.CDLL(LIBRARY_PATH)
+    declared = _declared_symbols()
+    assert len(declared) >= 12
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in include/xma_rocm.h but not exported"
+    assert sorted(SIGNATURES) == declared  # the ctypes table covers exactly the header
+    lib = get_library()
+    assert lib.xma_rocm_abi_version() == 1
+    # host-only entry points (no GPU work)
+    assert lib.xma_rocm_route_workspace_bytes(4 * 1024 * 1024, 64) == (4 * 1024 * 1024 // 2048) * 64 * 4
+    assert lib.xma_rocm_route_workspace_bytes(0, 8) == 8 * 4
+    assert lib.xma_rocm_route_workspace_bytes(-1, 8) == 0
+
+
+def test_argument_errors_are_reported_before_any_launch():
+    from xma.rocm import get_library
+
+    lib = get_library()
+    # bins < 1, E out of range, unsupported dtype, misaligned sizes: all rejected on the host
+    assert lib.xma_rocm_continuous_count(None, 0, 10, None, 0, None) == -1
+    assert b"continuous_count" in lib.xma_rocm_last_error()
+    assert lib.xma_rocm_route(None, 0, 10, 100000, None, None, None, None, None, None, 0, None) == -1
+    assert lib.xma_rocm_combine(None, 8, None, None, 8, 4, 2, 12, 0, None) == -1  # H % 8 != 0
+    assert lib.xma_rocm_combine(None, 8, None, None, 8, 4, 2, 16, 7, None) == -2  # dtype
+    rc = lib.xma_rocm_scatter2scatter(None, 64, None, 64 * 64, 64, 0, None, None, None, 64, None, 0, None, 16, 60, 64, 2, 1, 1, 1,
+                                      0, 0, None)
+    assert rc == -2 and b"multiples of 8" in lib.xma_rocm_last_error()
+    # empty problems are accepted without touching a pointer
+    assert lib.xma_rocm_combine(None, 8, None, None, 8, 0, 2, 16, 0, None) == 0
+    assert lib.xma_rocm_continuous_count(None, 0, 0, ctypes.c_void_p(16), 4, None) == 0
+
+
+def test_backend_selection_and_errors():
+    from xma import Accelerator, KernelBackend
+    from xma.functional import continuous_count, swiglu_packed
+    from xma.layers import MoE
+
+    assert KernelBackend.torch.verify_accelerator()
+    if not torch.cuda.is_available():
+        assert Accelerator.get_accelerator() == Accelerator.cpu
+        assert Accelerator.get_kernel_backend() == KernelBackend.torch
+        assert not KernelBackend.rocm.verify_accelerator()
+        with pytest.raises(AssertionError):  # explicit backend on the wrong accelerator (moe/__init__.py:205-208)
+            continuous_count(torch.zeros(4, dtype=torch.int32), 4, kernel_backend=KernelBackend.rocm)
+    x = torch.randint(0, 5, (100,))
+    assert continuous_count(x, 1).tolist() == [100]
+    assert continuous_count(x, 5, kernel_backend=KernelBackend.torch).dtype == torch.uint32
+    with pytest.raises(AssertionError):
+        continuous_count(x.view(10, 10), 5, kernel_backend=KernelBackend.torch)
+    with pytest.raises(AssertionError):
+        continuous_count(x.float(), 5, kernel_backend=KernelBackend.torch)
+    moe = MoE(4, 2, 16, 24, swiglu_packed, True, add_bias=False, std=0.02)
+    with pytest.raises((ValueError, AssertionError)):  # a backend this build does not have (moe/__init__.py:251-252)
+        moe(torch.randn(3, 16), kernel_backend=KernelBackend.triton)
+
+
+def test_module_layout_matches_reference_state_dict():
+    from xma.layers import MoE
+    from xma.layers.moe import Experts
+
+    moe = MoE(6, 2, 32, 48, nn.GLU(), True, add_bias=True, std=0.02)
+    sd = moe.state_dict()
+    assert {k: tuple(v.shape) for k, v in sd.items()} == {
+        "gate.weight": (6, 32),
+        "c_fc.weight": (6, 96, 32), "c_fc.bias": (6, 96), "c_fc.N_array": (6,), "c_fc.K_array": (6,),
+        "c_proj.weight": (6, 32, 48), "c_proj.bias": (6, 32), "c_proj.N_array": (6,), "c_proj.K_array": (6,),
+    }
+    assert sd["c_fc.N_array"].dtype == torch.uint32 and sd["c_fc.N_array"].view(torch.int32).tolist() == [96] * 6
+    assert sd["c_proj.K_array"].view(torch.int32).tolist() == [48] * 6
+    assert (sd["c_fc.bias"] == 0).all()
+    y, logits = moe(torch.randn(2, 5, 32))
+    assert y.shape == (2, 5, 32) and logits.shape == (10, 6)
+    e = Experts(3, 4, 5, add_bias=False, std=0.1)
+    assert e.bias is None and "in_features=4" in e.extra_repr()
+    moe1 = MoE(4, 1, 16, 8, nn.GELU(approximate="tanh"), False, add_bias=False, std=0.02)  # top-1 uses max
+    assert moe1(torch.randn(7, 16))[0].shape == (7, 16)
+
+
+def test_torch_backend_matches_oracle_in_bf16():
+    from oracle import moe as oracle
+    from xma import KernelBackend, set_seed
+    from xma.functional import swiglu_packed
+    from xma.layers import MoE
+
+    set_seed(3)
+    moe = MoE(8, 2, 64, 96, swiglu_packed, True, add_bias=False, std=0.02).to(torch.bfloat16)
+    x = torch.randn(50, 64).bfloat16()
+    rw, sel = oracle.routing_weights(torch.randn(50, 8), 2, torch.bfloat16)
+    y = moe._compute_experts(x, rw, sel, kernel_backend=KernelBackend.torch)
+    want = oracle.experts_forward(x, rw, sel, moe.c_fc.weight.data, moe.c_proj.weight.data, oracle.swiglu_packed)
+    assert torch.equal(y, want)
+
+
+def test_rocm_ops_fail_loudly_without_the_library(monkeypatch):
+    from xma.rocm import loader
+
+    monkeypatch.setattr(loader, "_lib", None)
+    monkeypatch.setattr(loader, "LIBRARY_PATH", "/nonexistent/libxma_rocm.so")
+    with pytest.raises(loader.RocmLibraryError):
+        loader.get_library()
