@@ -1,0 +1,73 @@
+// Argument blocks, tile constants and the workgroup -> tile mapping shared by the grouped GEMM kernels.
+#pragma once
+
+#include "common.hpp"
+
+constexpr int BM = 256, BN = 256; // output tile of every grouped GEMM kernel
+constexpr int GEMM_THREADS = 256;
+
+// exact n / d for 0 <= n < 2^31: q = (n * magic) >> shift with magic = ceil(2^shift / d), shift = 31 + ceil(log2 d)
+struct FastDiv {
+    uint32_t magic;
+    int shift;
+};
+inline FastDiv make_fastdiv(uint32_t d) {
+    int s = 0;
+    while ((1u << s) < d) ++s;
+    FastDiv f;
+    f.shift = 31 + s;
+    f.magic = (uint32_t)((((uint64_t)1 << f.shift) + d - 1) / d);
+    return f;
+}
+__device__ __forceinline__ uint32_t fastdiv(uint32_t n, FastDiv f) { return (uint32_t)(((uint64_t)n * f.magic) >> f.shift); }
+
+struct FwdArgs {
+    const uint16_t *X;
+    int64_t ldx;
+    const uint16_t *W;
+    int64_t w_es, ldw;
+    const int64_t *idx;
+    const int64_t *offs;
+    uint16_t *out;
+    int64_t ldo;
+    uint16_t *aux;
+    int64_t ldaux;
+    const uint16_t *scale;
+    int64_t M;
+    int N, K, E, fan_out, x_grouped, y_grouped;
+};
+
+struct DwArgs {
+    const uint16_t *DY;
+    int64_t lddy;
+    const uint16_t *X;
+    int64_t ldx;
+    const uint16_t *scale;
+    const int64_t *idx;
+    const int64_t *offs;
+    uint16_t *DW;
+    int64_t dw_es, lddw;
+    int N_out, K_in, E, dy_grouped, dy_fan_out, x_grouped, x_fan_out;
+    FastDiv dy_div, x_div;
+};
+
+// Workgroups are handed to the 8 XCDs round-robin by linear id.  Inside every aligned run of 256 ids give each XCD
+// 32 consecutive logical tiles, so tiles that share operand panels meet in one XCD's L2.
+__device__ __forceinline__ int xcd_remap(int bid, int grid) {
+    const int full = grid & ~255;
+    if (bid >= full) return bid;
+    const int w = bid & 255;
+    return (bid & ~255) + (w & 7) * 32 + (w >> 3);
+}
+
+template <typename K> inline int gemm_set_smem(K kernel, int bytes) {
+    hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+    if (err != hipSuccess) {
+        xma_set_error("hipFuncSetAttribute(max dynamic LDS = %d): %s", bytes, hipGetErrorString(err));
+        return XMA_ROCM_ELAUNCH;
+    }
+    return XMA_ROCM_OK;
+}
+
+// dW with a per-token scale on dY (register-staged loader, grouped_gemm_staged.hip)
+int launch_dw_scaled(const DwArgs &a, int dtype, int grid, hipStream_t st);

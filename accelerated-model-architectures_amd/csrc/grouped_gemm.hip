@@ -1,105 +1,180 @@
 // Grouped (per-expert, ragged) GEMMs of the MoE layer on CDNA4 MFMA.
 //
-// One workgroup = 256 threads = 4 waves (2 x 2), output tile 256 x 256, K step 64.
-// Each wave owns 128 x 128 = 4 x 4 v_mfma_f32_32x32x16 tiles (256 fp32 accumulators per lane).
-// Operand tiles live in LDS as [256 rows][64 k] 16-bit elements, 16-byte chunks XOR-swizzled,
-// double buffered (2 x 64 KB); global loads for step s+1 are issued before the MFMAs of step
-// s and written to the other buffer behind them, one barrier per K step.
+// One workgroup = 256 threads = 4 wave64 (2 x 2), output tile 256 x 256, K step 32.  Each wave owns 128 x 128 =
+// 4 x 4 v_mfma_f32_32x32x16 tiles (256 fp32 accumulators per lane, one wave per SIMD).
 //
-// MFMA operand roles: the "P" tile supplies the rows of the 32x32 result (register dimension:
-// a lane holds 4 consecutive P indices per accumulator quad) and the "Q" tile supplies its
-// columns (lane % 32).  P is always the dimension that is contiguous in the OUTPUT, so a lane
-// stores 8 contiguous bytes per quad and owns one output row: gather/scatter indices, row
-// scales and the SwiGLU pairs (adjacent columns) are all lane-local.
+// Operand tiles go from HBM straight into LDS with global_load_lds_dwordx4 (no VGPR staging, no ds_write): a wave
+// instruction moves 64 x 16 bytes to 1 KB of consecutive LDS, and the swizzle is applied on the GLOBAL side (which
+// lane fetches which 16-byte chunk).  Two LDS layouts, both 16 KB per 256 x 32 operand tile:
+//   row-major source (K contiguous in memory):  LDS [256 rows][4 chunks], chunk c of row r at slot c ^ ((r >> 1) & 3);
+//       MFMA fragments are one ds_read_b128 per lane.
+//   transposed source (K is the row index in memory: weights for dX, both operands for dW):
+//       LDS [32 k][32 chunks] exactly as in memory, chunk c of k-row kr at slot c ^ ((kr & 3) << 1);
+//       MFMA fragments are two ds_read_b64_tr_b16 per lane, which hand each lane 4 consecutive k of one column.
+//
+// Pipeline: a ring of 4 stages (128 KB of the 160 KB LDS).  In iteration kt the loads of K step kt + 3 are issued,
+// so three steps are in flight behind the one being multiplied; a wave waits only until step kt + 1 has landed
+// (s_waitcnt vmcnt(N) with the two younger steps still outstanding).  The single barrier of an iteration sits
+// between its two k16 sub-steps: the fragments of the second sub-step are already in registers, and the fragments
+// of the next K step are read behind the barrier while those MFMAs run, so the matrix pipe does not drain at the
+// step boundary.  Steps beyond the K extent are fetched from a page of zeros, which keeps the vmcnt arithmetic
+// uniform.  Instruction order inside a sub-step is pinned (one fragment read, two MFMAs, eight times).
+//
+// MFMA operand roles: the "P" tile supplies the rows of the 32x32 result (register dimension: a lane holds 4
+// consecutive P indices per accumulator quad) and the "Q" tile supplies its columns (lane % 32).  P is always the
+// dimension that is contiguous in the OUTPUT, so a lane stores 8 contiguous bytes per quad and owns one output row:
+// gather/scatter indices, row scales and the SwiGLU (gate, up) pairs are all lane-local.
 //
 //   forward / dX :  Q = activation rows (tokens),     P = weight rows (output features)
 //   dW           :  Q = dY columns (out features),    P = X columns (in features), K = tokens
 //
-// Tiles never straddle experts: the schedule is expert-major, derived on the device from the
-// inclusive expert offsets in each workgroup's prologue (no host read of the counts).
-#include "common.hpp"
+// Tiles never straddle experts: the schedule is expert-major, derived on the device from the inclusive expert
+// offsets in each workgroup's prologue (no host read of the counts).
+#include "gemm_common.hpp"
 
-namespace {
+namespace xma_rocm {
 
-constexpr int BM = 256, BN = 256, BK = 64;
-constexpr int THREADS = 256;
-constexpr int TILE_CHUNKS = 256 * 8;                              // 16-byte chunks per operand tile
-constexpr int SMEM_BYTES = 2 /*stages*/ * 2 /*operands*/ * TILE_CHUNKS * 16; // 128 KB
+constexpr int BK = 32, NSTAGE = 4;
+constexpr int OP_CHUNKS = 256 * 4;                     // 16-byte chunks per operand tile (16 KB)
+constexpr int STAGE_CHUNKS = 2 * OP_CHUNKS;            // Q tile then P tile
+constexpr int GEMM_SMEM_BYTES = NSTAGE * STAGE_CHUNKS * 16; // 128 KB
+constexpr int LOADS_PER_STEP = 8;                      // LDS-DMA instructions per wave and K step (4 Q + 4 P)
 
-struct FwdArgs {
-    const uint16_t *X;
-    int64_t ldx;
-    const uint16_t *W;
-    int64_t w_es, ldw;
-    const int64_t *idx;
-    const int64_t *offs;
-    uint16_t *out;
-    int64_t ldo;
-    uint16_t *aux;
-    int64_t ldaux;
-    const uint16_t *scale;
-    int64_t M;
-    int N, K, E, fan_out, x_grouped, y_grouped;
-};
+// 1 KB of zeros: the source of every chunk that lies beyond the K extent of an operand
+__device__ __attribute__((aligned(16))) uint32_t g_zero_page[256];
 
-struct DwArgs {
-    const uint16_t *DY;
-    int64_t lddy;
-    const uint16_t *X;
-    int64_t ldx;
-    const uint16_t *scale;
-    const int64_t *idx;
-    const int64_t *offs;
-    uint16_t *DW;
-    int64_t dw_es, lddw;
-    int N_out, K_in, E, dy_grouped, dy_fan_out, x_grouped, x_fan_out;
-};
+typedef short s16x4 __attribute__((ext_vector_type(4)));
 
-// Workgroups are handed to the 8 XCDs round-robin by linear id.  Inside every aligned run of
-// 256 ids give each XCD 32 consecutive logical tiles, so tiles that share operand panels
-// meet in one XCD's L2.
-__device__ __forceinline__ int xcd_remap(int bid, int grid) {
-    const int full = grid & ~255;
-    if (bid >= full) return bid;
-    const int w = bid & 255;
-    return (bid & ~255) + (w & 7) * 32 + (w >> 3);
+__device__ __forceinline__ void lds_dma16(const uint16_t *src, u32x4 *lds_wave_base) {
+    __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)src,
+                                     (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
 }
 
-// One K step of MFMA work for a wave: 4 k16 sub-steps x (4 P fragments, 4 Q fragments, 16 MFMAs).
-template <typename T>
-__device__ __forceinline__ void mma_tile(const u32x4 *__restrict__ sP, const u32x4 *__restrict__ sQ, int p_row0,
-                                         int q_row0, int lane, f32x16 (&acc)[4][4]) {
-    const int r = lane & 31, kc = lane >> 5;
+// Row-major tile [256][4 chunks]: an instruction covers 16 rows; wave w loads rows 64 w + 16 i + (lane >> 2), i = 0..3.
+// Slot lane & 3 of such a row holds logical chunk (lane & 3) ^ ((row >> 1) & 3) = (lane & 3) ^ ((lane >> 3) & 3).
+__device__ __forceinline__ void issue_rowmajor(u32x4 *sT, const uint16_t *const (&rowp)[4], int k0, int K, int wave,
+                                               int lane, const uint16_t *zero) {
+    const int k = k0 + ((((lane & 3) ^ ((lane >> 3) & 3))) << 3);
+    const bool ok = k < K;
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-        u32x4 pf[4], qf[4];
+    for (int i = 0; i < 4; ++i) lds_dma16(ok ? rowp[i] + k : zero, sT + (wave * 64 + i * 16) * 4);
+}
+
+// Transposed tile [32 k][32 chunks]: an instruction covers 2 k-rows; wave w loads k-rows 8 w + 2 j + (lane >> 5),
+// j = 0..3; krow[j] points at column 0 of the tile in the source row of that k (or at the zero page).  Slot lane & 31
+// holds logical chunk (lane & 31) ^ ((kr & 3) << 1), clamped to the last valid chunk of the row (columns past the
+// matrix edge are masked at the store).
+__device__ __forceinline__ void issue_transposed(u32x4 *sT, const uint16_t *const (&krow)[4], int max_chunk, int wave,
+                                                 int lane) {
+    const int half = lane >> 5, p = lane & 31;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            pf[i] = sP[lds_chunk(p_row0 + i * 32 + r, kk * 2 + kc)];
-            qf[i] = sQ[lds_chunk(q_row0 + i * 32 + r, kk * 2 + kc)];
-        }
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int i = 0; i < 4; ++i) acc[j][i] = Elem<T>::mfma(pf[j], qf[i], acc[j][i]);
+    for (int j = 0; j < 4; ++j) {
+        int c = p ^ (((2 * j + half) & 3) << 1);
+        if (c > max_chunk) c = max_chunk;
+        lds_dma16(krow[j] + (c << 3), sT + (wave * 8 + j * 2) * 32);
     }
+}
+
+// MFMA fragment: 8 consecutive k (k block lane / 32 of k16 sub-step kk) of tile row R0 + lane % 32
+template <int TR> __device__ __forceinline__ u32x4 read_frag(const u32x4 *sT, int R0, int kk, int lane) {
+    if (TR == 0) {
+        const int row = R0 + (lane & 31), c = kk * 2 + (lane >> 5);
+        return sT[row * 4 + (c ^ ((row >> 1) & 3))];
+    } else {
+        // ds_read_b64_tr_b16 works on groups of 16 lanes: lane p of a group supplies the address of 4 columns at one
+        // k-row, and receives 4 consecutive k of one column.  With p -> (k-row kb + p / 4, columns mb + 4 (p % 4))
+        // lane p ends up with column mb + p, k = kb .. kb + 3.
+        const int p = lane & 15, G = lane >> 4;
+        const int m = R0 + ((G & 1) << 4) + ((p & 3) << 2);
+        const int kr = kk * 16 + ((G >> 1) << 3) + (p >> 2);
+        const int byte = kr * 512 + ((((m >> 3) ^ ((kr & 3) << 1))) << 4) + ((m & 7) << 1);
+        // Issued as inline assembly: after an LDS-DMA load the compiler guards every LDS read it cannot prove
+        // disjoint with s_waitcnt vmcnt(0), which would drain the whole load pipeline at each fragment.  The price is
+        // that the compiler does not know these reads are in flight: wait_frags() below must precede their use.
+        const unsigned addr = (unsigned)(size_t)((__attribute__((address_space(3))) const char *)((const char *)sT + byte));
+        u32x2 lo, hi;
+        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(addr));
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:2048" : "=v"(hi) : "v"(addr)); // + 4 k-rows
+        u32x4 r = {lo[0], lo[1], hi[0], hi[1]};
+        return r;
+    }
+}
+
+struct Frags {
+    u32x4 p[4], q[4];
+};
+
+// All LDS reads of this wave have returned; the fragments are tied to the statement so that no MFMA using them can be
+// moved above it.
+__device__ __forceinline__ void wait_frags(Frags &f) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(f.p[0]), "+v"(f.p[1]), "+v"(f.p[2]), "+v"(f.p[3]), "+v"(f.q[0]), "+v"(f.q[1]), "+v"(f.q[2]),
+                   "+v"(f.q[3]));
+}
+
+template <int PTR, int QTR>
+__device__ __forceinline__ void load_frags(Frags &f, const u32x4 *stage, int kk, int p_row0, int q_row0, int lane) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        f.p[i] = read_frag<PTR>(stage + OP_CHUNKS, p_row0 + i * 32, kk, lane);
+        f.q[i] = read_frag<QTR>(stage, q_row0 + i * 32, kk, lane);
+    }
+}
+
+// The 16 MFMAs of one k16 sub-step on `cur`, with the 8 fragment reads of (`stage`, kk) into `nxt` pinned between the
+// first MFMAs: (two MFMAs, one P and one Q fragment) x 4, then 8 more MFMAs.  The reads are all issued in the first
+// half so that their latency is covered by the second half, whatever the compiler assumes at the next wait.
+template <typename T, int PTR, int QTR>
+__device__ __forceinline__ void mma_step(Frags &cur, Frags &nxt, const u32x4 *stage, int kk, int p_row0, int q_row0,
+                                         int lane, f32x16 (&acc)[4][4]) {
+    if (PTR || QTR) wait_frags(cur); // issued at least 8 MFMAs ago
+#pragma unroll
+    for (int g = 0; g < 8; ++g) {
+        __builtin_amdgcn_sched_barrier(0);
+        const int j = g >> 1, i0 = (g & 1) * 2;
+        acc[j][i0] = Elem<T>::mfma(cur.p[j], cur.q[i0], acc[j][i0]);
+        acc[j][i0 + 1] = Elem<T>::mfma(cur.p[j], cur.q[i0 + 1], acc[j][i0 + 1]);
+        __builtin_amdgcn_sched_barrier(0);
+        if (g < 4) {
+            nxt.p[g] = read_frag<PTR>(stage + OP_CHUNKS, p_row0 + g * 32, kk, lane);
+            nxt.q[g] = read_frag<QTR>(stage, q_row0 + g * 32, kk, lane);
+        }
+    }
+    __builtin_amdgcn_sched_barrier(0);
+}
+
+// Wait until at most `younger` of this wave's VMEM operations are outstanding (they retire in order), i.e. until the
+// K step the next sub-step reads has landed, make sure this wave's LDS reads have returned, then meet the other
+// waves.  The immediate has to be a literal, hence the macro; "memory" keeps the compiler from moving LDS accesses
+// across it.
+#define XMA_WAIT_STEP_AND_BARRIER(younger) asm volatile("s_waitcnt vmcnt(" #younger ") lgkmcnt(0)\n\ts_barrier" ::: "memory")
+#define XMA_WAIT_ALL_LOADS() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
+
+template <int N> __device__ __forceinline__ void zero_acc(f32x16 (&acc)[N][N]) {
+#pragma unroll
+    for (int j = 0; j < N; ++j)
+#pragma unroll
+        for (int i = 0; i < N; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.f;
 }
 
 // ------------------------------------------------------------------------------------------------
 // forward / dX kernel
-//   WT = 0: W[e] is (N, K) with K contiguous (x @ W^T)      -> P tile loaded row-major
-//   WT = 1: W[e] is (K, N) with N contiguous (dy @ W)       -> P tile transposed in registers
+//   WT = 0: W[e] is (N, K) with K contiguous (x @ W^T)      -> P tile row-major
+//   WT = 1: W[e] is (K, N) with N contiguous (dy @ W)       -> P tile transposed source
 // ------------------------------------------------------------------------------------------------
 template <typename T, int WT, int EPI>
-__global__ __launch_bounds__(THREADS, 1) void grouped_gemm_kernel(const FwdArgs a) {
+__global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const FwdArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     __shared__ int s_sched[4];
     u32x4 *tiles = (u32x4 *)smem;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int NT = (a.N + BN - 1) / BN;
 
     // ---- expert-major schedule: work[e] = ceil(rows_e / BM) * NT, prefix, locate this tile
-    int *s_pre = (int *)smem; // [E + 1], dead before the first tile store
+    int *s_pre = (int *)smem; // [E + 1], dead before the first tile load
     if (tid == 0) s_sched[0] = -1;
     if (wave == 0) {
         int carry = 0;
@@ -123,7 +198,7 @@ __global__ __launch_bounds__(THREADS, 1) void grouped_gemm_kernel(const FwdArgs 
     }
     __syncthreads();
     const int L = xcd_remap(blockIdx.x, gridDim.x);
-    for (int e = tid; e < a.E; e += THREADS)
+    for (int e = tid; e < a.E; e += GEMM_THREADS)
         if (s_pre[e] <= L && L < s_pre[e + 1]) {
             s_sched[0] = e;
             s_sched[1] = L - s_pre[e];
@@ -139,96 +214,71 @@ __global__ __launch_bounds__(THREADS, 1) void grouped_gemm_kernel(const FwdArgs 
     const int n0 = n_tile * BN;
     __syncthreads(); // s_pre is dead from here on
 
+
     // ---- loader set-up
-    // row-major loader: thread -> chunk (tid & 7) of rows (tid >> 3) + 32 i
-    const int lc = tid & 7, lr = tid >> 3;
-    const uint16_t *q_ptr[8];
+    const uint16_t *zero = (const uint16_t *)g_zero_page;
+    const uint16_t *q_ptr[4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        int r = lr + 32 * i;
+    for (int i = 0; i < 4; ++i) {
+        int r = wave * 64 + i * 16 + (lane >> 2);
         if (r >= rows_valid) r = rows_valid - 1; // duplicates, masked at the store
         const int64_t n = row0 + r;
         const int64_t src = a.x_grouped ? n : a.idx[n] / a.fan_out;
-        q_ptr[i] = a.X + src * a.ldx + lc * 8;
+        q_ptr[i] = a.X + src * a.ldx;
     }
     const uint16_t *We = a.W + (int64_t)e * a.w_es;
-    const uint16_t *p_ptr[8];
-    // transposing loader: thread -> 8 k-rows (8 * (tid >> 5) + j) x 8 columns (8 * (tid & 31))
-    const int tc = tid & 31, tk = tid >> 5;
+    const uint16_t *p_ptr[4];
+    int p_max_chunk = 0;
     if (WT == 0) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            int r = n0 + lr + 32 * i;
+        for (int i = 0; i < 4; ++i) {
+            int r = n0 + wave * 64 + i * 16 + (lane >> 2);
             if (r >= a.N) r = a.N - 1;
-            p_ptr[i] = We + (int64_t)r * a.ldw + lc * 8;
+            p_ptr[i] = We + (int64_t)r * a.ldw;
         }
     } else {
-        int c = n0 + tc * 8;
-        if (c >= a.N) c = a.N - 8;
+        p_max_chunk = ((a.N - n0) >> 3) - 1; // last valid 16-byte chunk of the tile's column range
 #pragma unroll
-        for (int j = 0; j < 8; ++j) p_ptr[j] = We + (int64_t)(tk * 8 + j) * a.ldw + c;
+        for (int j = 0; j < 4; ++j) p_ptr[j] = We + (int64_t)(wave * 8 + 2 * j + (lane >> 5)) * a.ldw + n0;
     }
+    const int KT = (a.K + BK - 1) / BK;
 
-    u32x4 q_reg[8], p_reg[8];
-    const u32x4 zero4 = {0u, 0u, 0u, 0u};
-
-    auto load_tiles = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const bool ok = k0 + lc * 8 < a.K;
-            q_reg[i] = ok ? *(const u32x4 *)(q_ptr[i] + k0) : zero4;
-        }
+    auto issue = [&](int kt) { // K step kt -> stage kt % NSTAGE; steps past the end read zeros
+        u32x4 *sQ = tiles + (kt & (NSTAGE - 1)) * STAGE_CHUNKS, *sP = sQ + OP_CHUNKS;
+        const int k0 = kt * BK;
+        issue_rowmajor(sQ, q_ptr, k0, a.K, wave, lane, zero);
         if (WT == 0) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                const bool ok = k0 + lc * 8 < a.K;
-                p_reg[i] = ok ? *(const u32x4 *)(p_ptr[i] + k0) : zero4;
-            }
+            issue_rowmajor(sP, p_ptr, k0, a.K, wave, lane, zero);
         } else {
+            const uint16_t *krow[4];
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const bool ok = k0 + tk * 8 + j < a.K;
-                p_reg[j] = ok ? *(const u32x4 *)(p_ptr[j] + (int64_t)k0 * a.ldw) : zero4;
+            for (int j = 0; j < 4; ++j) {
+                const int k = k0 + wave * 8 + 2 * j + (lane >> 5);
+                krow[j] = (k < a.K) ? p_ptr[j] + (int64_t)k0 * a.ldw : zero;
             }
-        }
-    };
-    auto store_tiles = [&](int stage) {
-        u32x4 *sQ = tiles + stage * 2 * TILE_CHUNKS, *sP = sQ + TILE_CHUNKS;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) sQ[lds_chunk(lr + 32 * i, lc)] = q_reg[i];
-        if (WT == 0) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) sP[lds_chunk(lr + 32 * i, lc)] = p_reg[i];
-        } else {
-            u32x4 t[8];
-            transpose8x8_b16(p_reg, t);
-#pragma unroll
-            for (int c = 0; c < 8; ++c) sP[lds_chunk(tc * 8 + c, tk)] = t[c];
+            issue_transposed(sP, krow, p_max_chunk, wave, lane);
         }
     };
 
     f32x16 acc[4][4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.f;
-
+    zero_acc(acc);
     const int wq = (wave & 1) * 128, wp = (wave >> 1) * 128; // wave's 128 x 128 corner inside the tile
-    const int KT = (a.K + BK - 1) / BK;
 
-    load_tiles(0);
-    store_tiles(0);
-    __syncthreads();
+    issue(0);
+    issue(1);
+    issue(2);
+    XMA_WAIT_STEP_AND_BARRIER(16); // step 0 has landed in every wave
+    Frags f0, f1;
+    load_frags<WT, 0>(f0, tiles, 0, wp, wq, lane);
     for (int kt = 0; kt < KT; ++kt) {
-        const int stage = kt & 1;
-        if (kt + 1 < KT) load_tiles((kt + 1) * BK);
-        const u32x4 *sQ = tiles + stage * 2 * TILE_CHUNKS, *sP = sQ + TILE_CHUNKS;
-        mma_tile<T>(sP, sQ, wp, wq, lane, acc);
-        if (kt + 1 < KT) store_tiles(stage ^ 1);
-        __syncthreads();
+        const u32x4 *cur = tiles + (kt & (NSTAGE - 1)) * STAGE_CHUNKS;
+        const u32x4 *nxt = tiles + ((kt + 1) & (NSTAGE - 1)) * STAGE_CHUNKS;
+        issue(kt + 3); // its stage held step kt - 1, which every wave left before the previous barrier
+        mma_step<T, WT, 0>(f0, f1, cur, 1, wp, wq, lane, acc);
+        XMA_WAIT_STEP_AND_BARRIER(16); // steps kt + 2 and kt + 3 may still be in flight; kt + 1 has landed
+        mma_step<T, WT, 0>(f1, f0, nxt, 0, wp, wq, lane, acc);
     }
+    XMA_WAIT_ALL_LOADS();
 
     // ---- epilogue: lane owns row (lane & 31) of each 32-row block; quad g of tile (j, i) holds
     //      columns n0 + wp + 32 j + 8 g + 4 (lane >> 5) + {0..3}
@@ -284,14 +334,18 @@ __global__ __launch_bounds__(THREADS, 1) void grouped_gemm_kernel(const FwdArgs 
 }
 
 // ------------------------------------------------------------------------------------------------
-// dW kernel: DW[e][o][i] = sum_n DY[n][o] X[n][i]; both operands are token-major, so both tiles go
-// through the transposing loader; the K loop runs over the expert's row range (zero-filled tail).
+// dW kernel: DW[e][o][i] = sum_n DY[n][o] X[n][i]; both operands are token-major = transposed sources; the K loop
+// runs over the expert's row range, k-rows past its end come from the zero page.
+//   GATHER = 0: both operands in grouped order (row n of the expert range)
+//   GATHER = 1: rows taken through sorted_scattered_idxs; the indices of step kt + 5 are loaded in iteration kt, so
+//               that two younger steps of loads may stay in flight when they are consumed
 // ------------------------------------------------------------------------------------------------
-template <typename T>
-__global__ __launch_bounds__(THREADS, 1) void grouped_gemm_dw_kernel(const DwArgs a) {
+template <typename T, int GATHER>
+__global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const DwArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     u32x4 *tiles = (u32x4 *)smem;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int OT = (a.N_out + 255) / 256, IT = (a.K_in + 255) / 256;
     const int L = xcd_remap(blockIdx.x, gridDim.x);
     const int e = L / (OT * IT);
@@ -300,80 +354,94 @@ __global__ __launch_bounds__(THREADS, 1) void grouped_gemm_dw_kernel(const DwArg
     const int64_t row_lo = e ? a.offs[e - 1] : 0, row_hi = a.offs[e];
     const int rows = (int)(row_hi - row_lo);
     const int KT = (rows + BK - 1) / BK;
+    const uint16_t *zero = (const uint16_t *)g_zero_page;
+    const int q_max_chunk = ((a.N_out - o0) >> 3) - 1, p_max_chunk = ((a.K_in - i0) >> 3) - 1;
+    const int kr_lane = wave * 8 + (lane >> 5); // this lane's k-rows of a step: kr_lane + 2 j
 
-    const int tc = tid & 31, tk = tid >> 5;
-    int oc = o0 + tc * 8, ic = i0 + tc * 8;
-    if (oc >= a.N_out) oc = a.N_out - 8;
-    if (ic >= a.K_in) ic = a.K_in - 8;
-
-    int64_t nxt_idx[8]; // scattered index of the 8 tokens this thread loads in the NEXT step
-    float q_scale[8];
-    u32x4 q_reg[8], p_reg[8];
-    const u32x4 zero4 = {0u, 0u, 0u, 0u};
-    const bool need_idx = !a.dy_grouped || !a.x_grouped || a.scale;
-
-    auto load_idx = [&](int kt) {
+    // scattered indices of this lane's 4 tokens for two K steps of the prefetch ring: even steps in idx_even, odd in idx_odd
+    uint32_t idx_even[4], idx_odd[4];
+    auto load_idx = [&](int kt, uint32_t (&slot)[4]) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int r = kt * BK + tk * 8 + j;
-            nxt_idx[j] = (need_idx && r < rows) ? a.idx[row_lo + r] : 0;
+        for (int j = 0; j < 4; ++j) {
+            // clamped, never predicated: every wave must issue exactly 4 loads here for the vmcnt arithmetic below
+            int r = kt * BK + kr_lane + 2 * j;
+            if (r >= rows) r = rows - 1;
+            slot[j] = (uint32_t)a.idx[row_lo + r];
         }
     };
-    auto load_tiles = [&](int kt) { // uses nxt_idx of step kt
+    auto issue = [&](int kt, const uint32_t (&slot)[4]) {
+        u32x4 *sQ = tiles + (kt & (NSTAGE - 1)) * STAGE_CHUNKS, *sP = sQ + OP_CHUNKS;
+        const uint16_t *qrow[4], *prow[4];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const int r = kt * BK + tk * 8 + j;
-            const bool ok = r < rows;
-            const int64_t n = row_lo + r;
-            const int64_t dsrc = a.dy_grouped ? n : nxt_idx[j] / a.dy_fan_out;
-            const int64_t xsrc = a.x_grouped ? n : nxt_idx[j] / a.x_fan_out;
-            q_reg[j] = ok ? *(const u32x4 *)(a.DY + dsrc * a.lddy + oc) : zero4;
-            p_reg[j] = ok ? *(const u32x4 *)(a.X + xsrc * a.ldx + ic) : zero4;
-            q_scale[j] = (ok && a.scale) ? Elem<T>::lo((uint32_t)a.scale[nxt_idx[j]]) : 1.f;
+        for (int j = 0; j < 4; ++j) {
+            const int r = kt * BK + kr_lane + 2 * j;
+            int64_t dsrc = row_lo + r, xsrc = row_lo + r;
+            if (GATHER) {
+                if (!a.dy_grouped) dsrc = fastdiv(slot[j], a.dy_div);
+                if (!a.x_grouped) xsrc = fastdiv(slot[j], a.x_div);
+            }
+            qrow[j] = (r < rows) ? a.DY + dsrc * a.lddy + o0 : zero;
+            prow[j] = (r < rows) ? a.X + xsrc * a.ldx + i0 : zero;
         }
-    };
-    auto store_tiles = [&](int stage) {
-        u32x4 *sQ = tiles + stage * 2 * TILE_CHUNKS, *sP = sQ + TILE_CHUNKS;
-        if (a.scale) {
-#pragma unroll
-            for (int j = 0; j < 8; ++j)
-#pragma unroll
-                for (int q = 0; q < 4; ++q)
-                    q_reg[j][q] = Elem<T>::pack(q_scale[j] * Elem<T>::lo(q_reg[j][q]), q_scale[j] * Elem<T>::hi(q_reg[j][q]));
-        }
-        u32x4 t[8];
-        transpose8x8_b16(q_reg, t);
-#pragma unroll
-        for (int c = 0; c < 8; ++c) sQ[lds_chunk(tc * 8 + c, tk)] = t[c];
-        transpose8x8_b16(p_reg, t);
-#pragma unroll
-        for (int c = 0; c < 8; ++c) sP[lds_chunk(tc * 8 + c, tk)] = t[c];
+        issue_transposed(sQ, qrow, q_max_chunk, wave, lane);
+        issue_transposed(sP, prow, p_max_chunk, wave, lane);
     };
 
     f32x16 acc[4][4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int i = 0; i < 4; ++i)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.f;
-
+    zero_acc(acc);
     const int wq = (wave & 1) * 128, wp = (wave >> 1) * 128;
     if (KT > 0) {
-        load_idx(0);
-        load_tiles(0);
-        if (KT > 1) load_idx(1);
-        store_tiles(0);
-        __syncthreads();
-        for (int kt = 0; kt < KT; ++kt) {
-            const int stage = kt & 1;
-            if (kt + 1 < KT) load_tiles(kt + 1);
-            if (kt + 2 < KT) load_idx(kt + 2);
-            const u32x4 *sQ = tiles + stage * 2 * TILE_CHUNKS, *sP = sQ + TILE_CHUNKS;
-            mma_tile<T>(sP, sQ, wp, wq, lane, acc);
-            if (kt + 1 < KT) store_tiles(stage ^ 1);
-            __syncthreads();
+        // VMEM order per wave (GATHER): idx(0) idx(1) dma(0) idx(2) dma(1) idx(3) dma(2) idx(4), then per iteration kt:
+        // dma(kt + 3) idx(kt + 5).  The indices of a step are loaded two steps before they are consumed, so two younger
+        // steps of loads may stay in flight at that point.  The loop is unrolled by two so that the two index slots
+        // are fixed registers; a trailing odd step multiplies zeros.
+        if (GATHER) {
+            load_idx(0, idx_even);
+            load_idx(1, idx_odd);
         }
+        __builtin_amdgcn_sched_barrier(0);
+        issue(0, idx_even);
+        __builtin_amdgcn_sched_barrier(0);
+        if (GATHER) load_idx(2, idx_even);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(1, idx_odd);
+        __builtin_amdgcn_sched_barrier(0);
+        if (GATHER) load_idx(3, idx_odd);
+        __builtin_amdgcn_sched_barrier(0);
+        issue(2, idx_even);
+        __builtin_amdgcn_sched_barrier(0);
+        if (GATHER) load_idx(4, idx_even);
+        __builtin_amdgcn_sched_barrier(0);
+        // outstanding behind dma(0): idx(2) dma(1) idx(3) dma(2) idx(4) = 4 + 8 + 4 + 8 + 4
+        if (GATHER)
+            XMA_WAIT_STEP_AND_BARRIER(28);
+        else
+            XMA_WAIT_STEP_AND_BARRIER(16);
+        Frags f0, f1;
+        load_frags<1, 1>(f0, tiles, 0, wp, wq, lane);
+
+        // one K step: issue step kt + 3 (its indices sit in `use`), refill `use` with the indices of step kt + 5
+        auto k_step = [&](int kt, uint32_t (&use)[4]) {
+            const u32x4 *cur = tiles + (kt & (NSTAGE - 1)) * STAGE_CHUNKS;
+            const u32x4 *nxt = tiles + ((kt + 1) & (NSTAGE - 1)) * STAGE_CHUNKS;
+            __builtin_amdgcn_sched_barrier(0);
+            issue(kt + 3, use);
+            __builtin_amdgcn_sched_barrier(0);
+            if (GATHER) load_idx(kt + 5, use);
+            __builtin_amdgcn_sched_barrier(0);
+            mma_step<T, 1, 1>(f0, f1, cur, 1, wp, wq, lane, acc);
+            // behind dma(kt + 1): idx(kt + 3) dma(kt + 2) idx(kt + 4) dma(kt + 3) idx(kt + 5) = 28 operations
+            if (GATHER)
+                XMA_WAIT_STEP_AND_BARRIER(28);
+            else
+                XMA_WAIT_STEP_AND_BARRIER(16);
+            mma_step<T, 1, 1>(f1, f0, nxt, 0, wp, wq, lane, acc);
+        };
+        for (int kt = 0; kt < KT; kt += 2) {
+            k_step(kt, idx_odd);      // step kt + 3 is odd
+            k_step(kt + 1, idx_even); // step kt + 4 is even
+        }
+        XMA_WAIT_ALL_LOADS();
     }
 
     // lane owns DW row o (from the Q tile), 4 consecutive in-features per quad
@@ -396,22 +464,18 @@ __global__ __launch_bounds__(THREADS, 1) void grouped_gemm_dw_kernel(const DwArg
     }
 }
 
-inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
-
-template <typename K> int set_smem(K kernel) {
-    hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, SMEM_BYTES);
-    if (err != hipSuccess) {
-        xma_set_error("hipFuncSetAttribute(max dynamic LDS = %d): %s", SMEM_BYTES, hipGetErrorString(err));
-        return XMA_ROCM_ELAUNCH;
-    }
-    return XMA_ROCM_OK;
+template <typename T, int WT, int EPI> int launch_fwd(const FwdArgs &a, int grid, hipStream_t st) {
+    int rc = gemm_set_smem(grouped_gemm_kernel<T, WT, EPI>, GEMM_SMEM_BYTES);
+    if (rc) return rc;
+    grouped_gemm_kernel<T, WT, EPI><<<grid, GEMM_THREADS, GEMM_SMEM_BYTES, st>>>(a);
+    return xma_check_launch("grouped_gemm_kernel");
 }
 
-template <typename T, int WT, int EPI> int launch_fwd(const FwdArgs &a, int grid, hipStream_t st) {
-    int rc = set_smem(grouped_gemm_kernel<T, WT, EPI>);
+template <typename T, int GATHER> int launch_dw(const DwArgs &a, int grid, hipStream_t st) {
+    int rc = gemm_set_smem(grouped_gemm_dw_kernel<T, GATHER>, GEMM_SMEM_BYTES);
     if (rc) return rc;
-    grouped_gemm_kernel<T, WT, EPI><<<grid, THREADS, SMEM_BYTES, st>>>(a);
-    return xma_check_launch("grouped_gemm_kernel");
+    grouped_gemm_dw_kernel<T, GATHER><<<grid, GEMM_THREADS, GEMM_SMEM_BYTES, st>>>(a);
+    return xma_check_launch("grouped_gemm_dw_kernel");
 }
 
 template <typename T> int dispatch_fwd(const FwdArgs &a, int wt, int epi, int grid, hipStream_t st) {
@@ -425,7 +489,11 @@ template <typename T> int dispatch_fwd(const FwdArgs &a, int wt, int epi, int gr
     return launch_fwd<T, 1, XMA_ROCM_EPI_SWIGLU_BWD>(a, grid, st);
 }
 
-} // namespace
+inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+} // namespace xma_rocm
+
+using namespace xma_rocm;
 
 extern "C" int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *W, int64_t w_expert_stride, int64_t ldw,
                                         int w_is_kn, const int64_t *sorted_scattered_idxs,
@@ -523,13 +591,11 @@ extern "C" int xma_rocm_group_bwd_W(const void *DY, int64_t lddy, int dy_grouped
     const int64_t grid = (int64_t)E * ((N_out + 255) / 256) * ((K_in + 255) / 256);
     XMA_REQUIRE(grid < ((int64_t)1 << 31), XMA_ROCM_EUNSUPPORTED, "group_bwd_W: grid too large");
     hipStream_t st = (hipStream_t)stream;
-    int rc;
-    if (dtype == XMA_ROCM_BF16) {
-        if ((rc = set_smem(grouped_gemm_dw_kernel<__bf16>))) return rc;
-        grouped_gemm_dw_kernel<__bf16><<<(int)grid, THREADS, SMEM_BYTES, st>>>(a);
-    } else {
-        if ((rc = set_smem(grouped_gemm_dw_kernel<_Float16>))) return rc;
-        grouped_gemm_dw_kernel<_Float16><<<(int)grid, THREADS, SMEM_BYTES, st>>>(a);
-    }
-    return xma_check_launch("grouped_gemm_dw_kernel");
+    a.dy_div = make_fastdiv((uint32_t)dy_fan_out);
+    a.x_div = make_fastdiv((uint32_t)x_fan_out);
+    if (dy_scale) return launch_dw_scaled(a, dtype, (int)grid, st);
+    const bool gather = !dy_grouped || !x_grouped;
+    if (dtype == XMA_ROCM_BF16)
+        return gather ? launch_dw<__bf16, 1>(a, (int)grid, st) : launch_dw<__bf16, 0>(a, (int)grid, st);
+    return gather ? launch_dw<_Float16, 1>(a, (int)grid, st) : launch_dw<_Float16, 0>(a, (int)grid, st);
 }

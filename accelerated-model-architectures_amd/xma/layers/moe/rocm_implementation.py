@@ -11,7 +11,7 @@ Differences from the reference's data flow, all of which remove HBM passes:
   * dW reads its gathered operand through the index instead of a materialised
     ``grouped_x`` / ``grouped_grad_out`` copy, and writes every element of dW
     (no zeros_like fill);
-  * the router-weight scaling of dy is applied inside the GEMMs;
+  * the router-weight scaling of dy is applied in the dX2 epilogue (dW2 reads one scaled grouped copy of dy);
   * backward reuses the un-weighted expert outputs saved by forward instead of
     recomputing them with another GEMM (triton_implementation/__init__.py:117-128);
   * combine and its backward are dedicated coalesced kernels, not bmm.
@@ -88,6 +88,16 @@ def _empty_dw_like(expert_weights: torch.Tensor) -> torch.Tensor:
     return torch.empty_like(expert_weights)
 
 
+def _scaled_grouped_dy(grad_out: torch.Tensor, sorted_scattered_idxs: torch.Tensor, flat_w: torch.Tensor, top_k: int):
+    """grouped_dy[n] = dy[idx[n] // k] * w[idx[n]] (the reference's grouped_grad_out, triton_implementation/__init__.py:134-140).
+    The scale sits on the reduction index of dW2, so it has to be on an operand; one HBM-bound pass over (T*k, H) is
+    cheaper than rescaling fragments inside the MFMA loop.  dX2 does not read this copy: it gathers dy through the index
+    and scales in its epilogue."""
+    out = torch.empty(sorted_scattered_idxs.numel(), grad_out.size(1), dtype=grad_out.dtype, device=grad_out.device)
+    ops.group_rocm(grad_out, sorted_scattered_idxs, out, flat_w, top_k)
+    return out
+
+
 # ----------------------------------------------------------------------------------------- autograd
 class _UpProjectionExperts(torch.autograd.Function):
     """x (T, H) -> grouped (T*k, out); counterpart of triton_implementation/__init__.py:12-72."""
@@ -145,7 +155,8 @@ class _DownProjectionExperts(torch.autograd.Function):
 
         flat_w = router_weights.view(-1)
         d_weights = _empty_dw_like(expert_weights)
-        ops.group_bwd_W_rocm(grad_out, x, sorted_scattered_idxs, expert_offsets, d_weights, flat_w, top_k, 0)
+        ops.group_bwd_W_rocm(_scaled_grouped_dy(grad_out, sorted_scattered_idxs, flat_w, top_k), x, sorted_scattered_idxs,
+                             expert_offsets, d_weights, None, 0, 0)
 
         d_input = torch.empty_like(x)
         ops.scatter2scatter_rocm(
@@ -190,7 +201,8 @@ class _FusedSwiGLUExperts(torch.autograd.Function):
             grad_out, w_proj.permute(0, 2, 1), sorted_scattered_idxs, expert_offsets, z, dz, flat_w, top_k
         )
         d_w_proj = _empty_dw_like(w_proj)
-        ops.group_bwd_W_rocm(grad_out, h, sorted_scattered_idxs, expert_offsets, d_w_proj, flat_w, top_k, 0)
+        ops.group_bwd_W_rocm(_scaled_grouped_dy(grad_out, sorted_scattered_idxs, flat_w, top_k), h, sorted_scattered_idxs,
+                             expert_offsets, d_w_proj, None, 0, 0)
         d_w_fc = _empty_dw_like(w_fc)
         ops.group_bwd_W_rocm(dz, x, sorted_scattered_idxs, expert_offsets, d_w_fc, None, 0, top_k)
 

@@ -120,12 +120,15 @@ def _kernel_table(moe, x, rw, sel, grad, cfg, iters):
     gemm("down(grouped_gemm NT)", lambda: ops.scatter2scatter_rocm(h, w_proj, ss, offs, eo, None, 1, True, False), f)
     gemm("dx2_swiglu_bwd(grouped_gemm NN)",
          lambda: ops.down_projection_dx_swiglu_rocm(grad, w_proj.permute(0, 2, 1), ss, offs, z, dz, flat_w, k), f)
-    gemm("dw2(grouped_gemm_dw)", lambda: ops.group_bwd_W_rocm(grad, h, ss, offs, dw_proj, flat_w, k, 0), f)
+    gdy = torch.empty(Tk, H, device=dev, dtype=x.dtype)
+    ops.group_rocm(grad, ss, gdy, flat_w, k)
+    gemm("dw2(grouped_gemm_dw)", lambda: ops.group_bwd_W_rocm(gdy, h, ss, offs, dw_proj, None, 0, 0), f)
     gemm("dw1(grouped_gemm_dw)", lambda: ops.group_bwd_W_rocm(dz, x, ss, offs, dw_fc, None, 0, k), 2 * f)
     gemm("dx1(grouped_gemm NN)", lambda: ops.scatter2scatter_rocm(dz, w_fc.permute(0, 2, 1), ss, offs, eo, None, 1, True, False), 2 * f)
     esz = 2
     mem("combine", lambda: ops.combine_rocm(eo, rw, y, k), Tk * H * esz + T * k * esz + T * H * esz)
     mem("combine_bwd", lambda: ops.combine_bwd_rocm(eo, grad, d_rw), Tk * H * esz + T * H * esz + T * k * esz)
+    mem("group(dy*w)", lambda: ops.group_rocm(grad, ss, gdy, flat_w, k), T * H * esz + Tk * H * esz + Tk * (8 + esz))
     mem("route", lambda: R.route(sel, E), Tk * 8 + Tk * 8 + Tk * 8 + E * 20)
     return table
 
