@@ -52,27 +52,23 @@ __device__ __forceinline__ void lds_dma16(const uint16_t *src, u32x4 *lds_wave_b
 
 // Row-major tile [256][4 chunks]: an instruction covers 16 rows; wave w loads rows 64 w + 16 i + (lane >> 2), i = 0..3.
 // Slot lane & 3 of such a row holds logical chunk (lane & 3) ^ ((row >> 1) & 3) = (lane & 3) ^ ((lane >> 3) & 3).
-__device__ __forceinline__ void issue_rowmajor(u32x4 *sT, const uint16_t *const (&rowp)[4], int k0, int K, int wave,
-                                               int lane, const uint16_t *zero) {
+// Piece i of the tile (one instruction):
+__device__ __forceinline__ void issue_rowmajor_piece(u32x4 *sT, const uint16_t *rowp_i, int i, int k0, int K, int wave,
+                                                     int lane, const uint16_t *zero) {
     const int k = k0 + ((((lane & 3) ^ ((lane >> 3) & 3))) << 3);
-    const bool ok = k < K;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) lds_dma16(ok ? rowp[i] + k : zero, sT + (wave * 64 + i * 16) * 4);
+    lds_dma16((k < K) ? rowp_i + k : zero, sT + (wave * 64 + i * 16) * 4);
 }
 
 // Transposed tile [32 k][32 chunks]: an instruction covers 2 k-rows; wave w loads k-rows 8 w + 2 j + (lane >> 5),
-// j = 0..3; krow[j] points at column 0 of the tile in the source row of that k (or at the zero page).  Slot lane & 31
+// j = 0..3; krow_j points at column 0 of the tile in the source row of that k (or at the zero page).  Slot lane & 31
 // holds logical chunk (lane & 31) ^ ((kr & 3) << 1), clamped to the last valid chunk of the row (columns past the
-// matrix edge are masked at the store).
-__device__ __forceinline__ void issue_transposed(u32x4 *sT, const uint16_t *const (&krow)[4], int max_chunk, int wave,
-                                                 int lane) {
+// matrix edge are masked at the store).  Piece j of the tile (one instruction):
+__device__ __forceinline__ void issue_transposed_piece(u32x4 *sT, const uint16_t *krow_j, int j, int max_chunk, int wave,
+                                                       int lane) {
     const int half = lane >> 5, p = lane & 31;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        int c = p ^ (((2 * j + half) & 3) << 1);
-        if (c > max_chunk) c = max_chunk;
-        lds_dma16(krow[j] + (c << 3), sT + (wave * 8 + j * 2) * 32);
-    }
+    int c = p ^ (((2 * j + half) & 3) << 1);
+    if (c > max_chunk) c = max_chunk;
+    lds_dma16(krow_j + (c << 3), sT + (wave * 8 + j * 2) * 32);
 }
 
 // MFMA fragment: 8 consecutive k (k block lane / 32 of k16 sub-step kk) of tile row R0 + lane % 32
@@ -121,12 +117,14 @@ __device__ __forceinline__ void load_frags(Frags &f, const u32x4 *stage, int kk,
     }
 }
 
-// The 16 MFMAs of one k16 sub-step on `cur`, with the 8 fragment reads of (`stage`, kk) into `nxt` pinned between the
-// first MFMAs: (two MFMAs, one P and one Q fragment) x 4, then 8 more MFMAs.  The reads are all issued in the first
-// half so that their latency is covered by the second half, whatever the compiler assumes at the next wait.
-template <typename T, int PTR, int QTR>
+// The 16 MFMAs of one k16 sub-step on `cur` as 8 pinned slots.  Slot g: two MFMAs; for g < 4 one P and one Q fragment
+// read of (`stage`, kk) into `nxt`; then `hook(g)`, which the callers use to issue one LDS-DMA load (with its address
+// arithmetic) per slot.  A wave issues in order, so anything not placed between MFMAs would leave the matrix pipe
+// idle for as long as it takes to issue; all fragment reads sit in the first half so that the second half covers
+// their latency.
+template <typename T, int PTR, int QTR, typename Hook>
 __device__ __forceinline__ void mma_step(Frags &cur, Frags &nxt, const u32x4 *stage, int kk, int p_row0, int q_row0,
-                                         int lane, f32x16 (&acc)[4][4]) {
+                                         int lane, f32x16 (&acc)[4][4], Hook hook) {
     if (PTR || QTR) wait_frags(cur); // issued at least 8 MFMAs ago
 #pragma unroll
     for (int g = 0; g < 8; ++g) {
@@ -139,15 +137,24 @@ __device__ __forceinline__ void mma_step(Frags &cur, Frags &nxt, const u32x4 *st
             nxt.p[g] = read_frag<PTR>(stage + OP_CHUNKS, p_row0 + g * 32, kk, lane);
             nxt.q[g] = read_frag<QTR>(stage, q_row0 + g * 32, kk, lane);
         }
+        hook(g);
     }
     __builtin_amdgcn_sched_barrier(0);
 }
+
+struct NoHook {
+    __device__ __forceinline__ void operator()(int) const {}
+};
 
 // Wait until at most `younger` of this wave's VMEM operations are outstanding (they retire in order), i.e. until the
 // K step the next sub-step reads has landed, make sure this wave's LDS reads have returned, then meet the other
 // waves.  The immediate has to be a literal, hence the macro; "memory" keeps the compiler from moving LDS accesses
 // across it.
+#ifdef XMA_EXP_NO_VMWAIT
+#define XMA_WAIT_STEP_AND_BARRIER(younger) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
+#else
 #define XMA_WAIT_STEP_AND_BARRIER(younger) asm volatile("s_waitcnt vmcnt(" #younger ") lgkmcnt(0)\n\ts_barrier" ::: "memory")
+#endif
 #define XMA_WAIT_ALL_LOADS() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
 
 template <int N> __device__ __forceinline__ void zero_acc(f32x16 (&acc)[N][N]) {
@@ -243,21 +250,23 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
     }
     const int KT = (a.K + BK - 1) / BK;
 
-    auto issue = [&](int kt) { // K step kt -> stage kt % NSTAGE; steps past the end read zeros
+    // piece 0..7 of K step kt -> stage kt % NSTAGE (pieces 0..3 = Q tile, 4..7 = P tile); steps past the end read zeros
+    auto issue_piece = [&](int kt, int piece) {
         u32x4 *sQ = tiles + (kt & (NSTAGE - 1)) * STAGE_CHUNKS, *sP = sQ + OP_CHUNKS;
         const int k0 = kt * BK;
-        issue_rowmajor(sQ, q_ptr, k0, a.K, wave, lane, zero);
-        if (WT == 0) {
-            issue_rowmajor(sP, p_ptr, k0, a.K, wave, lane, zero);
+        if (piece < 4) {
+            issue_rowmajor_piece(sQ, q_ptr[piece], piece, k0, a.K, wave, lane, zero);
+        } else if (WT == 0) {
+            issue_rowmajor_piece(sP, p_ptr[piece - 4], piece - 4, k0, a.K, wave, lane, zero);
         } else {
-            const uint16_t *krow[4];
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int k = k0 + wave * 8 + 2 * j + (lane >> 5);
-                krow[j] = (k < a.K) ? p_ptr[j] + (int64_t)k0 * a.ldw : zero;
-            }
-            issue_transposed(sP, krow, p_max_chunk, wave, lane);
+            const int j = piece - 4;
+            const int k = k0 + wave * 8 + 2 * j + (lane >> 5);
+            issue_transposed_piece(sP, (k < a.K) ? p_ptr[j] + (int64_t)k0 * a.ldw : zero, j, p_max_chunk, wave, lane);
         }
+    };
+    auto issue = [&](int kt) {
+#pragma unroll
+        for (int piece = 0; piece < 8; ++piece) issue_piece(kt, piece);
     };
 
     f32x16 acc[4][4];
@@ -273,10 +282,11 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
     for (int kt = 0; kt < KT; ++kt) {
         const u32x4 *cur = tiles + (kt & (NSTAGE - 1)) * STAGE_CHUNKS;
         const u32x4 *nxt = tiles + ((kt + 1) & (NSTAGE - 1)) * STAGE_CHUNKS;
-        issue(kt + 3); // its stage held step kt - 1, which every wave left before the previous barrier
-        mma_step<T, WT, 0>(f0, f1, cur, 1, wp, wq, lane, acc);
+        // the loads of step kt + 3 go out one per MFMA slot; their stage held step kt - 1, which every wave left
+        // before the previous barrier
+        mma_step<T, WT, 0>(f0, f1, cur, 1, wp, wq, lane, acc, [&](int g) { issue_piece(kt + 3, g); });
         XMA_WAIT_STEP_AND_BARRIER(16); // steps kt + 2 and kt + 3 may still be in flight; kt + 1 has landed
-        mma_step<T, WT, 0>(f1, f0, nxt, 0, wp, wq, lane, acc);
+        mma_step<T, WT, 0>(f1, f0, nxt, 0, wp, wq, lane, acc, NoHook());
     }
     XMA_WAIT_ALL_LOADS();
 
@@ -364,27 +374,36 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             // clamped, never predicated: every wave must issue exactly 4 loads here for the vmcnt arithmetic below
+            // Inline assembly (low dword of the int64 index): the compiler would guard the later use of a loop-carried
+            // loaded register with s_waitcnt vmcnt(0) and drain the LDS-DMA pipeline; wait_idx() does the exact wait.
             int r = kt * BK + kr_lane + 2 * j;
             if (r >= rows) r = rows - 1;
-            slot[j] = (uint32_t)a.idx[row_lo + r];
+            const int64_t *src = a.idx + row_lo + r;
+            asm volatile("global_load_dword %0, %1, off" : "=v"(slot[j]) : "v"(src) : "memory");
+        }
+    };
+    // The indices in `slot` were loaded two K steps ago; since then this wave issued one step of DMA (8) and one set of
+    // indices (4).  VMEM operations retire in order.
+    auto wait_idx = [&](uint32_t (&slot)[4]) {
+        asm volatile("s_waitcnt vmcnt(12)" : "+v"(slot[0]), "+v"(slot[1]), "+v"(slot[2]), "+v"(slot[3]));
+    };
+    // piece 0..7 of K step kt (0..3 = dY tile, 4..7 = X tile); `slot` holds the step's scattered indices
+    auto issue_piece = [&](int kt, const uint32_t (&slot)[4], int piece) {
+        u32x4 *sQ = tiles + (kt & (NSTAGE - 1)) * STAGE_CHUNKS, *sP = sQ + OP_CHUNKS;
+        const int j = piece & 3;
+        const int r = kt * BK + kr_lane + 2 * j;
+        int64_t src = row_lo + r;
+        if (piece < 4) {
+            if (GATHER && !a.dy_grouped) src = fastdiv(slot[j], a.dy_div);
+            issue_transposed_piece(sQ, (r < rows) ? a.DY + src * a.lddy + o0 : zero, j, q_max_chunk, wave, lane);
+        } else {
+            if (GATHER && !a.x_grouped) src = fastdiv(slot[j], a.x_div);
+            issue_transposed_piece(sP, (r < rows) ? a.X + src * a.ldx + i0 : zero, j, p_max_chunk, wave, lane);
         }
     };
     auto issue = [&](int kt, const uint32_t (&slot)[4]) {
-        u32x4 *sQ = tiles + (kt & (NSTAGE - 1)) * STAGE_CHUNKS, *sP = sQ + OP_CHUNKS;
-        const uint16_t *qrow[4], *prow[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int r = kt * BK + kr_lane + 2 * j;
-            int64_t dsrc = row_lo + r, xsrc = row_lo + r;
-            if (GATHER) {
-                if (!a.dy_grouped) dsrc = fastdiv(slot[j], a.dy_div);
-                if (!a.x_grouped) xsrc = fastdiv(slot[j], a.x_div);
-            }
-            qrow[j] = (r < rows) ? a.DY + dsrc * a.lddy + o0 : zero;
-            prow[j] = (r < rows) ? a.X + xsrc * a.ldx + i0 : zero;
-        }
-        issue_transposed(sQ, qrow, q_max_chunk, wave, lane);
-        issue_transposed(sP, prow, p_max_chunk, wave, lane);
+        for (int piece = 0; piece < 8; ++piece) issue_piece(kt, slot, piece);
     };
 
     f32x16 acc[4][4];
@@ -400,6 +419,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
             load_idx(1, idx_odd);
         }
         __builtin_amdgcn_sched_barrier(0);
+        if (GATHER) asm volatile("s_waitcnt vmcnt(0)" : "+v"(idx_even[0]), "+v"(idx_even[1]), "+v"(idx_even[2]), "+v"(idx_even[3]),
+                                 "+v"(idx_odd[0]), "+v"(idx_odd[1]), "+v"(idx_odd[2]), "+v"(idx_odd[3]));
         issue(0, idx_even);
         __builtin_amdgcn_sched_barrier(0);
         if (GATHER) load_idx(2, idx_even);
@@ -408,6 +429,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
         __builtin_amdgcn_sched_barrier(0);
         if (GATHER) load_idx(3, idx_odd);
         __builtin_amdgcn_sched_barrier(0);
+        if (GATHER) wait_idx(idx_even); // behind idx(2): dma(1) idx(3)
         issue(2, idx_even);
         __builtin_amdgcn_sched_barrier(0);
         if (GATHER) load_idx(4, idx_even);
@@ -420,22 +442,21 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
         Frags f0, f1;
         load_frags<1, 1>(f0, tiles, 0, wp, wq, lane);
 
-        // one K step: issue step kt + 3 (its indices sit in `use`), refill `use` with the indices of step kt + 5
+        // one K step: the loads of step kt + 3 (its indices sit in `use`) go out one per MFMA slot of the first sub-step,
+        // then `use` is refilled with the indices of step kt + 5
         auto k_step = [&](int kt, uint32_t (&use)[4]) {
             const u32x4 *cur = tiles + (kt & (NSTAGE - 1)) * STAGE_CHUNKS;
             const u32x4 *nxt = tiles + ((kt + 1) & (NSTAGE - 1)) * STAGE_CHUNKS;
-            __builtin_amdgcn_sched_barrier(0);
-            issue(kt + 3, use);
-            __builtin_amdgcn_sched_barrier(0);
+            if (GATHER) wait_idx(use);
+            mma_step<T, 1, 1>(f0, f1, cur, 1, wp, wq, lane, acc, [&](int g) { issue_piece(kt + 3, use, g); });
             if (GATHER) load_idx(kt + 5, use);
             __builtin_amdgcn_sched_barrier(0);
-            mma_step<T, 1, 1>(f0, f1, cur, 1, wp, wq, lane, acc);
             // behind dma(kt + 1): idx(kt + 3) dma(kt + 2) idx(kt + 4) dma(kt + 3) idx(kt + 5) = 28 operations
             if (GATHER)
                 XMA_WAIT_STEP_AND_BARRIER(28);
             else
                 XMA_WAIT_STEP_AND_BARRIER(16);
-            mma_step<T, 1, 1>(f1, f0, nxt, 0, wp, wq, lane, acc);
+            mma_step<T, 1, 1>(f1, f0, nxt, 0, wp, wq, lane, acc, NoHook());
         };
         for (int kt = 0; kt < KT; kt += 2) {
             k_step(kt, idx_odd);      // step kt + 3 is odd
