@@ -1,24 +1,25 @@
 // Grouped (per-expert, ragged) GEMMs of the MoE layer on CDNA4 MFMA.
 //
-// One workgroup = 256 threads = 4 wave64 (2 x 2), output tile 256 x 256, K step 32.  Each wave owns 128 x 128 =
+// One workgroup = 256 threads = 4 wave64 (2 x 2), output tile 256 x 256, K step 64.  Each wave owns 128 x 128 =
 // 4 x 4 v_mfma_f32_32x32x16 tiles (256 fp32 accumulators per lane, one wave per SIMD).
 //
 // Operand tiles go from HBM straight into LDS with global_load_lds_dwordx4 (no VGPR staging, no ds_write): a wave
 // instruction moves 64 x 16 bytes to 1 KB of consecutive LDS, and the swizzle is applied on the GLOBAL side (which
-// lane fetches which 16-byte chunk).  Two LDS layouts, both 16 KB per 256 x 32 operand tile:
-//   row-major source (K contiguous in memory):  LDS [256 rows][4 chunks], chunk c of row r at slot c ^ ((r >> 1) & 3);
+// lane fetches which 16-byte chunk).  Every such instruction covers whole 128-byte lines (8 per instruction): the
+// texture addresser works line by line, and half-line requests (a 32-wide K step) were measured at a third of the
+// throughput.  Two LDS layouts, both 32 KB per 256 x 64 operand tile:
+//   row-major source (K contiguous in memory):  LDS [256 rows][8 chunks], chunk c of row r at slot c ^ swz(r);
 //       MFMA fragments are one ds_read_b128 per lane.
 //   transposed source (K is the row index in memory: weights for dX, both operands for dW):
-//       LDS [32 k][32 chunks] exactly as in memory, chunk c of k-row kr at slot c ^ ((kr & 3) << 1);
+//       LDS [64 k][32 chunks] exactly as in memory, chunk c of k-row kr at slot c ^ ((kr & 3) << 1);
 //       MFMA fragments are two ds_read_b64_tr_b16 per lane, which hand each lane 4 consecutive k of one column.
 //
-// Pipeline: a ring of 4 stages (128 KB of the 160 KB LDS).  In iteration kt the loads of K step kt + 3 are issued,
-// so three steps are in flight behind the one being multiplied; a wave waits only until step kt + 1 has landed
-// (s_waitcnt vmcnt(N) with the two younger steps still outstanding).  The single barrier of an iteration sits
-// between its two k16 sub-steps: the fragments of the second sub-step are already in registers, and the fragments
-// of the next K step are read behind the barrier while those MFMAs run, so the matrix pipe does not drain at the
-// step boundary.  Steps beyond the K extent are fetched from a page of zeros, which keeps the vmcnt arithmetic
-// uniform.  Instruction order inside a sub-step is pinned (one fragment read, two MFMAs, eight times).
+// Pipeline: two stages (128 KB of the 160 KB LDS), one barrier per K step.  A K step is four k16 sub-steps of 16 MFMAs;
+// the fragments of sub-step kk + 1 are read while sub-step kk multiplies.  The barrier sits between sub-steps 2 and 3:
+// by then a wave holds the last fragments of the step in registers, so behind the barrier the other stage (step s + 1,
+// waited for with vmcnt(0) just before) is readable and this stage is free.  The loads of step s + 2 are issued one per
+// MFMA slot during sub-steps 0 and 1 of step s + 1, which leaves them a step and a half to land.  A wave issues in
+// order, so everything that is not an MFMA is pinned between MFMAs (sched_barrier) instead of in front of them.
 //
 // MFMA operand roles: the "P" tile supplies the rows of the 32x32 result (register dimension: a lane holds 4
 // consecutive P indices per accumulator quad) and the "Q" tile supplies its columns (lane % 32).  P is always the
@@ -34,11 +35,10 @@
 
 namespace xma_rocm {
 
-constexpr int BK = 32, NSTAGE = 4;
-constexpr int OP_CHUNKS = 256 * 4;                     // 16-byte chunks per operand tile (16 KB)
-constexpr int STAGE_CHUNKS = 2 * OP_CHUNKS;            // Q tile then P tile
+constexpr int BK = 64, NSTAGE = 2;
+constexpr int OP_CHUNKS = 256 * 8;                          // 16-byte chunks per operand tile (32 KB)
+constexpr int STAGE_CHUNKS = 2 * OP_CHUNKS;                 // Q tile then P tile
 constexpr int GEMM_SMEM_BYTES = NSTAGE * STAGE_CHUNKS * 16; // 128 KB
-constexpr int LOADS_PER_STEP = 8;                      // LDS-DMA instructions per wave and K step (4 Q + 4 P)
 
 // 1 KB of zeros: the source of every chunk that lies beyond the K extent of an operand
 __device__ __attribute__((aligned(16))) uint32_t g_zero_page[256];
@@ -50,17 +50,17 @@ __device__ __forceinline__ void lds_dma16(const uint16_t *src, u32x4 *lds_wave_b
                                      (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
 }
 
-// Row-major tile [256][4 chunks]: an instruction covers 16 rows; wave w loads rows 64 w + 16 i + (lane >> 2), i = 0..3.
-// Slot lane & 3 of such a row holds logical chunk (lane & 3) ^ ((row >> 1) & 3) = (lane & 3) ^ ((lane >> 3) & 3).
-// Piece i of the tile (one instruction):
+// Row-major tile [256][8 chunks]: an instruction covers 8 rows; wave w loads rows 64 w + 8 i + (lane >> 3), i = 0..7.
+// swz(r) = (r ^ (r >> 3)) & 7 = (lane >> 3) ^ i for these rows, so slot lane & 7 holds logical chunk
+// (lane & 7) ^ (lane >> 3) ^ i.  Piece i of the tile (one instruction):
 __device__ __forceinline__ void issue_rowmajor_piece(u32x4 *sT, const uint16_t *rowp_i, int i, int k0, int K, int wave,
                                                      int lane, const uint16_t *zero) {
-    const int k = k0 + ((((lane & 3) ^ ((lane >> 3) & 3))) << 3);
-    lds_dma16((k < K) ? rowp_i + k : zero, sT + (wave * 64 + i * 16) * 4);
+    const int k = k0 + ((((lane & 7) ^ (lane >> 3)) ^ i) << 3);
+    lds_dma16((k < K) ? rowp_i + k : zero, sT + (wave * 64 + i * 8) * 8);
 }
 
-// Transposed tile [32 k][32 chunks]: an instruction covers 2 k-rows; wave w loads k-rows 8 w + 2 j + (lane >> 5),
-// j = 0..3; krow_j points at column 0 of the tile in the source row of that k (or at the zero page).  Slot lane & 31
+// Transposed tile [64 k][32 chunks]: an instruction covers 2 k-rows; wave w loads k-rows 16 w + 2 j + (lane >> 5),
+// j = 0..7; krow_j points at column 0 of the tile in the source row of that k (or at the zero page).  Slot lane & 31
 // holds logical chunk (lane & 31) ^ ((kr & 3) << 1), clamped to the last valid chunk of the row (columns past the
 // matrix edge are masked at the store).  Piece j of the tile (one instruction):
 __device__ __forceinline__ void issue_transposed_piece(u32x4 *sT, const uint16_t *krow_j, int j, int max_chunk, int wave,
@@ -68,14 +68,13 @@ __device__ __forceinline__ void issue_transposed_piece(u32x4 *sT, const uint16_t
     const int half = lane >> 5, p = lane & 31;
     int c = p ^ (((2 * j + half) & 3) << 1);
     if (c > max_chunk) c = max_chunk;
-    lds_dma16(krow_j + (c << 3), sT + (wave * 8 + j * 2) * 32);
+    lds_dma16(krow_j + (c << 3), sT + (wave * 16 + j * 2) * 32);
 }
 
 // MFMA fragment: 8 consecutive k (k block lane / 32 of k16 sub-step kk) of tile row R0 + lane % 32
 template <int TR> __device__ __forceinline__ u32x4 read_frag(const u32x4 *sT, int R0, int kk, int lane) {
     if (TR == 0) {
-        const int row = R0 + (lane & 31), c = kk * 2 + (lane >> 5);
-        return sT[row * 4 + (c ^ ((row >> 1) & 3))];
+        return sT[lds_chunk(R0 + (lane & 31), kk * 2 + (lane >> 5))];
     } else {
         // ds_read_b64_tr_b16 works on groups of 16 lanes: lane p of a group supplies the address of 4 columns at one
         // k-row, and receives 4 consecutive k of one column.  With p -> (k-row kb + p / 4, columns mb + 4 (p % 4))
@@ -146,15 +145,9 @@ struct NoHook {
     __device__ __forceinline__ void operator()(int) const {}
 };
 
-// Wait until at most `younger` of this wave's VMEM operations are outstanding (they retire in order), i.e. until the
-// K step the next sub-step reads has landed, make sure this wave's LDS reads have returned, then meet the other
-// waves.  The immediate has to be a literal, hence the macro; "memory" keeps the compiler from moving LDS accesses
-// across it.
-#ifdef XMA_EXP_NO_VMWAIT
-#define XMA_WAIT_STEP_AND_BARRIER(younger) asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory")
-#else
-#define XMA_WAIT_STEP_AND_BARRIER(younger) asm volatile("s_waitcnt vmcnt(" #younger ") lgkmcnt(0)\n\ts_barrier" ::: "memory")
-#endif
+// Every LDS-DMA load of this wave has landed and its LDS reads have returned; then meet the other waves.  "memory"
+// keeps the compiler from moving LDS accesses across it.
+#define XMA_WAIT_LOADS_AND_BARRIER() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory")
 #define XMA_WAIT_ALL_LOADS() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
 
 template <int N> __device__ __forceinline__ void zero_acc(f32x16 (&acc)[N][N]) {
@@ -216,77 +209,84 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
     const int64_t row_lo = e ? a.offs[e - 1] : 0, row_hi = a.offs[e];
     const int tiles_m = (int)((row_hi - row_lo + BM - 1) / BM);
     const int m_tile = s_sched[1] % tiles_m, n_tile = s_sched[1] / tiles_m;
+#ifdef XMA_EXP_SAME_TILE
+    const int64_t row0 = row_lo;
+#else
     const int64_t row0 = row_lo + (int64_t)m_tile * BM;
+#endif
     const int rows_valid = (int)((row_hi - row0 < BM) ? row_hi - row0 : BM);
+#ifdef XMA_EXP_SAME_TILE
+    const int n0 = 0;
+#else
     const int n0 = n_tile * BN;
+#endif
     __syncthreads(); // s_pre is dead from here on
 
 
     // ---- loader set-up
     const uint16_t *zero = (const uint16_t *)g_zero_page;
-    const uint16_t *q_ptr[4];
+    const uint16_t *q_ptr[8];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        int r = wave * 64 + i * 16 + (lane >> 2);
+    for (int i = 0; i < 8; ++i) {
+        int r = wave * 64 + i * 8 + (lane >> 3);
         if (r >= rows_valid) r = rows_valid - 1; // duplicates, masked at the store
         const int64_t n = row0 + r;
         const int64_t src = a.x_grouped ? n : a.idx[n] / a.fan_out;
         q_ptr[i] = a.X + src * a.ldx;
     }
     const uint16_t *We = a.W + (int64_t)e * a.w_es;
-    const uint16_t *p_ptr[4];
+    const uint16_t *p_ptr[8];
     int p_max_chunk = 0;
     if (WT == 0) {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            int r = n0 + wave * 64 + i * 16 + (lane >> 2);
+        for (int i = 0; i < 8; ++i) {
+            int r = n0 + wave * 64 + i * 8 + (lane >> 3);
             if (r >= a.N) r = a.N - 1;
             p_ptr[i] = We + (int64_t)r * a.ldw;
         }
     } else {
         p_max_chunk = ((a.N - n0) >> 3) - 1; // last valid 16-byte chunk of the tile's column range
 #pragma unroll
-        for (int j = 0; j < 4; ++j) p_ptr[j] = We + (int64_t)(wave * 8 + 2 * j + (lane >> 5)) * a.ldw + n0;
+        for (int j = 0; j < 8; ++j) p_ptr[j] = We + (int64_t)(wave * 16 + 2 * j + (lane >> 5)) * a.ldw + n0;
     }
     const int KT = (a.K + BK - 1) / BK;
 
-    // piece 0..7 of K step kt -> stage kt % NSTAGE (pieces 0..3 = Q tile, 4..7 = P tile); steps past the end read zeros
+    // piece 0..15 of K step kt -> stage kt & 1 (pieces 0..7 = Q tile, 8..15 = P tile); chunks past K read zeros
     auto issue_piece = [&](int kt, int piece) {
-        u32x4 *sQ = tiles + (kt & (NSTAGE - 1)) * STAGE_CHUNKS, *sP = sQ + OP_CHUNKS;
+        u32x4 *sQ = tiles + (kt & 1) * STAGE_CHUNKS, *sP = sQ + OP_CHUNKS;
         const int k0 = kt * BK;
-        if (piece < 4) {
+        if (piece < 8) {
             issue_rowmajor_piece(sQ, q_ptr[piece], piece, k0, a.K, wave, lane, zero);
         } else if (WT == 0) {
-            issue_rowmajor_piece(sP, p_ptr[piece - 4], piece - 4, k0, a.K, wave, lane, zero);
+            issue_rowmajor_piece(sP, p_ptr[piece - 8], piece - 8, k0, a.K, wave, lane, zero);
         } else {
-            const int j = piece - 4;
-            const int k = k0 + wave * 8 + 2 * j + (lane >> 5);
+            const int j = piece - 8;
+            const int k = k0 + wave * 16 + 2 * j + (lane >> 5);
             issue_transposed_piece(sP, (k < a.K) ? p_ptr[j] + (int64_t)k0 * a.ldw : zero, j, p_max_chunk, wave, lane);
         }
-    };
-    auto issue = [&](int kt) {
-#pragma unroll
-        for (int piece = 0; piece < 8; ++piece) issue_piece(kt, piece);
     };
 
     f32x16 acc[4][4];
     zero_acc(acc);
     const int wq = (wave & 1) * 128, wp = (wave >> 1) * 128; // wave's 128 x 128 corner inside the tile
 
-    issue(0);
-    issue(1);
-    issue(2);
-    XMA_WAIT_STEP_AND_BARRIER(16); // step 0 has landed in every wave
+#pragma unroll
+    for (int piece = 0; piece < 16; ++piece) issue_piece(0, piece);
+#pragma unroll
+    for (int piece = 0; piece < 16; ++piece) issue_piece(1, piece);
+    asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory"); // step 0 has landed in every wave; step 1 is in flight
     Frags f0, f1;
     load_frags<WT, 0>(f0, tiles, 0, wp, wq, lane);
     for (int kt = 0; kt < KT; ++kt) {
-        const u32x4 *cur = tiles + (kt & (NSTAGE - 1)) * STAGE_CHUNKS;
-        const u32x4 *nxt = tiles + ((kt + 1) & (NSTAGE - 1)) * STAGE_CHUNKS;
-        // the loads of step kt + 3 go out one per MFMA slot; their stage held step kt - 1, which every wave left
-        // before the previous barrier
-        mma_step<T, WT, 0>(f0, f1, cur, 1, wp, wq, lane, acc, [&](int g) { issue_piece(kt + 3, g); });
-        XMA_WAIT_STEP_AND_BARRIER(16); // steps kt + 2 and kt + 3 may still be in flight; kt + 1 has landed
-        mma_step<T, WT, 0>(f1, f0, nxt, 0, wp, wq, lane, acc, NoHook());
+        const u32x4 *cur = tiles + (kt & 1) * STAGE_CHUNKS;
+        const u32x4 *nxt = tiles + ((kt + 1) & 1) * STAGE_CHUNKS;
+        // second half of the loads of step kt + 1 (their first half went out behind the previous barrier)
+        mma_step<T, WT, 0>(f0, f1, cur, 1, wp, wq, lane, acc, [&](int g) { if (kt > 0) issue_piece(kt + 1, 8 + g); });
+        mma_step<T, WT, 0>(f1, f0, cur, 2, wp, wq, lane, acc, NoHook());
+        mma_step<T, WT, 0>(f0, f1, cur, 3, wp, wq, lane, acc, NoHook());
+        XMA_WAIT_LOADS_AND_BARRIER(); // step kt + 1 has landed; nobody reads this stage any more
+        // this stage is free now: first half of the loads of step kt + 2 (a step past the end reads zeros, never used)
+        mma_step<T, WT, 0>(f1, f0, nxt, 0, wp, wq, lane, acc, [&](int g) { issue_piece(kt + 2, g); });
     }
     XMA_WAIT_ALL_LOADS();
 
@@ -366,101 +366,84 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
     const int KT = (rows + BK - 1) / BK;
     const uint16_t *zero = (const uint16_t *)g_zero_page;
     const int q_max_chunk = ((a.N_out - o0) >> 3) - 1, p_max_chunk = ((a.K_in - i0) >> 3) - 1;
-    const int kr_lane = wave * 8 + (lane >> 5); // this lane's k-rows of a step: kr_lane + 2 j
+    const int kr_lane = wave * 16 + (lane >> 5); // this lane's k-rows of a step: kr_lane + 2 j, j = 0..7
 
-    // scattered indices of this lane's 4 tokens for two K steps of the prefetch ring: even steps in idx_even, odd in idx_odd
-    uint32_t idx_even[4], idx_odd[4];
-    auto load_idx = [&](int kt, uint32_t (&slot)[4]) {
+    // Scattered indices of this lane's 8 tokens of the step that is loaded next.  They are fetched one step ahead with
+    // inline assembly (low dword of the int64 index): the compiler would guard the later use of a loop-carried loaded
+    // register with a wait of its own choosing; here the wait is the vmcnt(0) in front of each step's barrier, and
+    // use_idx() ties the registers to a point behind it.
+    uint32_t idx_next[8];
+    auto load_idx = [&](int kt) {
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            // clamped, never predicated: every wave must issue exactly 4 loads here for the vmcnt arithmetic below
-            // Inline assembly (low dword of the int64 index): the compiler would guard the later use of a loop-carried
-            // loaded register with s_waitcnt vmcnt(0) and drain the LDS-DMA pipeline; wait_idx() does the exact wait.
+        for (int j = 0; j < 8; ++j) {
             int r = kt * BK + kr_lane + 2 * j;
-            if (r >= rows) r = rows - 1;
+            if (r >= rows) r = rows - 1; // clamped, never predicated
             const int64_t *src = a.idx + row_lo + r;
-            asm volatile("global_load_dword %0, %1, off" : "=v"(slot[j]) : "v"(src) : "memory");
+            asm volatile("global_load_dword %0, %1, off" : "=v"(idx_next[j]) : "v"(src) : "memory");
         }
     };
-    // The indices in `slot` were loaded two K steps ago; since then this wave issued one step of DMA (8) and one set of
-    // indices (4).  VMEM operations retire in order.
-    auto wait_idx = [&](uint32_t (&slot)[4]) {
-        asm volatile("s_waitcnt vmcnt(12)" : "+v"(slot[0]), "+v"(slot[1]), "+v"(slot[2]), "+v"(slot[3]));
+    auto use_idx = [&]() {
+        asm volatile("s_waitcnt vmcnt(0)"
+                     : "+v"(idx_next[0]), "+v"(idx_next[1]), "+v"(idx_next[2]), "+v"(idx_next[3]), "+v"(idx_next[4]),
+                       "+v"(idx_next[5]), "+v"(idx_next[6]), "+v"(idx_next[7]));
     };
-    // piece 0..7 of K step kt (0..3 = dY tile, 4..7 = X tile); `slot` holds the step's scattered indices
-    auto issue_piece = [&](int kt, const uint32_t (&slot)[4], int piece) {
-        u32x4 *sQ = tiles + (kt & (NSTAGE - 1)) * STAGE_CHUNKS, *sP = sQ + OP_CHUNKS;
-        const int j = piece & 3;
+    // piece 0..15 of K step kt (0..7 = dY tile, 8..15 = X tile)
+    auto issue_piece = [&](int kt, int piece) {
+        u32x4 *sQ = tiles + (kt & 1) * STAGE_CHUNKS, *sP = sQ + OP_CHUNKS;
+        const int j = piece & 7;
         const int r = kt * BK + kr_lane + 2 * j;
         int64_t src = row_lo + r;
-        if (piece < 4) {
-            if (GATHER && !a.dy_grouped) src = fastdiv(slot[j], a.dy_div);
+        if (piece < 8) {
+            if (GATHER && !a.dy_grouped) src = fastdiv(idx_next[j], a.dy_div);
             issue_transposed_piece(sQ, (r < rows) ? a.DY + src * a.lddy + o0 : zero, j, q_max_chunk, wave, lane);
         } else {
-            if (GATHER && !a.x_grouped) src = fastdiv(slot[j], a.x_div);
+            if (GATHER && !a.x_grouped) src = fastdiv(idx_next[j], a.x_div);
             issue_transposed_piece(sP, (r < rows) ? a.X + src * a.ldx + i0 : zero, j, p_max_chunk, wave, lane);
         }
-    };
-    auto issue = [&](int kt, const uint32_t (&slot)[4]) {
-#pragma unroll
-        for (int piece = 0; piece < 8; ++piece) issue_piece(kt, slot, piece);
     };
 
     f32x16 acc[4][4];
     zero_acc(acc);
     const int wq = (wave & 1) * 128, wp = (wave >> 1) * 128;
     if (KT > 0) {
-        // VMEM order per wave (GATHER): idx(0) idx(1) dma(0) idx(2) dma(1) idx(3) dma(2) idx(4), then per iteration kt:
-        // dma(kt + 3) idx(kt + 5).  The indices of a step are loaded two steps before they are consumed, so two younger
-        // steps of loads may stay in flight at that point.  The loop is unrolled by two so that the two index slots
-        // are fixed registers; a trailing odd step multiplies zeros.
+        // VMEM order per wave: idx(0) | dma(0) idx(1) | dma(1) idx(2) | loop kt: dma(kt+1)[8..15] ... idx(kt+3) ... wait(0),
+        // barrier, dma(kt+2)[0..7].  Indices are always loaded before a vmcnt(0) that precedes their use.
         if (GATHER) {
-            load_idx(0, idx_even);
-            load_idx(1, idx_odd);
+            load_idx(0);
+            use_idx();
         }
+#pragma unroll
+        for (int piece = 0; piece < 16; ++piece) issue_piece(0, piece);
         __builtin_amdgcn_sched_barrier(0);
-        if (GATHER) asm volatile("s_waitcnt vmcnt(0)" : "+v"(idx_even[0]), "+v"(idx_even[1]), "+v"(idx_even[2]), "+v"(idx_even[3]),
-                                 "+v"(idx_odd[0]), "+v"(idx_odd[1]), "+v"(idx_odd[2]), "+v"(idx_odd[3]));
-        issue(0, idx_even);
+        if (GATHER) {
+            load_idx(1);
+            use_idx(); // vmcnt(0): also step 0 has landed
+        }
+#pragma unroll
+        for (int piece = 0; piece < 16; ++piece) issue_piece(1, piece);
         __builtin_amdgcn_sched_barrier(0);
-        if (GATHER) load_idx(2, idx_even);
+        if (GATHER) load_idx(2);
         __builtin_amdgcn_sched_barrier(0);
-        issue(1, idx_odd);
-        __builtin_amdgcn_sched_barrier(0);
-        if (GATHER) load_idx(3, idx_odd);
-        __builtin_amdgcn_sched_barrier(0);
-        if (GATHER) wait_idx(idx_even); // behind idx(2): dma(1) idx(3)
-        issue(2, idx_even);
-        __builtin_amdgcn_sched_barrier(0);
-        if (GATHER) load_idx(4, idx_even);
-        __builtin_amdgcn_sched_barrier(0);
-        // outstanding behind dma(0): idx(2) dma(1) idx(3) dma(2) idx(4) = 4 + 8 + 4 + 8 + 4
         if (GATHER)
-            XMA_WAIT_STEP_AND_BARRIER(28);
+            asm volatile("s_waitcnt vmcnt(24)\n\ts_barrier" ::: "memory"); // behind dma(0): [idx(1) waited] dma(1) idx(2)
         else
-            XMA_WAIT_STEP_AND_BARRIER(16);
+            asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");
         Frags f0, f1;
         load_frags<1, 1>(f0, tiles, 0, wp, wq, lane);
-
-        // one K step: the loads of step kt + 3 (its indices sit in `use`) go out one per MFMA slot of the first sub-step,
-        // then `use` is refilled with the indices of step kt + 5
-        auto k_step = [&](int kt, uint32_t (&use)[4]) {
-            const u32x4 *cur = tiles + (kt & (NSTAGE - 1)) * STAGE_CHUNKS;
-            const u32x4 *nxt = tiles + ((kt + 1) & (NSTAGE - 1)) * STAGE_CHUNKS;
-            if (GATHER) wait_idx(use);
-            mma_step<T, 1, 1>(f0, f1, cur, 1, wp, wq, lane, acc, [&](int g) { issue_piece(kt + 3, use, g); });
-            if (GATHER) load_idx(kt + 5, use);
+        for (int kt = 0; kt < KT; ++kt) {
+            const u32x4 *cur = tiles + (kt & 1) * STAGE_CHUNKS;
+            const u32x4 *nxt = tiles + ((kt + 1) & 1) * STAGE_CHUNKS;
+            // idx_next holds the indices of step kt + 2 from here to the end of the iteration, except in iteration 0,
+            // where the second half of step 1 was already issued by the prologue
+            mma_step<T, 1, 1>(f0, f1, cur, 1, wp, wq, lane, acc, [&](int g) { if (kt > 0) issue_piece(kt + 1, 8 + g); });
             __builtin_amdgcn_sched_barrier(0);
-            // behind dma(kt + 1): idx(kt + 3) dma(kt + 2) idx(kt + 4) dma(kt + 3) idx(kt + 5) = 28 operations
-            if (GATHER)
-                XMA_WAIT_STEP_AND_BARRIER(28);
-            else
-                XMA_WAIT_STEP_AND_BARRIER(16);
-            mma_step<T, 1, 1>(f1, f0, nxt, 0, wp, wq, lane, acc, NoHook());
-        };
-        for (int kt = 0; kt < KT; kt += 2) {
-            k_step(kt, idx_odd);      // step kt + 3 is odd
-            k_step(kt + 1, idx_even); // step kt + 4 is even
+            if (GATHER && kt > 0) load_idx(kt + 2);
+            __builtin_amdgcn_sched_barrier(0);
+            mma_step<T, 1, 1>(f1, f0, cur, 2, wp, wq, lane, acc, NoHook());
+            mma_step<T, 1, 1>(f0, f1, cur, 3, wp, wq, lane, acc, NoHook());
+            XMA_WAIT_LOADS_AND_BARRIER();
+            if (GATHER) use_idx();
+            mma_step<T, 1, 1>(f1, f0, nxt, 0, wp, wq, lane, acc, [&](int g) { issue_piece(kt + 2, g); });
         }
         XMA_WAIT_ALL_LOADS();
     }
