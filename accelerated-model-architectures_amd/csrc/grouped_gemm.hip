@@ -50,46 +50,83 @@ __device__ __forceinline__ void lds_dma16(const uint16_t *src, u32x4 *lds_wave_b
                                      (__attribute__((address_space(3))) void *)lds_wave_base, 16, 0, 0);
 }
 
-// Row-major tile [256][8 chunks]: an instruction covers 8 rows; wave w loads rows 64 w + 8 i + (lane >> 3), i = 0..7.
-// swz(r) = (r ^ (r >> 3)) & 7 = (lane >> 3) ^ i for these rows, so slot lane & 7 holds logical chunk
-// (lane & 7) ^ (lane >> 3) ^ i.  Piece i of the tile (one instruction):
-__device__ __forceinline__ void issue_rowmajor_piece(u32x4 *sT, const uint16_t *rowp_i, int i, int k0, int K, int wave,
-                                                     int lane, const uint16_t *zero) {
-    const int k = k0 + ((((lane & 7) ^ (lane >> 3)) ^ i) << 3);
-    lds_dma16((k < K) ? rowp_i + k : zero, sT + (wave * 64 + i * 8) * 8);
+template <int N> struct IC {
+    static constexpr int value = N;
+};
+// compile-time loop: f(IC<0>{}), ..., f(IC<N-1>{}) - the index is a constant expression inside f (asm immediates)
+template <int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (N > 0) {
+        static_for<N - 1>(f);
+        f(IC<N - 1>{});
+    }
 }
 
-// Transposed tile [64 k][32 chunks]: an instruction covers 2 k-rows; wave w loads k-rows 16 w + 2 j + (lane >> 5),
-// j = 0..7; krow_j points at column 0 of the tile in the source row of that k (or at the zero page).  Slot lane & 31
-// holds logical chunk (lane & 31) ^ ((kr & 3) << 1), clamped to the last valid chunk of the row (columns past the
-// matrix edge are masked at the store).  Piece j of the tile (one instruction):
-__device__ __forceinline__ void issue_transposed_piece(u32x4 *sT, const uint16_t *krow_j, int j, int max_chunk, int wave,
-                                                       int lane) {
-    const int half = lane >> 5, p = lane & 31;
-    int c = p ^ (((2 * j + half) & 3) << 1);
-    if (c > max_chunk) c = max_chunk;
-    lds_dma16(krow_j + (c << 3), sT + (wave * 16 + j * 2) * 32);
+// ---- LDS layouts (byte offsets inside one 32 KB operand tile)
+//
+// Row-major tile [256 rows][8 chunks of 16 B]: chunk c of row r sits at slot c ^ (r & 7).  An LDS-DMA instruction
+// covers 8 rows (1 KB); wave w loads rows 64 w + 8 i + (lane >> 3), i = 0..7, and lane fills slot lane & 7, i.e. it
+// fetches logical chunk (lane & 7) ^ (lane >> 3) - the same for every i, so a lane's global address of piece i is a
+// fixed per-lane pointer plus the K offset of the step.
+__device__ __forceinline__ int rowmajor_lane_chunk(int lane) { return (lane & 7) ^ (lane >> 3); }
+// MFMA fragment of rows R0 + 32 i + (lane & 31), k16 sub-step kk: since R0 and 32 i are multiples of 8 the slot is
+// ((2 kk + (lane >> 5)) ^ (lane & 7)): one per-lane byte offset per kk, and i is an immediate (4096 i).
+__device__ __forceinline__ uint32_t rowmajor_frag_offset(int R0, int kk, int lane) {
+    return (uint32_t)((R0 + (lane & 31)) * 128 + (((2 * kk + (lane >> 5)) ^ (lane & 7)) << 4));
+}
+//
+// Transposed tile [64 k-rows][32 chunks of 16 B], exactly as in memory: chunk c of k-row kr sits at slot
+// c ^ ((kr & 3) << 1).  An LDS-DMA instruction covers 2 k-rows; wave w loads k-rows 16 w + 2 j + (lane >> 5), j = 0..7,
+// and lane fills slot lane & 31, i.e. it fetches logical chunk (lane & 31) ^ (((2 j + (lane >> 5)) & 3) << 1).
+__device__ __forceinline__ int transposed_lane_chunk(int j, int lane) {
+    return (lane & 31) ^ (((2 * j + (lane >> 5)) & 3) << 1);
+}
+// MFMA fragment through ds_read_b64_tr_b16, which works on groups of 16 lanes: lane p of a group supplies the
+// address of 4 columns at one k-row and receives 4 consecutive k of one column.  With
+// p -> (k-row kb + p / 4, columns mb + 4 (p % 4)) lane p ends up with column mb + p, k = kb .. kb + 3; two reads
+// (kb and kb + 4) give the 8 k of an MFMA operand.  For the 32-row block i of the wave's 128 rows the chunk index is
+// (R0 / 8 + 4 i + c_lane) ^ s with s in {0, 2, 4, 6}: blocks 0 and 1 need one per-lane offset each, blocks 2 and 3
+// are those plus 128 bytes; kk adds 8192 bytes, the second read 2048.
+__device__ __forceinline__ uint32_t transposed_frag_offset(int R0, int odd, int lane) {
+    const int p = lane & 15, G = lane >> 4;
+    const int m = R0 + odd * 32 + ((G & 1) << 4) + ((p & 3) << 2);
+    const int kr = ((G >> 1) << 3) + (p >> 2);
+    return (uint32_t)(kr * 512 + ((((m >> 3) ^ ((kr & 3) << 1))) << 4) + ((m & 7) << 1));
 }
 
-// MFMA fragment: 8 consecutive k (k block lane / 32 of k16 sub-step kk) of tile row R0 + lane % 32
-template <int TR> __device__ __forceinline__ u32x4 read_frag(const u32x4 *sT, int R0, int kk, int lane) {
-    if (TR == 0) {
-        return sT[lds_chunk(R0 + (lane & 31), kk * 2 + (lane >> 5))];
+// per-lane LDS byte addresses of one operand's fragments in the CURRENT stage
+template <int TR> struct FragBase {
+    uint32_t b[TR ? 2 : 4]; // row-major: one per kk; transposed: blocks 0/2 and blocks 1/3
+};
+
+template <int TR> __device__ __forceinline__ void make_frag_base(FragBase<TR> &f, uint32_t tile_lds_addr, int R0, int lane) {
+    if constexpr (TR == 0) {
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) f.b[kk] = tile_lds_addr + rowmajor_frag_offset(R0, kk, lane);
     } else {
-        // ds_read_b64_tr_b16 works on groups of 16 lanes: lane p of a group supplies the address of 4 columns at one
-        // k-row, and receives 4 consecutive k of one column.  With p -> (k-row kb + p / 4, columns mb + 4 (p % 4))
-        // lane p ends up with column mb + p, k = kb .. kb + 3.
-        const int p = lane & 15, G = lane >> 4;
-        const int m = R0 + ((G & 1) << 4) + ((p & 3) << 2);
-        const int kr = kk * 16 + ((G >> 1) << 3) + (p >> 2);
-        const int byte = kr * 512 + ((((m >> 3) ^ ((kr & 3) << 1))) << 4) + ((m & 7) << 1);
-        // Issued as inline assembly: after an LDS-DMA load the compiler guards every LDS read it cannot prove
-        // disjoint with s_waitcnt vmcnt(0), which would drain the whole load pipeline at each fragment.  The price is
-        // that the compiler does not know these reads are in flight: wait_frags() below must precede their use.
-        const unsigned addr = (unsigned)(size_t)((__attribute__((address_space(3))) const char *)((const char *)sT + byte));
+        f.b[0] = tile_lds_addr + transposed_frag_offset(R0, 0, lane);
+        f.b[1] = tile_lds_addr + transposed_frag_offset(R0, 1, lane);
+    }
+}
+template <int TR> __device__ __forceinline__ void flip_stage(FragBase<TR> &f) {
+#pragma unroll
+    for (int q = 0; q < (TR ? 2 : 4); ++q) f.b[q] ^= (uint32_t)(STAGE_CHUNKS * 16);
+}
+
+// All fragment reads are inline assembly with an immediate offset: (1) after an LDS-DMA load the compiler guards every
+// LDS read it cannot prove disjoint with s_waitcnt vmcnt(0), which would drain the load pipeline at each fragment;
+// (2) it keeps address arithmetic out of the MFMA stream.  The compiler therefore does not know these reads are in
+// flight: wait_frags() must precede their use.
+template <int TR, int I, int KK> __device__ __forceinline__ u32x4 read_frag(const FragBase<TR> &f) {
+    if constexpr (TR == 0) {
+        u32x4 r;
+        asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(f.b[KK]), "n"(I * 4096));
+        return r;
+    } else {
         u32x2 lo, hi;
-        asm volatile("ds_read_b64_tr_b16 %0, %1" : "=v"(lo) : "v"(addr));
-        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:2048" : "=v"(hi) : "v"(addr)); // + 4 k-rows
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(lo) : "v"(f.b[I & 1]), "n"(KK * 8192 + (I >> 1) * 128));
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2"
+                     : "=v"(hi)
+                     : "v"(f.b[I & 1]), "n"(KK * 8192 + (I >> 1) * 128 + 2048));
         u32x4 r = {lo[0], lo[1], hi[0], hi[1]};
         return r;
     }
@@ -107,43 +144,45 @@ __device__ __forceinline__ void wait_frags(Frags &f) {
                    "+v"(f.q[3]));
 }
 
-template <int PTR, int QTR>
-__device__ __forceinline__ void load_frags(Frags &f, const u32x4 *stage, int kk, int p_row0, int q_row0, int lane) {
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        f.p[i] = read_frag<PTR>(stage + OP_CHUNKS, p_row0 + i * 32, kk, lane);
-        f.q[i] = read_frag<QTR>(stage, q_row0 + i * 32, kk, lane);
-    }
+template <int PTR, int QTR, int KK>
+__device__ __forceinline__ void load_frags(Frags &f, const FragBase<PTR> &pb, const FragBase<QTR> &qb) {
+    static_for<4>([&](auto I) {
+        f.p[I.value] = read_frag<PTR, I.value, KK>(pb);
+        f.q[I.value] = read_frag<QTR, I.value, KK>(qb);
+    });
 }
 
 // The 16 MFMAs of one k16 sub-step on `cur` as 8 pinned slots.  Slot g: two MFMAs; for g < 4 one P and one Q fragment
-// read of (`stage`, kk) into `nxt`; then `hook(g)`, which the callers use to issue one LDS-DMA load (with its address
-// arithmetic) per slot.  A wave issues in order, so anything not placed between MFMAs would leave the matrix pipe
-// idle for as long as it takes to issue; all fragment reads sit in the first half so that the second half covers
-// their latency.
-template <typename T, int PTR, int QTR, typename Hook>
-__device__ __forceinline__ void mma_step(Frags &cur, Frags &nxt, const u32x4 *stage, int kk, int p_row0, int q_row0,
-                                         int lane, f32x16 (&acc)[4][4], Hook hook) {
-    if (PTR || QTR) wait_frags(cur); // issued at least 8 MFMAs ago
-#pragma unroll
-    for (int g = 0; g < 8; ++g) {
+// read of sub-step KK (of the stage pb/qb point at) into `nxt`; then `hook(IC<g>)`, which the callers use to issue one
+// LDS-DMA load per slot.  A wave issues in order, so anything not placed between MFMAs would leave the matrix pipe idle
+// for as long as it takes to issue; all fragment reads sit in the first half so that the second half covers their
+// latency.
+template <typename T, int PTR, int QTR, int KK, typename Hook>
+__device__ __forceinline__ void mma_step(Frags &cur, Frags &nxt, const FragBase<PTR> &pb, const FragBase<QTR> &qb,
+                                         f32x16 (&acc)[4][4], Hook hook) {
+    wait_frags(cur); // issued at least 8 MFMAs ago
+    static_for<8>([&](auto G) {
+        constexpr int g = G.value, j = g >> 1, i0 = (g & 1) * 2;
         __builtin_amdgcn_sched_barrier(0);
-        const int j = g >> 1, i0 = (g & 1) * 2;
         acc[j][i0] = Elem<T>::mfma(cur.p[j], cur.q[i0], acc[j][i0]);
         acc[j][i0 + 1] = Elem<T>::mfma(cur.p[j], cur.q[i0 + 1], acc[j][i0 + 1]);
         __builtin_amdgcn_sched_barrier(0);
-        if (g < 4) {
-            nxt.p[g] = read_frag<PTR>(stage + OP_CHUNKS, p_row0 + g * 32, kk, lane);
-            nxt.q[g] = read_frag<QTR>(stage, q_row0 + g * 32, kk, lane);
+        if constexpr (g < 4) {
+            nxt.p[g] = read_frag<PTR, g, KK>(pb);
+            nxt.q[g] = read_frag<QTR, g, KK>(qb);
         }
-        hook(g);
-    }
+        hook(G);
+    });
     __builtin_amdgcn_sched_barrier(0);
 }
 
 struct NoHook {
-    __device__ __forceinline__ void operator()(int) const {}
+    template <typename G> __device__ __forceinline__ void operator()(G) const {}
 };
+
+__device__ __forceinline__ uint32_t lds_addr_of(const void *p) {
+    return (uint32_t)(size_t)((__attribute__((address_space(3))) const char *)p);
+}
 
 // Every LDS-DMA load of this wave has landed and its LDS reads have returned; then meet the other waves.  "memory"
 // keeps the compiler from moving LDS accesses across it.
@@ -223,71 +262,100 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
     __syncthreads(); // s_pre is dead from here on
 
 
-    // ---- loader set-up
+    // ---- loader set-up: one fixed per-lane global pointer per LDS-DMA piece (k = 0); a step adds a uniform offset
     const uint16_t *zero = (const uint16_t *)g_zero_page;
-    const uint16_t *q_ptr[8];
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        int r = wave * 64 + i * 8 + (lane >> 3);
-        if (r >= rows_valid) r = rows_valid - 1; // duplicates, masked at the store
-        const int64_t n = row0 + r;
-        const int64_t src = a.x_grouped ? n : a.idx[n] / a.fan_out;
-        q_ptr[i] = a.X + src * a.ldx;
-    }
-    const uint16_t *We = a.W + (int64_t)e * a.w_es;
-    const uint16_t *p_ptr[8];
-    int p_max_chunk = 0;
-    if (WT == 0) {
+    const int KT = (a.K + BK - 1) / BK;
+    const bool k_tail = (a.K & (BK - 1)) != 0; // the last step has chunks past K: they are fetched from the zero page
+    const uint16_t *q_ptr[8], *p_ptr[8];
+    {
+        const int c = rowmajor_lane_chunk(lane);
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            int r = n0 + wave * 64 + i * 8 + (lane >> 3);
-            if (r >= a.N) r = a.N - 1;
-            p_ptr[i] = We + (int64_t)r * a.ldw;
+            int r = wave * 64 + i * 8 + (lane >> 3);
+            if (r >= rows_valid) r = rows_valid - 1; // duplicates, masked at the store
+            const int64_t n = row0 + r;
+            const int64_t src = a.x_grouped ? n : a.idx[n] / a.fan_out;
+            q_ptr[i] = a.X + src * a.ldx + c * 8;
         }
-    } else {
-        p_max_chunk = ((a.N - n0) >> 3) - 1; // last valid 16-byte chunk of the tile's column range
+        const uint16_t *We = a.W + (int64_t)e * a.w_es;
+        if (WT == 0) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) p_ptr[j] = We + (int64_t)(wave * 16 + 2 * j + (lane >> 5)) * a.ldw + n0;
-    }
-    const int KT = (a.K + BK - 1) / BK;
-
-    // piece 0..15 of K step kt -> stage kt & 1 (pieces 0..7 = Q tile, 8..15 = P tile); chunks past K read zeros
-    auto issue_piece = [&](int kt, int piece) {
-        u32x4 *sQ = tiles + (kt & 1) * STAGE_CHUNKS, *sP = sQ + OP_CHUNKS;
-        const int k0 = kt * BK;
-        if (piece < 8) {
-            issue_rowmajor_piece(sQ, q_ptr[piece], piece, k0, a.K, wave, lane, zero);
-        } else if (WT == 0) {
-            issue_rowmajor_piece(sP, p_ptr[piece - 8], piece - 8, k0, a.K, wave, lane, zero);
+            for (int i = 0; i < 8; ++i) {
+                int r = n0 + wave * 64 + i * 8 + (lane >> 3);
+                if (r >= a.N) r = a.N - 1;
+                p_ptr[i] = We + (int64_t)r * a.ldw + c * 8;
+            }
         } else {
-            const int j = piece - 8;
-            const int k = k0 + wave * 16 + 2 * j + (lane >> 5);
-            issue_transposed_piece(sP, (k < a.K) ? p_ptr[j] + (int64_t)k0 * a.ldw : zero, j, p_max_chunk, wave, lane);
+            const int max_chunk = ((a.N - n0) >> 3) - 1; // last valid 16-byte chunk of the tile's column range
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                int cj = transposed_lane_chunk(j, lane);
+                if (cj > max_chunk) cj = max_chunk; // columns past the edge are masked at the store
+                p_ptr[j] = We + (int64_t)(wave * 16 + 2 * j + (lane >> 5)) * a.ldw + n0 + cj * 8;
+            }
         }
+    }
+    const int64_t p_step = (WT == 0) ? BK : (int64_t)BK * a.ldw; // elements per K step along the P pointers
+    const uint32_t lds0 = lds_addr_of(smem);
+
+    // piece 0..15 of K step kt -> stage kt & 1 (pieces 0..7 = Q tile, 8..15 = P tile).  FULL: the caller guarantees
+    // that step kt exists and has no chunk past K, so the piece is one M0 update, one 64-bit add and the load; a wave
+    // with a single instruction stream cannot afford more than a few instructions per MFMA.
+    auto issue_piece = [&](int kt, auto PIECE, auto FULL) {
+        constexpr int piece = PIECE.value;
+        constexpr int slot =
+            (piece >> 3) * OP_CHUNKS + ((piece < 8 || WT == 0) ? (piece & 7) * 64 : (piece & 7) * 64); // 1 KB per piece
+        if constexpr (!FULL.value) {
+            if (kt >= KT) return; // uniform
+        }
+        u32x4 *dst = tiles + (kt & 1) * STAGE_CHUNKS + slot + wave * 512; // a wave's 8 pieces are 8 KB apart per wave
+        const uint16_t *src = (piece < 8) ? q_ptr[piece] + (int64_t)kt * BK : p_ptr[piece - 8] + (int64_t)kt * p_step;
+        if constexpr (!FULL.value) {
+            if (k_tail && kt == KT - 1) { // uniform branch, taken by at most one step of a tile
+                asm volatile("" ::: "memory"); // keeps this rare path a branch instead of selects in every piece
+                if (piece < 8 || WT == 0) {
+                    if (kt * BK + rowmajor_lane_chunk(lane) * 8 >= a.K) src = zero;
+                } else {
+                    if (kt * BK + wave * 16 + 2 * (piece - 8) + (lane >> 5) >= a.K) src = zero;
+                }
+            }
+        }
+        lds_dma16(src, dst);
     };
 
     f32x16 acc[4][4];
     zero_acc(acc);
     const int wq = (wave & 1) * 128, wp = (wave >> 1) * 128; // wave's 128 x 128 corner inside the tile
+    FragBase<0> qb;
+    FragBase<WT> pb;
+    make_frag_base<0>(qb, lds0, wq, lane);
+    make_frag_base<WT>(pb, lds0 + OP_CHUNKS * 16, wp, lane);
 
-#pragma unroll
-    for (int piece = 0; piece < 16; ++piece) issue_piece(0, piece);
-#pragma unroll
-    for (int piece = 0; piece < 16; ++piece) issue_piece(1, piece);
-    asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory"); // step 0 has landed in every wave; step 1 is in flight
+    static_for<16>([&](auto P) { issue_piece(0, P, IC<0>{}); });
+    static_for<8>([&](auto P) { issue_piece(1, P, IC<0>{}); });
+    // step 0 has landed in every wave (the first half of step 1 may be in flight)
+    if (KT > 1)
+        asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+    else
+        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     Frags f0, f1;
-    load_frags<WT, 0>(f0, tiles, 0, wp, wq, lane);
-    for (int kt = 0; kt < KT; ++kt) {
-        const u32x4 *cur = tiles + (kt & 1) * STAGE_CHUNKS;
-        const u32x4 *nxt = tiles + ((kt + 1) & 1) * STAGE_CHUNKS;
-        // second half of the loads of step kt + 1 (their first half went out behind the previous barrier)
-        mma_step<T, WT, 0>(f0, f1, cur, 1, wp, wq, lane, acc, [&](int g) { if (kt > 0) issue_piece(kt + 1, 8 + g); });
-        mma_step<T, WT, 0>(f1, f0, cur, 2, wp, wq, lane, acc, NoHook());
-        mma_step<T, WT, 0>(f0, f1, cur, 3, wp, wq, lane, acc, NoHook());
+    load_frags<WT, 0, 0>(f0, pb, qb);
+    // one K step; FULL: steps kt + 1 and kt + 2 exist and are complete
+    auto k_step = [&](int kt, auto FULL) {
+        // second half of the loads of step kt + 1 (the first half went out behind the previous barrier)
+        mma_step<T, WT, 0, 1>(f0, f1, pb, qb, acc, [&](auto G) { issue_piece(kt + 1, IC<8 + G.value>{}, FULL); });
+        mma_step<T, WT, 0, 2>(f1, f0, pb, qb, acc, NoHook());
+        mma_step<T, WT, 0, 3>(f0, f1, pb, qb, acc, NoHook());
         XMA_WAIT_LOADS_AND_BARRIER(); // step kt + 1 has landed; nobody reads this stage any more
-        // this stage is free now: first half of the loads of step kt + 2 (a step past the end reads zeros, never used)
-        mma_step<T, WT, 0>(f1, f0, nxt, 0, wp, wq, lane, acc, [&](int g) { issue_piece(kt + 2, g); });
-    }
+        flip_stage(pb);
+        flip_stage(qb);
+        // the stage just left is free: first half of the loads of step kt + 2; fragments of sub-step 0 of step kt + 1
+        mma_step<T, WT, 0, 0>(f1, f0, pb, qb, acc, [&](auto G) { issue_piece(kt + 2, G, FULL); });
+    };
+    const int KT_full = a.K / BK; // steps without a chunk past K
+    int kt = 0;
+    for (; kt + 2 < KT_full; ++kt) k_step(kt, IC<1>{});
+    for (; kt < KT; ++kt) k_step(kt, IC<0>{});
     XMA_WAIT_ALL_LOADS();
 
     // ---- epilogue: lane owns row (lane & 31) of each 32-row block; quad g of tile (j, i) holds
@@ -368,6 +436,24 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
     const int q_max_chunk = ((a.N_out - o0) >> 3) - 1, p_max_chunk = ((a.K_in - i0) >> 3) - 1;
     const int kr_lane = wave * 16 + (lane >> 5); // this lane's k-rows of a step: kr_lane + 2 j, j = 0..7
 
+    // Per-lane column offsets (elements) of the 8 pieces of each operand; rows change every step.  For an operand in
+    // grouped order the row is row_lo + 64 kt + kr, so the piece pointer advances by a uniform 64 ld per step.
+    int q_col[8], p_col[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        int cq = transposed_lane_chunk(j, lane), cp = cq;
+        if (cq > q_max_chunk) cq = q_max_chunk; // columns past the edge are masked at the store
+        if (cp > p_max_chunk) cp = p_max_chunk;
+        q_col[j] = o0 + cq * 8;
+        p_col[j] = i0 + cp * 8;
+    }
+    const uint16_t *q_grp[8], *p_grp[8]; // grouped-order pointers at step 0
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        q_grp[j] = a.DY + (row_lo + kr_lane + 2 * j) * a.lddy + q_col[j];
+        p_grp[j] = a.X + (row_lo + kr_lane + 2 * j) * a.ldx + p_col[j];
+    }
+
     // Scattered indices of this lane's 8 tokens of the step that is loaded next.  They are fetched one step ahead with
     // inline assembly (low dword of the int64 index): the compiler would guard the later use of a loop-carried loaded
     // register with a wait of its own choosing; here the wait is the vmcnt(0) in front of each step's barrier, and
@@ -387,64 +473,83 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
                      : "+v"(idx_next[0]), "+v"(idx_next[1]), "+v"(idx_next[2]), "+v"(idx_next[3]), "+v"(idx_next[4]),
                        "+v"(idx_next[5]), "+v"(idx_next[6]), "+v"(idx_next[7]));
     };
-    // piece 0..15 of K step kt (0..7 = dY tile, 8..15 = X tile)
-    auto issue_piece = [&](int kt, int piece) {
-        u32x4 *sQ = tiles + (kt & 1) * STAGE_CHUNKS, *sP = sQ + OP_CHUNKS;
-        const int j = piece & 7;
-        const int r = kt * BK + kr_lane + 2 * j;
-        int64_t src = row_lo + r;
-        if (piece < 8) {
-            if (GATHER && !a.dy_grouped) src = fastdiv(idx_next[j], a.dy_div);
-            issue_transposed_piece(sQ, (r < rows) ? a.DY + src * a.lddy + o0 : zero, j, q_max_chunk, wave, lane);
-        } else {
-            if (GATHER && !a.x_grouped) src = fastdiv(idx_next[j], a.x_div);
-            issue_transposed_piece(sP, (r < rows) ? a.X + src * a.ldx + i0 : zero, j, p_max_chunk, wave, lane);
+    // piece 0..15 of K step kt (0..7 = dY tile, 8..15 = X tile); FULL: step kt exists and lies inside the expert's rows
+    auto issue_piece = [&](int kt, auto PIECE, auto FULL) {
+        constexpr int piece = PIECE.value, j = piece & 7;
+        if constexpr (!FULL.value) {
+            if (kt >= KT) return; // uniform
         }
+        u32x4 *dst = tiles + (kt & 1) * STAGE_CHUNKS + (piece >> 3) * OP_CHUNKS + j * 64 + wave * 512;
+        const uint16_t *src;
+        if constexpr (piece < 8) {
+            if (GATHER && !a.dy_grouped)
+                src = a.DY + (int64_t)fastdiv(idx_next[j], a.dy_div) * a.lddy + q_col[j];
+            else
+                src = q_grp[j] + (int64_t)kt * BK * a.lddy;
+        } else {
+            if (GATHER && !a.x_grouped)
+                src = a.X + (int64_t)fastdiv(idx_next[j], a.x_div) * a.ldx + p_col[j];
+            else
+                src = p_grp[j] + (int64_t)kt * BK * a.ldx;
+        }
+        if constexpr (!FULL.value) {
+            if (kt == KT - 1) { // uniform branch: k-rows past the expert's range come from the zero page
+                asm volatile("" ::: "memory"); // keeps this rare path a branch
+                if (kt * BK + kr_lane + 2 * j >= rows) src = zero;
+            }
+        }
+        lds_dma16(src, dst);
     };
 
     f32x16 acc[4][4];
     zero_acc(acc);
     const int wq = (wave & 1) * 128, wp = (wave >> 1) * 128;
     if (KT > 0) {
-        // VMEM order per wave: idx(0) | dma(0) idx(1) | dma(1) idx(2) | loop kt: dma(kt+1)[8..15] ... idx(kt+3) ... wait(0),
-        // barrier, dma(kt+2)[0..7].  Indices are always loaded before a vmcnt(0) that precedes their use.
+        // VMEM order per wave: idx(0) | dma(0) idx(1) | dma(1)[0..7] idx(2)? - see below; in the loop the indices of a
+        // step are always loaded before a vmcnt(0) that precedes their use.
+        const uint32_t lds0 = lds_addr_of(smem);
+        FragBase<1> qb, pb;
+        make_frag_base<1>(qb, lds0, wq, lane);
+        make_frag_base<1>(pb, lds0 + OP_CHUNKS * 16, wp, lane);
         if (GATHER) {
             load_idx(0);
             use_idx();
         }
-#pragma unroll
-        for (int piece = 0; piece < 16; ++piece) issue_piece(0, piece);
+        static_for<16>([&](auto P) { issue_piece(0, P, IC<0>{}); });
         __builtin_amdgcn_sched_barrier(0);
         if (GATHER) {
             load_idx(1);
-            use_idx(); // vmcnt(0): also step 0 has landed
+            use_idx(); // vmcnt(0): step 0 has landed as well
         }
-#pragma unroll
-        for (int piece = 0; piece < 16; ++piece) issue_piece(1, piece);
+        static_for<8>([&](auto P) { issue_piece(1, P, IC<0>{}); });
         __builtin_amdgcn_sched_barrier(0);
-        if (GATHER) load_idx(2);
-        __builtin_amdgcn_sched_barrier(0);
-        if (GATHER)
-            asm volatile("s_waitcnt vmcnt(24)\n\ts_barrier" ::: "memory"); // behind dma(0): [idx(1) waited] dma(1) idx(2)
+        // step 0 has landed in every wave; behind it at most the first half of step 1 (none if this is the only step)
+        if (KT > 1)
+            asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
         else
-            asm volatile("s_waitcnt vmcnt(16)\n\ts_barrier" ::: "memory");
+            asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
         Frags f0, f1;
-        load_frags<1, 1>(f0, tiles, 0, wp, wq, lane);
-        for (int kt = 0; kt < KT; ++kt) {
-            const u32x4 *cur = tiles + (kt & 1) * STAGE_CHUNKS;
-            const u32x4 *nxt = tiles + ((kt + 1) & 1) * STAGE_CHUNKS;
-            // idx_next holds the indices of step kt + 2 from here to the end of the iteration, except in iteration 0,
-            // where the second half of step 1 was already issued by the prologue
-            mma_step<T, 1, 1>(f0, f1, cur, 1, wp, wq, lane, acc, [&](int g) { if (kt > 0) issue_piece(kt + 1, 8 + g); });
+        load_frags<1, 1, 0>(f0, pb, qb);
+        // one K step; FULL: steps kt + 1 and kt + 2 lie completely inside the expert's rows
+        auto k_step = [&](int kt, auto FULL) {
+            // idx_next holds the indices of step kt + 1 here; the second half of that step's loads goes out now, then
+            // the indices of step kt + 2 are requested (they land before the barrier's vmcnt(0))
+            mma_step<T, 1, 1, 1>(f0, f1, pb, qb, acc, [&](auto G) { issue_piece(kt + 1, IC<8 + G.value>{}, FULL); });
             __builtin_amdgcn_sched_barrier(0);
-            if (GATHER && kt > 0) load_idx(kt + 2);
+            if (GATHER) load_idx(kt + 2);
             __builtin_amdgcn_sched_barrier(0);
-            mma_step<T, 1, 1>(f1, f0, cur, 2, wp, wq, lane, acc, NoHook());
-            mma_step<T, 1, 1>(f0, f1, cur, 3, wp, wq, lane, acc, NoHook());
+            mma_step<T, 1, 1, 2>(f1, f0, pb, qb, acc, NoHook());
+            mma_step<T, 1, 1, 3>(f0, f1, pb, qb, acc, NoHook());
             XMA_WAIT_LOADS_AND_BARRIER();
             if (GATHER) use_idx();
-            mma_step<T, 1, 1>(f1, f0, nxt, 0, wp, wq, lane, acc, [&](int g) { issue_piece(kt + 2, g); });
-        }
+            flip_stage(pb);
+            flip_stage(qb);
+            mma_step<T, 1, 1, 0>(f1, f0, pb, qb, acc, [&](auto G) { issue_piece(kt + 2, G, FULL); });
+        };
+        const int KT_full = rows / BK;
+        int kt = 0;
+        for (; kt + 2 < KT_full; ++kt) k_step(kt, IC<1>{});
+        for (; kt < KT; ++kt) k_step(kt, IC<0>{});
         XMA_WAIT_ALL_LOADS();
     }
 
