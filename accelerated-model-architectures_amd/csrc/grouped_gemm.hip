@@ -341,22 +341,53 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
     Frags f0, f1;
     load_frags<WT, 0, 0>(f0, pb, qb);
     // one K step; FULL: steps kt + 1 and kt + 2 exist and are complete
+#ifdef XMA_EXP_TIMING2
+    uint64_t acc_t[5] = {0, 0, 0, 0, 0};
+#endif
     auto k_step = [&](int kt, auto FULL) {
+#ifdef XMA_EXP_TIMING2
+        const uint64_t ta = wall_clock64();
+#endif
         // second half of the loads of step kt + 1 (the first half went out behind the previous barrier)
         mma_step<T, WT, 0, 1>(f0, f1, pb, qb, acc, [&](auto G) { issue_piece(kt + 1, IC<8 + G.value>{}, FULL); });
+#ifdef XMA_EXP_TIMING2
+        const uint64_t tb = wall_clock64();
+#endif
         mma_step<T, WT, 0, 2>(f1, f0, pb, qb, acc, NoHook());
         mma_step<T, WT, 0, 3>(f0, f1, pb, qb, acc, NoHook());
+#ifdef XMA_EXP_TIMING2
+        const uint64_t tc = wall_clock64();
+        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        const uint64_t td = wall_clock64();
+#endif
         XMA_WAIT_LOADS_AND_BARRIER(); // step kt + 1 has landed; nobody reads this stage any more
+#ifdef XMA_EXP_TIMING2
+        const uint64_t te = wall_clock64();
+#endif
         flip_stage(pb);
         flip_stage(qb);
         // the stage just left is free: first half of the loads of step kt + 2; fragments of sub-step 0 of step kt + 1
         mma_step<T, WT, 0, 0>(f1, f0, pb, qb, acc, [&](auto G) { issue_piece(kt + 2, G, FULL); });
+#ifdef XMA_EXP_TIMING2
+        const uint64_t tf = wall_clock64();
+        acc_t[0] += tb - ta;
+        acc_t[1] += tc - tb;
+        acc_t[2] += td - tc;
+        acc_t[3] += te - td;
+        acc_t[4] += tf - te;
+#endif
     };
     const int KT_full = a.K / BK; // steps without a chunk past K
     int kt = 0;
     for (; kt + 2 < KT_full; ++kt) k_step(kt, IC<1>{});
     for (; kt < KT; ++kt) k_step(kt, IC<0>{});
     XMA_WAIT_ALL_LOADS();
+#ifdef XMA_EXP_TIMING2
+    if (EPI == XMA_ROCM_EPI_STORE && a.aux && lane == 0) {
+        uint64_t *dbg = (uint64_t *)a.aux + ((size_t)blockIdx.x * 4 + wave) * 8;
+        for (int q = 0; q < 5; ++q) dbg[q] = acc_t[q];
+    }
+#endif
 
     // ---- epilogue: lane owns row (lane & 31) of each 32-row block; quad g of tile (j, i) holds
     //      columns n0 + wp + 32 j + 8 g + 4 (lane >> 5) + {0..3}

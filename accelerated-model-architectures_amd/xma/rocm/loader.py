@@ -29,7 +29,8 @@ _p, _i64, _i32, _int, _sz = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int32, cty
 SIGNATURES = {
     "xma_rocm_abi_version": (_int, []),
     "xma_rocm_last_error": (ctypes.c_char_p, []),
-    "xma_rocm_continuous_count": (_int, [_p, _int, _i64, _p, _i32, _p]),
+    "xma_rocm_continuous_count_workspace_bytes": (_sz, [_i64, _i32]),
+    "xma_rocm_continuous_count": (_int, [_p, _int, _i64, _p, _i32, _p, _sz, _p]),
     "xma_rocm_route_workspace_bytes": (_sz, [_i64, _i32]),
     "xma_rocm_route": (_int, [_p, _int, _i64, _i32, _p, _p, _p, _p, _p, _p, _sz, _p]),
     "xma_rocm_scatter2scatter": (

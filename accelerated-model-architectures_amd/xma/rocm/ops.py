@@ -54,15 +54,25 @@ def _weight_layout(W: torch.Tensor) -> tuple[int, int, int]:
 
 
 # --------------------------------------------------------------------------- a1
-@torch.library.custom_op("xma_rocm::continuous_count", mutates_args={"y"})
-def continuous_count_rocm(x: torch.Tensor, y: torch.Tensor) -> None:
+def continuous_count_workspace_elements(n: int, bins: int) -> int:
+    return (get_library().xma_rocm_continuous_count_workspace_bytes(n, bins) + 3) // 4
+
+
+@torch.library.custom_op("xma_rocm::continuous_count", mutates_args={"y", "workspace"})
+def continuous_count_rocm(x: torch.Tensor, y: torch.Tensor, workspace: torch.Tensor | None) -> None:
     """y (uint32, zero-filled by the caller) += histogram of x
-    (reference op: _continuous_count_cuda, continuous_count/cuda_implementation.py:171-197)."""
+    (reference op: _continuous_count_cuda, continuous_count/cuda_implementation.py:171-197).  `workspace` (int32, from
+    continuous_count_workspace_elements) lets large inputs take the two-pass path."""
     assert x.is_cuda and y.is_cuda and x.dim() == 1 and x.is_contiguous() and y.is_contiguous()
     assert x.dtype in (torch.int32, torch.int64) and y.dtype == torch.uint32
+    if workspace is not None:
+        assert workspace.dtype == torch.int32 and workspace.is_contiguous() and workspace.is_cuda
     lib = get_library()
     check(
-        lib.xma_rocm_continuous_count(_ptr(x), int(x.dtype == torch.int64), x.numel(), _ptr(y), y.numel(), _stream(x)),
+        lib.xma_rocm_continuous_count(
+            _ptr(x), int(x.dtype == torch.int64), x.numel(), _ptr(y), y.numel(), _ptr(workspace),
+            0 if workspace is None else workspace.numel() * 4, _stream(x),
+        ),
         "xma_rocm_continuous_count",
     )
 

@@ -259,13 +259,14 @@ def run_routing(args):
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
     y = torch.zeros(E, dtype=torch.uint32, device="cuda")
+    hws = torch.empty(ops.continuous_count_workspace_elements(n, E), dtype=torch.int32, device="cuda")
 
     def hist():
         it[0] += 1
-        ops.continuous_count_rocm(bufs[it[0] % nbuf], y)
+        ops.continuous_count_rocm(bufs[it[0] % nbuf], y, hws)
 
     hist_ms = _time_gpu(hist, args.kernel_iters * 10, warmup=5)
-    hist_warm_ms = _time_gpu(lambda: ops.continuous_count_rocm(bufs[0], y), args.kernel_iters * 10, warmup=5)
+    hist_warm_ms = _time_gpu(lambda: ops.continuous_count_rocm(bufs[0], y, hws), args.kernel_iters * 10, warmup=5)
     route_ms = _time_gpu(step, args.kernel_iters * 5, warmup=5)
     hist_bytes = n * 4 + E * 4
     route_bytes = n * 4 + n * 8 + n * 4 + E * 20

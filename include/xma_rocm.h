@@ -54,12 +54,16 @@ XMA_API const char *xma_rocm_last_error(void);
 /*
  * Histogram of ids in [0, bins): counts[b] += #{i : ids[i] == b}.  ids outside
  * the range are ignored.  Like the reference kernel the result is ACCUMULATED
- * into `counts`, which the caller zero-fills first.
+ * into `counts`, which the caller zero-fills first.  `workspace` may be NULL;
+ * with at least xma_rocm_continuous_count_workspace_bytes(n, bins) bytes large
+ * inputs take a two-pass path (per-workgroup partial histograms, then one
+ * reduction) instead of thousands of same-address device atomics.
  * Replaces _continuous_count_cuda, xma/functional/continuous_count/cuda_implementation.py:171-197
  * (called from xma/functional/continuous_count/__init__.py:43-45).
  */
+XMA_API size_t xma_rocm_continuous_count_workspace_bytes(int64_t n, int32_t bins);
 XMA_API int xma_rocm_continuous_count(const void *ids, int ids_are_int64, int64_t n, uint32_t *counts, int32_t bins,
-                              void *stream);
+                                      void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * Routing in one op: counts, inclusive/exclusive expert offsets and the STABLE

@@ -24,14 +24,16 @@ def test_library_exports_every_declared_symbol():
     assert os.path.isfile(LIBRARY_PATH), "build the library first: python __graft_entry__.py"
     lib = ctypes.CDLL(LIBRARY_PATH)
     declared = _declared_symbols()
-    assert len(declared) >= 12
+    assert len(declared) >= 13
     for name in declared:
         assert hasattr(lib, name), f"{name} declared in include/xma_rocm.h but not exported"
     assert sorted(SIGNATURES) == declared  # the ctypes table covers exactly the header
     lib = get_library()
     assert lib.xma_rocm_abi_version() == 1
     # host-only entry points (no GPU work)
-    assert lib.xma_rocm_route_workspace_bytes(4 * 1024 * 1024, 64) == (4 * 1024 * 1024 // 2048) * 64 * 4
+    assert lib.xma_rocm_route_workspace_bytes(4 * 1024 * 1024, 64) == (4 * 1024 * 1024 // 4096) * 64 * 4
+    assert lib.xma_rocm_continuous_count_workspace_bytes(4 * 1024 * 1024, 64) == 256 * 64 * 4
+    assert lib.xma_rocm_continuous_count_workspace_bytes(1000, 64) == 0
     assert lib.xma_rocm_route_workspace_bytes(0, 8) == 8 * 4
     assert lib.xma_rocm_route_workspace_bytes(-1, 8) == 0
 
@@ -41,7 +43,7 @@ def test_argument_errors_are_reported_before_any_launch():
 
     lib = get_library()
     # bins < 1, E out of range, unsupported dtype, misaligned sizes: all rejected on the host
-    assert lib.xma_rocm_continuous_count(None, 0, 10, None, 0, None) == -1
+    assert lib.xma_rocm_continuous_count(None, 0, 10, None, 0, None, 0, None) == -1
     assert b"continuous_count" in lib.xma_rocm_last_error()
     assert lib.xma_rocm_route(None, 0, 10, 100000, None, None, None, None, None, None, 0, None) == -1
     assert lib.xma_rocm_combine(None, 8, None, None, 8, 4, 2, 12, 0, None) == -1  # H % 8 != 0
@@ -51,7 +53,7 @@ def test_argument_errors_are_reported_before_any_launch():
     assert rc == -2 and b"multiples of 8" in lib.xma_rocm_last_error()
     # empty problems are accepted without touching a pointer
     assert lib.xma_rocm_combine(None, 8, None, None, 8, 0, 2, 16, 0, None) == 0
-    assert lib.xma_rocm_continuous_count(None, 0, 0, ctypes.c_void_p(16), 4, None) == 0
+    assert lib.xma_rocm_continuous_count(None, 0, 0, ctypes.c_void_p(16), 4, None, 0, None) == 0
 
 
 def test_backend_selection_and_errors():
