@@ -445,12 +445,11 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
 // ------------------------------------------------------------------------------------------------
 // dW kernel: DW[e][o][i] = sum_n DY[n][o] X[n][i]; both operands are token-major = transposed sources; the K loop
 // runs over the expert's row range, k-rows past its end come from the zero page.
-//   GATHER = 0: both operands in grouped order (row n of the expert range)
-//   GATHER = 1: rows taken through sorted_scattered_idxs; the indices of step kt + 5 are loaded in iteration kt, so
-//               that two younger steps of loads may stay in flight when they are consumed
+//   GQ / GP = 1: the rows of dY / X are taken through sorted_scattered_idxs (index / fan_out); 0: grouped order
 // ------------------------------------------------------------------------------------------------
-template <typename T, int GATHER>
+template <typename T, int GQ, int GP>
 __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const DwArgs a) {
+    constexpr int GATHER = GQ | GP;
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     u32x4 *tiles = (u32x4 *)smem;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -513,12 +512,12 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
         u32x4 *dst = tiles + (kt & 1) * STAGE_CHUNKS + (piece >> 3) * OP_CHUNKS + j * 64 + wave * 512;
         const uint16_t *src;
         if constexpr (piece < 8) {
-            if (GATHER && !a.dy_grouped)
+            if (GQ)
                 src = a.DY + (int64_t)fastdiv(idx_next[j], a.dy_div) * a.lddy + q_col[j];
             else
                 src = q_grp[j] + (int64_t)kt * BK * a.lddy;
         } else {
-            if (GATHER && !a.x_grouped)
+            if (GP)
                 src = a.X + (int64_t)fastdiv(idx_next[j], a.x_div) * a.ldx + p_col[j];
             else
                 src = p_grp[j] + (int64_t)kt * BK * a.ldx;
@@ -611,11 +610,16 @@ template <typename T, int WT, int EPI> int launch_fwd(const FwdArgs &a, int grid
     return xma_check_launch("grouped_gemm_kernel");
 }
 
-template <typename T, int GATHER> int launch_dw(const DwArgs &a, int grid, hipStream_t st) {
-    int rc = gemm_set_smem(grouped_gemm_dw_kernel<T, GATHER>, GEMM_SMEM_BYTES);
+template <typename T, int GQ, int GP> int launch_dw(const DwArgs &a, int grid, hipStream_t st) {
+    int rc = gemm_set_smem(grouped_gemm_dw_kernel<T, GQ, GP>, GEMM_SMEM_BYTES);
     if (rc) return rc;
-    grouped_gemm_dw_kernel<T, GATHER><<<grid, GEMM_THREADS, GEMM_SMEM_BYTES, st>>>(a);
+    grouped_gemm_dw_kernel<T, GQ, GP><<<grid, GEMM_THREADS, GEMM_SMEM_BYTES, st>>>(a);
     return xma_check_launch("grouped_gemm_dw_kernel");
+}
+
+template <typename T> int dispatch_dw(const DwArgs &a, int grid, hipStream_t st) {
+    if (a.dy_grouped) return a.x_grouped ? launch_dw<T, 0, 0>(a, grid, st) : launch_dw<T, 0, 1>(a, grid, st);
+    return a.x_grouped ? launch_dw<T, 1, 0>(a, grid, st) : launch_dw<T, 1, 1>(a, grid, st);
 }
 
 template <typename T> int dispatch_fwd(const FwdArgs &a, int wt, int epi, int grid, hipStream_t st) {
@@ -734,8 +738,6 @@ extern "C" int xma_rocm_group_bwd_W(const void *DY, int64_t lddy, int dy_grouped
     a.dy_div = make_fastdiv((uint32_t)dy_fan_out);
     a.x_div = make_fastdiv((uint32_t)x_fan_out);
     if (dy_scale) return launch_dw_scaled(a, dtype, (int)grid, st);
-    const bool gather = !dy_grouped || !x_grouped;
-    if (dtype == XMA_ROCM_BF16)
-        return gather ? launch_dw<__bf16, 1>(a, (int)grid, st) : launch_dw<__bf16, 0>(a, (int)grid, st);
-    return gather ? launch_dw<_Float16, 1>(a, (int)grid, st) : launch_dw<_Float16, 0>(a, (int)grid, st);
+    if (dtype == XMA_ROCM_BF16) return dispatch_dw<__bf16>(a, (int)grid, st);
+    return dispatch_dw<_Float16>(a, (int)grid, st);
 }

@@ -111,9 +111,10 @@ __global__ __launch_bounds__(HIST_THREADS) void histogram_global_kernel(const Id
 // route: a unit is the ROUTE_CHUNK consecutive ids of one workgroup (4 waves x 1024).
 //   pass 1  unit_hist[u][e]               (LDS atomics)
 //   pass 2  block e: exclusive prefix over units of column e (in place) and counts[e]
-//   pass 3  per unit: per-wave counts -> local offsets; stable rank of every id inside its wave (64 ids per step:
-//           peers = lanes with the same id through log2(E) ballots, rank = popcount(peers below), running counter in
-//           wave-private LDS); the unit is sorted into LDS and leaves as one contiguous run per expert.
+//   pass 3  per unit: per-wave counts -> local offsets; stable rank of every id inside its wave (64 ids per step,
+//           returning LDS atomic adds on wave-private counters, which serve equal addresses of one instruction in lane
+//           order; XMA_ROUTE_BALLOT_RANKS selects ranks from log2(E) ballots instead); the unit is sorted into LDS
+//           and leaves as one contiguous run per expert.
 // ------------------------------------------------------------------------------------------------
 constexpr int ROUTE_THREADS = 256;
 constexpr int ROUTE_WAVES = ROUTE_THREADS / WAVE;

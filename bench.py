@@ -312,12 +312,24 @@ def run_routing(args):
     print(json.dumps(out))
 
 
+def run_copy(args):
+    """counter calibration: a plain device copy of known size (1 GiB read + 1 GiB written per launch), the kernel
+    that FETCH_SIZE / WRITE_SIZE readings of the other workloads are scaled by"""
+    nbytes = 1 << 30
+    src = torch.empty(nbytes, dtype=torch.uint8, device="cuda").fill_(1)
+    dst = torch.empty_like(src)
+    ms = _time_gpu(lambda: dst.copy_(src), args.steps, warmup=args.warmup)
+    print(json.dumps({"metric": "copy_gb_per_s", "value": round(2 * nbytes / ms / 1e6, 1), "unit": "GB/s", "n_gpus": 1,
+                      "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+                      "config": {"workload": f"copy: torch copy_ of {nbytes} bytes (reads {nbytes}, writes {nbytes} per launch)"}}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5"])
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "copy"])
     ap.add_argument("--zipf", action="store_true", help="c2 only: Zipf(s=1.1) ids instead of uniform")
     ap.add_argument("--kernel-iters", type=int, default=5)
     ap.add_argument("--cpu-fraction", type=int, default=8, help="CPU baseline runs on T / this many tokens")
@@ -330,7 +342,9 @@ def main():
     from xma.rocm import get_library
 
     get_library()
-    if args.workload == "c2":
+    if args.workload == "copy":
+        run_copy(args)
+    elif args.workload == "c2":
         run_routing(args)
     else:
         run_moe(args, WORKLOADS[args.workload], args.workload)
