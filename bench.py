@@ -41,6 +41,15 @@ WORKLOADS = {
 }
 
 
+# HBM bytes per launch of each workload's dominant kernel, from two counter runs (FETCH_SIZE scaled by 2.0, WRITE_SIZE by
+# 1.0: the factors a 1 GiB device copy, `--workload copy`, gives for the same counters).  bench.py cannot read hardware
+# counters itself; the figures are re-measured with rocprofv3 whenever the kernel changes.
+MEASURED_TRAFFIC_BYTES = {
+    "c3": 11.83e9,  # up-projection + SwiGLU GEMM: 10.13 GB fetched + 1.70 GB written (3.42 GB algorithmic)
+    "c2": 70.9e6,  # route_scatter_kernel: 17.1 MB fetched + 53.8 MB written
+}
+
+
 def _time_gpu(fn, iters: int, warmup: int = 2) -> float:
     """average milliseconds per call, events on the current (launch) stream"""
     for _ in range(warmup):
@@ -173,7 +182,7 @@ def run_moe(args, cfg, name):
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(gemms[dom]["tflops"] / PEAK_BF16_TFLOPS, 4),
-        "traffic": None,
+        "traffic": MEASURED_TRAFFIC_BYTES.get(name) if dom.startswith("up_swiglu") else None,
         "all_gemms_tflops": round(total_flops / total_ms / 1e9, 1),
         "all_gemms_frac": round(total_flops / total_ms / 1e9 / PEAK_BF16_TFLOPS, 4),
     }
@@ -297,7 +306,7 @@ def run_routing(args):
             "peak": PEAK_HBM_GBS,
             "unit": "GB/s",
             "frac": round(route_bytes / route_ms / 1e6 / PEAK_HBM_GBS, 4),
-            "traffic": None,
+            "traffic": None if args.zipf else MEASURED_TRAFFIC_BYTES["c2"] + 17.1e6 + 4.2e6,  # scatter + unit hist + scan
         },
         "cpu_baseline": {"value": round(n / dt, 1), "unit": "ids/s", "cores": 1, "kind": "port",
                          "sample": f"numpy stable argsort + bincount + cumsum of the same {n} ids, mean of {reps}"},
