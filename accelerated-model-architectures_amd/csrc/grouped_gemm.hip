@@ -152,25 +152,24 @@ __device__ __forceinline__ void load_frags(Frags &f, const FragBase<PTR> &pb, co
     });
 }
 
-// The 16 MFMAs of one k16 sub-step on `cur` as 8 pinned slots.  Slot g: two MFMAs; for g < 4 one P and one Q fragment
+// The 16 MFMAs of one k16 sub-step on `cur` as 8 pinned slots (NI < 4: only the first NI of the wave's four 32-wide Q
+// blocks hold valid rows; the MFMAs and fragment reads of the others are left out).  Slot g: two MFMAs; for g < 4 one P and one Q fragment
 // read of sub-step KK (of the stage pb/qb point at) into `nxt`; then `hook(IC<g>)`, which the callers use to issue one
 // LDS-DMA load per slot.  A wave issues in order, so anything not placed between MFMAs would leave the matrix pipe idle
 // for as long as it takes to issue; all fragment reads sit in the first half so that the second half covers their
 // latency.
-template <typename T, int PTR, int QTR, int KK, typename Hook>
+template <typename T, int PTR, int QTR, int KK, int NI = 4, typename Hook>
 __device__ __forceinline__ void mma_step(Frags &cur, Frags &nxt, const FragBase<PTR> &pb, const FragBase<QTR> &qb,
                                          f32x16 (&acc)[4][4], Hook hook) {
     wait_frags(cur); // issued at least 8 MFMAs ago
     static_for<8>([&](auto G) {
         constexpr int g = G.value, j = g >> 1, i0 = (g & 1) * 2;
         __builtin_amdgcn_sched_barrier(0);
-        acc[j][i0] = Elem<T>::mfma(cur.p[j], cur.q[i0], acc[j][i0]);
-        acc[j][i0 + 1] = Elem<T>::mfma(cur.p[j], cur.q[i0 + 1], acc[j][i0 + 1]);
+        if constexpr (i0 < NI) acc[j][i0] = Elem<T>::mfma(cur.p[j], cur.q[i0], acc[j][i0]);
+        if constexpr (i0 + 1 < NI) acc[j][i0 + 1] = Elem<T>::mfma(cur.p[j], cur.q[i0 + 1], acc[j][i0 + 1]);
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (g < 4) {
-            nxt.p[g] = read_frag<PTR, g, KK>(pb);
-            nxt.q[g] = read_frag<QTR, g, KK>(qb);
-        }
+        if constexpr (g < 4 && NI > 0) nxt.p[g] = read_frag<PTR, g, KK>(pb);
+        if constexpr (g < NI) nxt.q[g] = read_frag<QTR, g, KK>(qb);
         hook(G);
     });
     __builtin_amdgcn_sched_barrier(0);
@@ -248,19 +247,10 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
     const int64_t row_lo = e ? a.offs[e - 1] : 0, row_hi = a.offs[e];
     const int tiles_m = (int)((row_hi - row_lo + BM - 1) / BM);
     const int m_tile = s_sched[1] % tiles_m, n_tile = s_sched[1] / tiles_m;
-#ifdef XMA_EXP_SAME_TILE
-    const int64_t row0 = row_lo;
-#else
     const int64_t row0 = row_lo + (int64_t)m_tile * BM;
-#endif
     const int rows_valid = (int)((row_hi - row0 < BM) ? row_hi - row0 : BM);
-#ifdef XMA_EXP_SAME_TILE
-    const int n0 = 0;
-#else
     const int n0 = n_tile * BN;
-#endif
     __syncthreads(); // s_pre is dead from here on
-
 
     // ---- loader set-up: one fixed per-lane global pointer per LDS-DMA piece (k = 0); a step adds a uniform offset
     const uint16_t *zero = (const uint16_t *)g_zero_page;
@@ -338,56 +328,44 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
         asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
     else
         asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-    Frags f0, f1;
-    load_frags<WT, 0, 0>(f0, pb, qb);
-    // one K step; FULL: steps kt + 1 and kt + 2 exist and are complete
-#ifdef XMA_EXP_TIMING2
-    uint64_t acc_t[5] = {0, 0, 0, 0, 0};
-#endif
-    auto k_step = [&](int kt, auto FULL) {
-#ifdef XMA_EXP_TIMING2
-        const uint64_t ta = wall_clock64();
-#endif
-        // second half of the loads of step kt + 1 (the first half went out behind the previous barrier)
-        mma_step<T, WT, 0, 1>(f0, f1, pb, qb, acc, [&](auto G) { issue_piece(kt + 1, IC<8 + G.value>{}, FULL); });
-#ifdef XMA_EXP_TIMING2
-        const uint64_t tb = wall_clock64();
-#endif
-        mma_step<T, WT, 0, 2>(f1, f0, pb, qb, acc, NoHook());
-        mma_step<T, WT, 0, 3>(f0, f1, pb, qb, acc, NoHook());
-#ifdef XMA_EXP_TIMING2
-        const uint64_t tc = wall_clock64();
-        asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
-        const uint64_t td = wall_clock64();
-#endif
-        XMA_WAIT_LOADS_AND_BARRIER(); // step kt + 1 has landed; nobody reads this stage any more
-#ifdef XMA_EXP_TIMING2
-        const uint64_t te = wall_clock64();
-#endif
-        flip_stage(pb);
-        flip_stage(qb);
-        // the stage just left is free: first half of the loads of step kt + 2; fragments of sub-step 0 of step kt + 1
-        mma_step<T, WT, 0, 0>(f1, f0, pb, qb, acc, [&](auto G) { issue_piece(kt + 2, G, FULL); });
-#ifdef XMA_EXP_TIMING2
-        const uint64_t tf = wall_clock64();
-        acc_t[0] += tb - ta;
-        acc_t[1] += tc - tb;
-        acc_t[2] += td - tc;
-        acc_t[3] += te - td;
-        acc_t[4] += tf - te;
-#endif
-    };
+    // Q blocks (32 rows) of this wave that hold valid rows: 4 except in an expert's last row tile.  A wave with fewer
+    // skips the MFMAs and fragment reads of the empty blocks (rounded up to 0, 1, 2 or 4 blocks); it still issues its
+    // share of the loads and meets every barrier.
+    const int q_blocks = (rows_valid > wq) ? (rows_valid - wq + 31) >> 5 : 0;
     const int KT_full = a.K / BK; // steps without a chunk past K
-    int kt = 0;
-    for (; kt + 2 < KT_full; ++kt) k_step(kt, IC<1>{});
-    for (; kt < KT; ++kt) k_step(kt, IC<0>{});
+    auto main_loop = [&](auto NI_) {
+        constexpr int NI = NI_.value;
+        Frags f0, f1;
+        if constexpr (NI > 0) {
+            static_for<4>([&](auto I) { f0.p[I.value] = read_frag<WT, I.value, 0>(pb); });
+            static_for<NI>([&](auto I) { f0.q[I.value] = read_frag<0, I.value, 0>(qb); });
+        }
+        // one K step; FULL: steps kt + 1 and kt + 2 exist and are complete
+        auto k_step = [&](int kt, auto FULL) {
+            // second half of the loads of step kt + 1 (the first half went out behind the previous barrier)
+            mma_step<T, WT, 0, 1, NI>(f0, f1, pb, qb, acc, [&](auto G) { issue_piece(kt + 1, IC<8 + G.value>{}, FULL); });
+            mma_step<T, WT, 0, 2, NI>(f1, f0, pb, qb, acc, NoHook());
+            mma_step<T, WT, 0, 3, NI>(f0, f1, pb, qb, acc, NoHook());
+            XMA_WAIT_LOADS_AND_BARRIER(); // step kt + 1 has landed; nobody reads this stage any more
+            flip_stage(pb);
+            flip_stage(qb);
+            // the stage just left is free: first half of the loads of step kt + 2; fragments of sub-step 0 of step kt + 1
+            mma_step<T, WT, 0, 0, NI>(f1, f0, pb, qb, acc, [&](auto G) { issue_piece(kt + 2, G, FULL); });
+        };
+        int kt = 0;
+        if constexpr (NI == 4)
+            for (; kt + 2 < KT_full; ++kt) k_step(kt, IC<1>{});
+        for (; kt < KT; ++kt) k_step(kt, IC<0>{});
+    };
+    if (q_blocks > 2)
+        main_loop(IC<4>{});
+    else if (q_blocks == 2)
+        main_loop(IC<2>{});
+    else if (q_blocks == 1)
+        main_loop(IC<1>{});
+    else
+        main_loop(IC<0>{});
     XMA_WAIT_ALL_LOADS();
-#ifdef XMA_EXP_TIMING2
-    if (EPI == XMA_ROCM_EPI_STORE && a.aux && lane == 0) {
-        uint64_t *dbg = (uint64_t *)a.aux + ((size_t)blockIdx.x * 4 + wave) * 8;
-        for (int q = 0; q < 5; ++q) dbg[q] = acc_t[q];
-    }
-#endif
 
     // ---- epilogue: lane owns row (lane & 31) of each 32-row block; quad g of tile (j, i) holds
     //      columns n0 + wp + 32 j + 8 g + 4 (lane >> 5) + {0..3}
