@@ -92,4 +92,5 @@ __device__ __forceinline__ void transpose8x8_b16(const u32x4 in[8], u32x4 out[8]
     }
 }
 
-__device__ __forceinline__ float sigmoidf_fast(float x) { return 1.0f / (1.0f + __expf(-x)); }
+// v_exp_f32 and v_rcp_f32 (1 ulp each) instead of an IEEE division: the result is rounded to 16 bits anyway
+__device__ __forceinline__ float sigmoidf_fast(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }

@@ -36,6 +36,15 @@
 namespace xma_rocm {
 
 constexpr int BK = 64, NSTAGE = 2;
+// The 16 LDS-DMA pieces of a K step are issued one per MFMA slot: DMA_N0 in the sub-step right behind the barrier that
+// frees their stage, DMA_N1 and DMA_N2 in the two sub-steps after it.
+#ifndef XMA_DMA_N0
+#define XMA_DMA_N0 8
+#define XMA_DMA_N1 8
+#define XMA_DMA_N2 0
+#endif
+constexpr int DMA_N0 = XMA_DMA_N0, DMA_N1 = XMA_DMA_N1, DMA_N2 = XMA_DMA_N2;
+static_assert(DMA_N0 + DMA_N1 + DMA_N2 == 16 && DMA_N0 <= 16 && DMA_N1 <= 8 && DMA_N2 <= 8, "piece schedule");
 constexpr int OP_CHUNKS = 256 * 8;                          // 16-byte chunks per operand tile (32 KB)
 constexpr int STAGE_CHUNKS = 2 * OP_CHUNKS;                 // Q tile then P tile
 constexpr int GEMM_SMEM_BYTES = NSTAGE * STAGE_CHUNKS * 16; // 128 KB
@@ -188,6 +197,20 @@ __device__ __forceinline__ uint32_t lds_addr_of(const void *p) {
 #define XMA_WAIT_LOADS_AND_BARRIER() asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_barrier" ::: "memory")
 #define XMA_WAIT_ALL_LOADS() asm volatile("s_waitcnt vmcnt(0)" ::: "memory")
 
+// Epilogue staging in LDS, private to a wave: one 32-row block of its 128 x 128 corner as 16-bit values (rows padded
+// by 16 bytes against bank conflicts), followed by the 32 x 64 block of SwiGLU activations.
+constexpr int EPI_Z_STRIDE = 128 * 2 + 16, EPI_H_STRIDE = 64 * 2 + 16;
+constexpr int EPI_WAVE_BYTES = 32 * EPI_Z_STRIDE + 32 * EPI_H_STRIDE;
+static_assert(4 * EPI_WAVE_BYTES <= GEMM_SMEM_BYTES, "epilogue staging must fit into the operand stages");
+
+// LDS written by some lanes of a wave is read by others of the same wave: instructions of one wave reach the LDS in
+// order, so only the compiler has to be kept from reordering.
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
 template <int N> __device__ __forceinline__ void zero_acc(f32x16 (&acc)[N][N]) {
 #pragma unroll
     for (int j = 0; j < N; ++j)
@@ -206,6 +229,9 @@ template <typename T, int WT, int EPI>
 __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const FwdArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     __shared__ int s_sched[4];
+#ifdef XMA_EXP_TIMING3
+    const uint64_t t3_start = wall_clock64();
+#endif
     u32x4 *tiles = (u32x4 *)smem;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -322,10 +348,10 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
     make_frag_base<WT>(pb, lds0 + OP_CHUNKS * 16, wp, lane);
 
     static_for<16>([&](auto P) { issue_piece(0, P, IC<0>{}); });
-    static_for<8>([&](auto P) { issue_piece(1, P, IC<0>{}); });
-    // step 0 has landed in every wave (the first half of step 1 may be in flight)
+    static_for<DMA_N0>([&](auto P) { issue_piece(1, P, IC<0>{}); });
+    // step 0 has landed in every wave (the first loads of step 1 may be in flight)
     if (KT > 1)
-        asm volatile("s_waitcnt vmcnt(8)\n\ts_barrier" ::: "memory");
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(DMA_N0) : "memory");
     else
         asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
     // Q blocks (32 rows) of this wave that hold valid rows: 4 except in an expert's last row tile.  A wave with fewer
@@ -333,6 +359,9 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
     // share of the loads and meets every barrier.
     const int q_blocks = (rows_valid > wq) ? (rows_valid - wq + 31) >> 5 : 0;
     const int KT_full = a.K / BK; // steps without a chunk past K
+#ifdef XMA_EXP_TIMING3
+    const uint64_t t3_loop = wall_clock64();
+#endif
     auto main_loop = [&](auto NI_) {
         constexpr int NI = NI_.value;
         Frags f0, f1;
@@ -342,15 +371,22 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
         }
         // one K step; FULL: steps kt + 1 and kt + 2 exist and are complete
         auto k_step = [&](int kt, auto FULL) {
-            // second half of the loads of step kt + 1 (the first half went out behind the previous barrier)
-            mma_step<T, WT, 0, 1, NI>(f0, f1, pb, qb, acc, [&](auto G) { issue_piece(kt + 1, IC<8 + G.value>{}, FULL); });
-            mma_step<T, WT, 0, 2, NI>(f1, f0, pb, qb, acc, NoHook());
+            // rest of the loads of step kt + 1 (the first DMA_N0 went out behind the previous barrier)
+            mma_step<T, WT, 0, 1, NI>(f0, f1, pb, qb, acc, [&](auto G) {
+                if constexpr (G.value < DMA_N1) issue_piece(kt + 1, IC<DMA_N0 + G.value>{}, FULL);
+            });
+            mma_step<T, WT, 0, 2, NI>(f1, f0, pb, qb, acc, [&](auto G) {
+                if constexpr (G.value < DMA_N2) issue_piece(kt + 1, IC<DMA_N0 + DMA_N1 + G.value>{}, FULL);
+            });
             mma_step<T, WT, 0, 3, NI>(f0, f1, pb, qb, acc, NoHook());
             XMA_WAIT_LOADS_AND_BARRIER(); // step kt + 1 has landed; nobody reads this stage any more
             flip_stage(pb);
             flip_stage(qb);
-            // the stage just left is free: first half of the loads of step kt + 2; fragments of sub-step 0 of step kt + 1
-            mma_step<T, WT, 0, 0, NI>(f1, f0, pb, qb, acc, [&](auto G) { issue_piece(kt + 2, G, FULL); });
+            // the stage just left is free: first loads of step kt + 2; fragments of sub-step 0 of step kt + 1
+            mma_step<T, WT, 0, 0, NI>(f1, f0, pb, qb, acc, [&](auto G) {
+                if constexpr (G.value < DMA_N0) issue_piece(kt + 2, G, FULL);
+                if constexpr (G.value + 8 < DMA_N0) issue_piece(kt + 2, IC<G.value + 8>{}, FULL);
+            });
         };
         int kt = 0;
         if constexpr (NI == 4)
@@ -365,59 +401,146 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
         main_loop(IC<1>{});
     else
         main_loop(IC<0>{});
-    XMA_WAIT_ALL_LOADS();
+    // every load has landed, every fragment read has returned (the last sub-step reads ahead into registers nobody
+    // uses), and no wave touches the operand tiles any more: LDS becomes the staging area of the epilogue
+    XMA_WAIT_LOADS_AND_BARRIER();
+#ifdef XMA_EXP_TIMING3
+    const uint64_t t3_epi = wall_clock64();
+#endif
 
     // ---- epilogue: lane owns row (lane & 31) of each 32-row block; quad g of tile (j, i) holds
     //      columns n0 + wp + 32 j + 8 g + 4 (lane >> 5) + {0..3}
     const int lrow = lane & 31, lhalf = lane >> 5;
+    if constexpr (EPI != XMA_ROCM_EPI_SWIGLU_BWD) {
+        // A store instruction of the accumulator layout would touch 32 rows with 16 bytes each.  Instead every
+        // 32-row block goes through a wave-private LDS area and leaves as whole rows: 16 lanes x 16 bytes per row of
+        // 128 columns (8 lanes per row of the 64 activation columns), i.e. full 128-byte lines.
+        unsigned char *stage = smem + wave * EPI_WAVE_BYTES;
+        unsigned char *z_w = stage + lrow * EPI_Z_STRIDE + lhalf * 8;
+        unsigned char *h_w = stage + 32 * EPI_Z_STRIDE + lrow * EPI_H_STRIDE + lhalf * 4;
+        const unsigned char *z_r = stage + (lane >> 4) * EPI_Z_STRIDE + (lane & 15) * 16;
+        const unsigned char *h_r = stage + 32 * EPI_Z_STRIDE + (lane >> 3) * EPI_H_STRIDE + (lane & 7) * 16;
+        const int cz = n0 + wp + (lane & 15) * 8;        // this lane's 8 output columns on the way out
+        const int ch = ((n0 + wp) >> 1) + (lane & 7) * 8; // and its 8 activation columns
+        const bool write_z = (EPI == XMA_ROCM_EPI_STORE) || a.out != nullptr;
+        // destination row and scale of this lane's row in each of the four blocks, fetched before the first store:
+        // loads and stores retire in order, so a load between the blocks would wait for the stores before it
+        int dst_i[4];
+        float sc_i[4];
+        const bool need_idx = !a.y_grouped || a.scale != nullptr;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int r = wq + i * 32 + lrow;
-        if (r >= rows_valid) continue;
-        const int64_t n = row0 + r;
-        int64_t sidx = 0;
-        if (!a.y_grouped || a.scale) sidx = a.idx[n];
-        const int64_t dst = a.y_grouped ? n : sidx;
-        float sc = 1.f;
-        if (a.scale) sc = Elem<T>::lo((uint32_t)a.scale[sidx]);
+        for (int i = 0; i < 4; ++i) {
+            int r = wq + i * 32 + lrow;
+            if (r >= rows_valid) r = rows_valid - 1; // duplicates are computed and never stored
+            const int64_t n = row0 + r;
+            dst_i[i] = need_idx ? (int)a.idx[n] : (int)n;
+        }
+        if (a.scale) {
+            uint16_t raw[4];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+            for (int i = 0; i < 4; ++i) raw[i] = a.scale[dst_i[i]];
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int col = n0 + wp + j * 32 + g * 8 + lhalf * 4;
-                if (col >= a.N) continue;
-                const float v0 = acc[j][i][4 * g] * sc, v1 = acc[j][i][4 * g + 1] * sc;
-                const float v2 = acc[j][i][4 * g + 2] * sc, v3 = acc[j][i][4 * g + 3] * sc;
-                if (EPI == XMA_ROCM_EPI_STORE) {
-                    u32x2 o = {Elem<T>::pack(v0, v1), Elem<T>::pack(v2, v3)};
-                    *(u32x2 *)(a.out + dst * a.ldo + col) = o;
-                } else if (EPI == XMA_ROCM_EPI_SWIGLU) {
-                    // columns are (gate, up, gate, up); the activation is taken from the rounded
-                    // pre-activations, exactly what a separate pass over the stored z would see
+            for (int i = 0; i < 4; ++i) sc_i[i] = Elem<T>::lo((uint32_t)raw[i]);
+        } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sc_i[i] = 1.f;
+        }
+        if (a.y_grouped) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                int r = wq + i * 32 + lrow;
+                if (r >= rows_valid) r = rows_valid - 1;
+                dst_i[i] = (int)(row0 + r);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (wq + i * 32 >= rows_valid) break; // wave-uniform
+            const int dst = dst_i[i];
+            const float sc = sc_i[i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const float v0 = acc[j][i][4 * g] * sc, v1 = acc[j][i][4 * g + 1] * sc;
+                    const float v2 = acc[j][i][4 * g + 2] * sc, v3 = acc[j][i][4 * g + 3] * sc;
                     const uint32_t z0 = Elem<T>::pack(v0, v1), z1 = Elem<T>::pack(v2, v3);
-                    if (a.out) {
-                        u32x2 o = {z0, z1};
-                        *(u32x2 *)(a.out + dst * a.ldo + col) = o;
+                    u32x2 o = {z0, z1};
+                    *(u32x2 *)(z_w + (j * 32 + g * 8) * 2) = o;
+                    if constexpr (EPI == XMA_ROCM_EPI_SWIGLU) {
+                        // columns are (gate, up, gate, up); the activation is taken from the rounded
+                        // pre-activations, exactly what a separate pass over the stored z would see
+                        const float g0 = Elem<T>::lo(z0), u0 = Elem<T>::hi(z0);
+                        const float g1 = Elem<T>::lo(z1), u1 = Elem<T>::hi(z1);
+                        const float h0 = u0 * g0 * sigmoidf_fast(g0), h1 = u1 * g1 * sigmoidf_fast(g1);
+                        *(uint32_t *)(h_w + (j * 16 + g * 4) * 2) = Elem<T>::pack(h0, h1);
                     }
-                    const float g0 = Elem<T>::lo(z0), u0 = Elem<T>::hi(z0);
-                    const float g1 = Elem<T>::lo(z1), u1 = Elem<T>::hi(z1);
-                    const float h0 = u0 * g0 * sigmoidf_fast(g0), h1 = u1 * g1 * sigmoidf_fast(g1);
-                    *(uint32_t *)(a.aux + dst * a.ldaux + (col >> 1)) = Elem<T>::pack(h0, h1);
-                } else { // EPI_SWIGLU_BWD: v* = d h for 4 columns; z has 8 columns (g, u) x 4
+                }
+            }
+            wave_lds_sync();
+            const int rbase = wq + i * 32;
+            if (write_z) {
+#pragma unroll
+                for (int it = 0; it < 8; ++it) {
+                    const int rr = 4 * it + (lane >> 4);
+                    const u32x4 v = *(const u32x4 *)(z_r + it * 4 * EPI_Z_STRIDE);
+                    const int d = __shfl(dst, rr);
+                    if (rbase + rr < rows_valid && cz < a.N) *(u32x4 *)(a.out + (int64_t)d * a.ldo + cz) = v;
+                }
+            }
+            if constexpr (EPI == XMA_ROCM_EPI_SWIGLU) {
+#pragma unroll
+                for (int it = 0; it < 4; ++it) {
+                    const int rr = 8 * it + (lane >> 3);
+                    const u32x4 v = *(const u32x4 *)(h_r + it * 8 * EPI_H_STRIDE);
+                    const int d = __shfl(dst, rr);
+                    if (rbase + rr < rows_valid && 2 * ch < a.N) *(u32x4 *)(a.aux + (int64_t)d * a.ldaux + ch) = v;
+                }
+            }
+            wave_lds_sync(); // the next block overwrites the area
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int r = wq + i * 32 + lrow;
+            if (r >= rows_valid) continue;
+            const int64_t n = row0 + r;
+            float sc = 1.f;
+            if (a.scale) sc = Elem<T>::lo((uint32_t)a.scale[a.idx[n]]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int col = n0 + wp + j * 32 + g * 8 + lhalf * 4;
+                    if (col >= a.N) continue;
+                    // acc * scale = d h for 4 columns; z has 8 columns (g, u) x 4
                     const u32x4 z = *(const u32x4 *)(a.aux + n * a.ldaux + 2 * col);
-                    const float dh[4] = {v0, v1, v2, v3};
                     u32x4 o;
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
+                        const float dh = acc[j][i][4 * g + q] * sc;
                         const float gg = Elem<T>::lo(z[q]), uu = Elem<T>::hi(z[q]);
-                        const float s = sigmoidf_fast(gg), silu = gg * s;
-                        o[q] = Elem<T>::pack(dh[q] * uu * (s + silu * (1.f - s)), dh[q] * silu);
+                        const float sg = sigmoidf_fast(gg), silu = gg * sg;
+                        o[q] = Elem<T>::pack(dh * uu * (sg + silu * (1.f - sg)), dh * silu);
                     }
-                    *(u32x4 *)(a.out + dst * a.ldo + 2 * col) = o;
+                    *(u32x4 *)(a.out + n * a.ldo + 2 * col) = o;
                 }
             }
         }
     }
+#ifdef XMA_EXP_TIMING3
+    if (EPI == XMA_ROCM_EPI_STORE && a.aux) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const uint64_t t3_end = wall_clock64();
+        if (tid == 0) {
+            uint32_t hwid, xcc;
+            asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+            asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+            uint64_t *dbg = (uint64_t *)a.aux + (size_t)blockIdx.x * 8;
+            dbg[0] = t3_start, dbg[1] = t3_loop, dbg[2] = t3_epi, dbg[3] = t3_end, dbg[4] = hwid, dbg[5] = xcc, dbg[6] = rows_valid;
+        }
+    }
+#endif
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -561,23 +684,35 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
         XMA_WAIT_ALL_LOADS();
     }
 
-    // lane owns DW row o (from the Q tile), 4 consecutive in-features per quad
+    // lane owns DW row o (from the Q tile), 4 consecutive in-features per quad; each 32-row block is staged in a
+    // wave-private LDS area and leaves as whole rows (see the forward kernel's epilogue)
+    XMA_WAIT_LOADS_AND_BARRIER(); // no wave reads the operand tiles any more
     const int lrow = lane & 31, lhalf = lane >> 5;
     uint16_t *DWe = a.DW + (int64_t)e * a.dw_es;
+    unsigned char *stage = smem + wave * EPI_WAVE_BYTES;
+    unsigned char *z_w = stage + lrow * EPI_Z_STRIDE + lhalf * 8;
+    const unsigned char *z_r = stage + (lane >> 4) * EPI_Z_STRIDE + (lane & 15) * 16;
+    const int cz = i0 + wp + (lane & 15) * 8;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        const int o = o0 + wq + i * 32 + lrow;
-        if (o >= a.N_out) continue;
+        const int obase = o0 + wq + i * 32;
+        if (obase >= a.N_out) break; // wave-uniform
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const int col = i0 + wp + j * 32 + g * 8 + lhalf * 4;
-                if (col >= a.K_in) continue;
                 u32x2 v = {Elem<T>::pack(acc[j][i][4 * g], acc[j][i][4 * g + 1]),
                            Elem<T>::pack(acc[j][i][4 * g + 2], acc[j][i][4 * g + 3])};
-                *(u32x2 *)(DWe + (int64_t)o * a.lddw + col) = v;
+                *(u32x2 *)(z_w + (j * 32 + g * 8) * 2) = v;
             }
+        wave_lds_sync();
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int o = obase + 4 * it + (lane >> 4);
+            const u32x4 v = *(const u32x4 *)(z_r + it * 4 * EPI_Z_STRIDE);
+            if (o < a.N_out && cz < a.K_in) *(u32x4 *)(DWe + (int64_t)o * a.lddw + cz) = v;
+        }
+        wave_lds_sync(); // the next block overwrites the area
     }
 }
 
