@@ -6,7 +6,8 @@
 constexpr int BM = 256, BN = 256; // output tile of every grouped GEMM kernel
 constexpr int GEMM_THREADS = 256;
 
-// exact n / d for 0 <= n < 2^31: q = (n * magic) >> shift with magic = ceil(2^shift / d), shift = 31 + ceil(log2 d)
+// exact n / d for 0 <= n < 2^31 in three 32-bit instructions: with s = ceil(log2 d) and magic = ceil(2^(31+s) / d)
+// (which fits 32 bits), n / d = mulhi(2 n, magic) >> s
 struct FastDiv {
     uint32_t magic;
     int shift;
@@ -15,11 +16,11 @@ inline FastDiv make_fastdiv(uint32_t d) {
     int s = 0;
     while ((1u << s) < d) ++s;
     FastDiv f;
-    f.shift = 31 + s;
-    f.magic = (uint32_t)((((uint64_t)1 << f.shift) + d - 1) / d);
+    f.shift = s;
+    f.magic = (uint32_t)((((uint64_t)1 << (31 + s)) + d - 1) / d);
     return f;
 }
-__device__ __forceinline__ uint32_t fastdiv(uint32_t n, FastDiv f) { return (uint32_t)(((uint64_t)n * f.magic) >> f.shift); }
+__device__ __forceinline__ uint32_t fastdiv(uint32_t n, FastDiv f) { return __umulhi(n << 1, f.magic) >> f.shift; }
 
 struct FwdArgs {
     const uint16_t *X;

@@ -551,6 +551,9 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
 template <typename T, int GQ, int GP>
 __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const DwArgs a) {
     constexpr int GATHER = GQ | GP;
+#ifdef XMA_EXP_TIMING3
+    const uint64_t t3_start = wall_clock64();
+#endif
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     u32x4 *tiles = (u32x4 *)smem;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -578,27 +581,37 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
         q_col[j] = o0 + cq * 8;
         p_col[j] = i0 + cp * 8;
     }
-    const uint16_t *q_grp[8], *p_grp[8]; // grouped-order pointers at step 0
+    // Per-lane byte pointers of the 8 pieces of each operand: for an operand in grouped order the address of step 0
+    // (the row is row_lo + 64 kt + kr, so a step adds a uniform 64 rows); for a gathered operand the column position in
+    // row 0, to which token * row pitch is added (one 32 x 32 -> 64-bit multiply-add per piece).
+    const uint32_t lddy_b = (uint32_t)a.lddy * 2, ldx_b = (uint32_t)a.ldx * 2;
+    const char *q_base[8], *p_base[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
-        q_grp[j] = a.DY + (row_lo + kr_lane + 2 * j) * a.lddy + q_col[j];
-        p_grp[j] = a.X + (row_lo + kr_lane + 2 * j) * a.ldx + p_col[j];
+        q_base[j] = (const char *)(a.DY + q_col[j]) + (GQ ? 0 : (row_lo + kr_lane + 2 * j) * (int64_t)lddy_b);
+        p_base[j] = (const char *)(a.X + p_col[j]) + (GP ? 0 : (row_lo + kr_lane + 2 * j) * (int64_t)ldx_b);
     }
 
     // Scattered indices of this lane's 8 tokens of the step that is loaded next.  They are fetched one step ahead with
     // inline assembly (low dword of the int64 index): the compiler would guard the later use of a loop-carried loaded
     // register with a wait of its own choosing; here the wait is the vmcnt(0) in front of each step's barrier, and
-    // use_idx() ties the registers to a point behind it.
+    // use_idx() ties the registers to a point behind it.  FULL: all rows of the step lie inside the expert, the address
+    // is one per-lane pointer plus an immediate.
     uint32_t idx_next[8];
-    auto load_idx = [&](int kt) {
-#pragma unroll
-        for (int j = 0; j < 8; ++j) {
+    const int64_t *idx_lane = a.idx + row_lo + kr_lane;
+    auto load_idx_one = [&](int kt, auto J, auto FULL) {
+        constexpr int j = J.value;
+        if constexpr (FULL.value) {
+            const int64_t *src = idx_lane + (int64_t)kt * BK;
+            asm volatile("global_load_dword %0, %1, off offset:%2" : "=v"(idx_next[j]) : "v"(src), "n"(16 * j) : "memory");
+        } else {
             int r = kt * BK + kr_lane + 2 * j;
             if (r >= rows) r = rows - 1; // clamped, never predicated
             const int64_t *src = a.idx + row_lo + r;
             asm volatile("global_load_dword %0, %1, off" : "=v"(idx_next[j]) : "v"(src) : "memory");
         }
     };
+    auto load_idx = [&](int kt) { static_for<8>([&](auto J) { load_idx_one(kt, J, IC<0>{}); }); };
     auto use_idx = [&]() {
         asm volatile("s_waitcnt vmcnt(0)"
                      : "+v"(idx_next[0]), "+v"(idx_next[1]), "+v"(idx_next[2]), "+v"(idx_next[3]), "+v"(idx_next[4]),
@@ -611,30 +624,33 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
             if (kt >= KT) return; // uniform
         }
         u32x4 *dst = tiles + (kt & 1) * STAGE_CHUNKS + (piece >> 3) * OP_CHUNKS + j * 64 + wave * 512;
-        const uint16_t *src;
+        const char *src;
         if constexpr (piece < 8) {
             if (GQ)
-                src = a.DY + (int64_t)fastdiv(idx_next[j], a.dy_div) * a.lddy + q_col[j];
+                src = q_base[j] + (uint64_t)fastdiv(idx_next[j], a.dy_div) * lddy_b;
             else
-                src = q_grp[j] + (int64_t)kt * BK * a.lddy;
+                src = q_base[j] + (uint64_t)(uint32_t)(kt * BK) * lddy_b;
         } else {
             if (GP)
-                src = a.X + (int64_t)fastdiv(idx_next[j], a.x_div) * a.ldx + p_col[j];
+                src = p_base[j] + (uint64_t)fastdiv(idx_next[j], a.x_div) * ldx_b;
             else
-                src = p_grp[j] + (int64_t)kt * BK * a.ldx;
+                src = p_base[j] + (uint64_t)(uint32_t)(kt * BK) * ldx_b;
         }
         if constexpr (!FULL.value) {
             if (kt == KT - 1) { // uniform branch: k-rows past the expert's range come from the zero page
                 asm volatile("" ::: "memory"); // keeps this rare path a branch
-                if (kt * BK + kr_lane + 2 * j >= rows) src = zero;
+                if (kt * BK + kr_lane + 2 * j >= rows) src = (const char *)zero;
             }
         }
-        lds_dma16(src, dst);
+        lds_dma16((const uint16_t *)src, dst);
     };
 
     f32x16 acc[4][4];
     zero_acc(acc);
     const int wq = (wave & 1) * 128, wp = (wave >> 1) * 128;
+#ifdef XMA_EXP_TIMING3
+    uint64_t t3_loop = 0;
+#endif
     if (KT > 0) {
         // VMEM order per wave: idx(0) | dma(0) idx(1) | dma(1)[0..7] idx(2)? - see below; in the loop the indices of a
         // step are always loaded before a vmcnt(0) that precedes their use.
@@ -660,16 +676,18 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
         else
             asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
         Frags f0, f1;
+#ifdef XMA_EXP_TIMING3
+        t3_loop = wall_clock64();
+#endif
         load_frags<1, 1, 0>(f0, pb, qb);
         // one K step; FULL: steps kt + 1 and kt + 2 lie completely inside the expert's rows
         auto k_step = [&](int kt, auto FULL) {
             // idx_next holds the indices of step kt + 1 here; the second half of that step's loads goes out now, then
             // the indices of step kt + 2 are requested (they land before the barrier's vmcnt(0))
             mma_step<T, 1, 1, 1>(f0, f1, pb, qb, acc, [&](auto G) { issue_piece(kt + 1, IC<8 + G.value>{}, FULL); });
-            __builtin_amdgcn_sched_barrier(0);
-            if (GATHER) load_idx(kt + 2);
-            __builtin_amdgcn_sched_barrier(0);
-            mma_step<T, 1, 1, 2>(f1, f0, pb, qb, acc, NoHook());
+            mma_step<T, 1, 1, 2>(f1, f0, pb, qb, acc, [&](auto G) {
+                if constexpr (GATHER != 0) load_idx_one(kt + 2, G, FULL);
+            });
             mma_step<T, 1, 1, 3>(f0, f1, pb, qb, acc, NoHook());
             XMA_WAIT_LOADS_AND_BARRIER();
             if (GATHER) use_idx();
@@ -687,6 +705,9 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
     // lane owns DW row o (from the Q tile), 4 consecutive in-features per quad; each 32-row block is staged in a
     // wave-private LDS area and leaves as whole rows (see the forward kernel's epilogue)
     XMA_WAIT_LOADS_AND_BARRIER(); // no wave reads the operand tiles any more
+#ifdef XMA_EXP_TIMING3
+    const uint64_t t3_epi = wall_clock64();
+#endif
     const int lrow = lane & 31, lhalf = lane >> 5;
     uint16_t *DWe = a.DW + (int64_t)e * a.dw_es;
     unsigned char *stage = smem + wave * EPI_WAVE_BYTES;
@@ -714,6 +735,19 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
         }
         wave_lds_sync(); // the next block overwrites the area
     }
+#ifdef XMA_EXP_TIMING3
+    if (a.scale) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const uint64_t t3_end = wall_clock64();
+        if (tid == 0) {
+            uint32_t hwid, xcc;
+            asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
+            asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
+            uint64_t *dbg = (uint64_t *)a.scale + (size_t)blockIdx.x * 8;
+            dbg[0] = t3_start, dbg[1] = t3_loop, dbg[2] = t3_epi, dbg[3] = t3_end, dbg[4] = hwid, dbg[5] = xcc, dbg[6] = KT;
+        }
+    }
+#endif
 }
 
 template <typename T, int WT, int EPI> int launch_fwd(const FwdArgs &a, int grid, hipStream_t st) {
@@ -823,6 +857,8 @@ extern "C" int xma_rocm_group_bwd_W(const void *DY, int64_t lddy, int dy_grouped
                     dw_expert_stride % 8 == 0,
                 XMA_ROCM_EUNSUPPORTED, "group_bwd_W: N_out=%d K_in=%d and leading dimensions must be multiples of 8",
                 N_out, K_in);
+    XMA_REQUIRE(lddy < ((int64_t)1 << 30) && ldx < ((int64_t)1 << 30) && lddy > 0 && ldx > 0, XMA_ROCM_EUNSUPPORTED,
+                "group_bwd_W: leading dimensions must be below 2^30 elements");
     XMA_REQUIRE(DY && X && DW && expert_offsets && aligned16(DY) && aligned16(X) && aligned16(DW), XMA_ROCM_EINVAL,
                 "group_bwd_W: null or misaligned operand");
     XMA_REQUIRE(sorted_scattered_idxs || (dy_grouped && x_grouped && !dy_scale), XMA_ROCM_EINVAL,
@@ -850,7 +886,9 @@ extern "C" int xma_rocm_group_bwd_W(const void *DY, int64_t lddy, int dy_grouped
     hipStream_t st = (hipStream_t)stream;
     a.dy_div = make_fastdiv((uint32_t)dy_fan_out);
     a.x_div = make_fastdiv((uint32_t)x_fan_out);
+#ifndef XMA_EXP_TIMING3
     if (dy_scale) return launch_dw_scaled(a, dtype, (int)grid, st);
+#endif
     if (dtype == XMA_ROCM_BF16) return dispatch_dw<__bf16>(a, (int)grid, st);
     return dispatch_dw<_Float16>(a, (int)grid, st);
 }
