@@ -201,7 +201,10 @@ __device__ __forceinline__ uint32_t lds_addr_of(const void *p) {
 // by 16 bytes against bank conflicts), followed by the 32 x 64 block of SwiGLU activations.
 constexpr int EPI_Z_STRIDE = 128 * 2 + 16, EPI_H_STRIDE = 64 * 2 + 16;
 constexpr int EPI_WAVE_BYTES = 32 * EPI_Z_STRIDE + 32 * EPI_H_STRIDE;
-static_assert(4 * EPI_WAVE_BYTES <= GEMM_SMEM_BYTES, "epilogue staging must fit into the operand stages");
+// SwiGLU backward stages 32 rows of 256 pre-activation columns per wave
+constexpr int EPI_BWD_STRIDE = 256 * 2 + 16, EPI_BWD_WAVE_BYTES = 32 * EPI_BWD_STRIDE;
+static_assert(4 * EPI_WAVE_BYTES <= GEMM_SMEM_BYTES && 4 * EPI_BWD_WAVE_BYTES <= GEMM_SMEM_BYTES,
+              "epilogue staging must fit into the operand stages");
 
 // LDS written by some lanes of a wave is read by others of the same wave: instructions of one wave reach the LDS in
 // order, so only the compiler has to be kept from reordering.
@@ -325,7 +328,13 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
             if (kt >= KT) return; // uniform
         }
         u32x4 *dst = tiles + (kt & 1) * STAGE_CHUNKS + slot + wave * 512; // a wave's 8 pieces are 8 KB apart per wave
+#if defined(XMA_EXP_NOADVANCE)
+        const uint16_t *src = (piece < 8) ? q_ptr[piece] : p_ptr[piece - 8];
+#elif defined(XMA_EXP_WRAP)
+        const uint16_t *src = (piece < 8) ? q_ptr[piece] + (int64_t)(kt & 3) * BK : p_ptr[piece - 8] + (int64_t)(kt & 3) * p_step;
+#else
         const uint16_t *src = (piece < 8) ? q_ptr[piece] + (int64_t)kt * BK : p_ptr[piece - 8] + (int64_t)kt * p_step;
+#endif
         if constexpr (!FULL.value) {
             if (k_tail && kt == KT - 1) { // uniform branch, taken by at most one step of a tile
                 asm volatile("" ::: "memory"); // keeps this rare path a branch instead of selects in every piece
@@ -393,6 +402,9 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
             for (; kt + 2 < KT_full; ++kt) k_step(kt, IC<1>{});
         for (; kt < KT; ++kt) k_step(kt, IC<0>{});
     };
+#ifdef XMA_EXP_TIMING2
+    const uint64_t c0 = clock64(), w0 = wall_clock64();
+#endif
     if (q_blocks > 2)
         main_loop(IC<4>{});
     else if (q_blocks == 2)
@@ -401,6 +413,14 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
         main_loop(IC<1>{});
     else
         main_loop(IC<0>{});
+#ifdef XMA_EXP_TIMING2
+    if (EPI == XMA_ROCM_EPI_STORE && a.aux && lane == 0) {
+        const uint64_t c1 = clock64(), w1 = wall_clock64();
+        uint64_t *dbg = (uint64_t *)a.aux + ((size_t)blockIdx.x * 4 + wave) * 8;
+        dbg[5] = c1 - c0;
+        dbg[6] = w1 - w0;
+    }
+#endif
     // every load has landed, every fragment read has returned (the last sub-step reads ahead into registers nobody
     // uses), and no wave touches the operand tiles any more: LDS becomes the staging area of the epilogue
     XMA_WAIT_LOADS_AND_BARRIER();
@@ -500,21 +520,49 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
             wave_lds_sync(); // the next block overwrites the area
         }
     } else {
+        // SwiGLU backward: the accumulators are d h for the wave's 128 columns; z and dz have twice as many (gate, up
+        // interleaved).  Each 32-row block of z comes in as whole rows (2 rows of 512 bytes per instruction) through
+        // the wave-private LDS area, every lane turns its own 16-byte pieces into dz in place, and the block leaves
+        // the same way.  The z rows of block i + 1 are requested before the stores of block i go out: loads and
+        // stores retire in order, so a load issued behind the stores would wait for them.
+        unsigned char *stage = smem + wave * EPI_BWD_WAVE_BYTES;
+        unsigned char *row_io = stage + (lane >> 5) * EPI_BWD_STRIDE + (lane & 31) * 16; // + 2 it rows
+        unsigned char *mine = stage + lrow * EPI_BWD_STRIDE + lhalf * 16;                // + (32 j + 8 g) * 4 bytes
+        const int cz = 2 * (n0 + wp) + (lane & 31) * 8; // this lane's 8 columns of z / dz on the way in and out
+        const bool col_ok = cz < 2 * a.N;
+        float sc_i[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
-            const int r = wq + i * 32 + lrow;
-            if (r >= rows_valid) continue;
-            const int64_t n = row0 + r;
-            float sc = 1.f;
-            if (a.scale) sc = Elem<T>::lo((uint32_t)a.scale[a.idx[n]]);
+            int r = wq + i * 32 + lrow;
+            if (r >= rows_valid) r = rows_valid - 1;
+            sc_i[i] = 1.f;
+            if (a.scale) sc_i[i] = Elem<T>::lo((uint32_t)a.scale[a.idx[row0 + r]]);
+        }
+        u32x4 zin[16];
+        auto load_block = [&](int i) {
+#pragma unroll
+            for (int it = 0; it < 16; ++it) {
+                int r = wq + i * 32 + 2 * it + (lane >> 5);
+                if (r >= rows_valid) r = rows_valid - 1;
+                zin[it] = u32x4{0u, 0u, 0u, 0u};
+                if (col_ok) zin[it] = *(const u32x4 *)(a.aux + (row0 + r) * a.ldaux + cz);
+            }
+        };
+        if (wq < rows_valid) load_block(0);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            if (wq + i * 32 >= rows_valid) break; // wave-uniform
+#pragma unroll
+            for (int it = 0; it < 16; ++it) *(u32x4 *)(row_io + 2 * it * EPI_BWD_STRIDE) = zin[it];
+            if (i < 3 && wq + (i + 1) * 32 < rows_valid) load_block(i + 1);
+            wave_lds_sync();
+            const float sc = sc_i[i];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const int col = n0 + wp + j * 32 + g * 8 + lhalf * 4;
-                    if (col >= a.N) continue;
-                    // acc * scale = d h for 4 columns; z has 8 columns (g, u) x 4
-                    const u32x4 z = *(const u32x4 *)(a.aux + n * a.ldaux + 2 * col);
+                    u32x4 *zp = (u32x4 *)(mine + (j * 32 + g * 8) * 4);
+                    const u32x4 z = *zp;
                     u32x4 o;
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
@@ -523,9 +571,17 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
                         const float sg = sigmoidf_fast(gg), silu = gg * sg;
                         o[q] = Elem<T>::pack(dh * uu * (sg + silu * (1.f - sg)), dh * silu);
                     }
-                    *(u32x4 *)(a.out + n * a.ldo + 2 * col) = o;
+                    *zp = o;
                 }
             }
+            wave_lds_sync();
+#pragma unroll
+            for (int it = 0; it < 16; ++it) {
+                const int r = wq + i * 32 + 2 * it + (lane >> 5);
+                const u32x4 v = *(const u32x4 *)(row_io + 2 * it * EPI_BWD_STRIDE);
+                if (r < rows_valid && col_ok) *(u32x4 *)(a.out + (row0 + r) * a.ldo + cz) = v;
+            }
+            wave_lds_sync(); // the next block overwrites the area
         }
     }
 #ifdef XMA_EXP_TIMING3
