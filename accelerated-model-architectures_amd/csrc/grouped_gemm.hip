@@ -38,12 +38,8 @@ namespace xma_rocm {
 constexpr int BK = 64, NSTAGE = 2;
 // The 16 LDS-DMA pieces of a K step are issued one per MFMA slot: DMA_N0 in the sub-step right behind the barrier that
 // frees their stage, DMA_N1 and DMA_N2 in the two sub-steps after it.
-#ifndef XMA_DMA_N0
-#define XMA_DMA_N0 8
-#define XMA_DMA_N1 8
-#define XMA_DMA_N2 0
-#endif
-constexpr int DMA_N0 = XMA_DMA_N0, DMA_N1 = XMA_DMA_N1, DMA_N2 = XMA_DMA_N2;
+// (8, 8, 0) measured best; (6, 6, 4), (12, 4, 0) the same within noise, all 16 in the first sub-step slower.
+constexpr int DMA_N0 = 8, DMA_N1 = 8, DMA_N2 = 0;
 static_assert(DMA_N0 + DMA_N1 + DMA_N2 == 16 && DMA_N0 <= 16 && DMA_N1 <= 8 && DMA_N2 <= 8, "piece schedule");
 constexpr int OP_CHUNKS = 256 * 8;                          // 16-byte chunks per operand tile (32 KB)
 constexpr int STAGE_CHUNKS = 2 * OP_CHUNKS;                 // Q tile then P tile
@@ -232,9 +228,6 @@ template <typename T, int WT, int EPI>
 __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const FwdArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     __shared__ int s_sched[4];
-#ifdef XMA_EXP_TIMING3
-    const uint64_t t3_start = wall_clock64();
-#endif
     u32x4 *tiles = (u32x4 *)smem;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -328,13 +321,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
             if (kt >= KT) return; // uniform
         }
         u32x4 *dst = tiles + (kt & 1) * STAGE_CHUNKS + slot + wave * 512; // a wave's 8 pieces are 8 KB apart per wave
-#if defined(XMA_EXP_NOADVANCE)
-        const uint16_t *src = (piece < 8) ? q_ptr[piece] : p_ptr[piece - 8];
-#elif defined(XMA_EXP_WRAP)
-        const uint16_t *src = (piece < 8) ? q_ptr[piece] + (int64_t)(kt & 3) * BK : p_ptr[piece - 8] + (int64_t)(kt & 3) * p_step;
-#else
         const uint16_t *src = (piece < 8) ? q_ptr[piece] + (int64_t)kt * BK : p_ptr[piece - 8] + (int64_t)kt * p_step;
-#endif
         if constexpr (!FULL.value) {
             if (k_tail && kt == KT - 1) { // uniform branch, taken by at most one step of a tile
                 asm volatile("" ::: "memory"); // keeps this rare path a branch instead of selects in every piece
@@ -368,9 +355,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
     // share of the loads and meets every barrier.
     const int q_blocks = (rows_valid > wq) ? (rows_valid - wq + 31) >> 5 : 0;
     const int KT_full = a.K / BK; // steps without a chunk past K
-#ifdef XMA_EXP_TIMING3
-    const uint64_t t3_loop = wall_clock64();
-#endif
     auto main_loop = [&](auto NI_) {
         constexpr int NI = NI_.value;
         Frags f0, f1;
@@ -402,9 +386,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
             for (; kt + 2 < KT_full; ++kt) k_step(kt, IC<1>{});
         for (; kt < KT; ++kt) k_step(kt, IC<0>{});
     };
-#ifdef XMA_EXP_TIMING2
-    const uint64_t c0 = clock64(), w0 = wall_clock64();
-#endif
     if (q_blocks > 2)
         main_loop(IC<4>{});
     else if (q_blocks == 2)
@@ -413,20 +394,9 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
         main_loop(IC<1>{});
     else
         main_loop(IC<0>{});
-#ifdef XMA_EXP_TIMING2
-    if (EPI == XMA_ROCM_EPI_STORE && a.aux && lane == 0) {
-        const uint64_t c1 = clock64(), w1 = wall_clock64();
-        uint64_t *dbg = (uint64_t *)a.aux + ((size_t)blockIdx.x * 4 + wave) * 8;
-        dbg[5] = c1 - c0;
-        dbg[6] = w1 - w0;
-    }
-#endif
     // every load has landed, every fragment read has returned (the last sub-step reads ahead into registers nobody
     // uses), and no wave touches the operand tiles any more: LDS becomes the staging area of the epilogue
     XMA_WAIT_LOADS_AND_BARRIER();
-#ifdef XMA_EXP_TIMING3
-    const uint64_t t3_epi = wall_clock64();
-#endif
 
     // ---- epilogue: lane owns row (lane & 31) of each 32-row block; quad g of tile (j, i) holds
     //      columns n0 + wp + 32 j + 8 g + 4 (lane >> 5) + {0..3}
@@ -584,19 +554,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
             wave_lds_sync(); // the next block overwrites the area
         }
     }
-#ifdef XMA_EXP_TIMING3
-    if (EPI == XMA_ROCM_EPI_STORE && a.aux) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        const uint64_t t3_end = wall_clock64();
-        if (tid == 0) {
-            uint32_t hwid, xcc;
-            asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-            asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-            uint64_t *dbg = (uint64_t *)a.aux + (size_t)blockIdx.x * 8;
-            dbg[0] = t3_start, dbg[1] = t3_loop, dbg[2] = t3_epi, dbg[3] = t3_end, dbg[4] = hwid, dbg[5] = xcc, dbg[6] = rows_valid;
-        }
-    }
-#endif
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -607,9 +564,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
 template <typename T, int GQ, int GP>
 __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const DwArgs a) {
     constexpr int GATHER = GQ | GP;
-#ifdef XMA_EXP_TIMING3
-    const uint64_t t3_start = wall_clock64();
-#endif
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     u32x4 *tiles = (u32x4 *)smem;
     const int tid = threadIdx.x, lane = tid & 63;
@@ -704,9 +658,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
     f32x16 acc[4][4];
     zero_acc(acc);
     const int wq = (wave & 1) * 128, wp = (wave >> 1) * 128;
-#ifdef XMA_EXP_TIMING3
-    uint64_t t3_loop = 0;
-#endif
     if (KT > 0) {
         // VMEM order per wave: idx(0) | dma(0) idx(1) | dma(1)[0..7] idx(2)? - see below; in the loop the indices of a
         // step are always loaded before a vmcnt(0) that precedes their use.
@@ -732,9 +683,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
         else
             asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
         Frags f0, f1;
-#ifdef XMA_EXP_TIMING3
-        t3_loop = wall_clock64();
-#endif
         load_frags<1, 1, 0>(f0, pb, qb);
         // one K step; FULL: steps kt + 1 and kt + 2 lie completely inside the expert's rows
         auto k_step = [&](int kt, auto FULL) {
@@ -761,9 +709,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
     // lane owns DW row o (from the Q tile), 4 consecutive in-features per quad; each 32-row block is staged in a
     // wave-private LDS area and leaves as whole rows (see the forward kernel's epilogue)
     XMA_WAIT_LOADS_AND_BARRIER(); // no wave reads the operand tiles any more
-#ifdef XMA_EXP_TIMING3
-    const uint64_t t3_epi = wall_clock64();
-#endif
     const int lrow = lane & 31, lhalf = lane >> 5;
     uint16_t *DWe = a.DW + (int64_t)e * a.dw_es;
     unsigned char *stage = smem + wave * EPI_WAVE_BYTES;
@@ -791,19 +736,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
         }
         wave_lds_sync(); // the next block overwrites the area
     }
-#ifdef XMA_EXP_TIMING3
-    if (a.scale) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        const uint64_t t3_end = wall_clock64();
-        if (tid == 0) {
-            uint32_t hwid, xcc;
-            asm volatile("s_getreg_b32 %0, hwreg(HW_REG_HW_ID)" : "=s"(hwid));
-            asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(xcc));
-            uint64_t *dbg = (uint64_t *)a.scale + (size_t)blockIdx.x * 8;
-            dbg[0] = t3_start, dbg[1] = t3_loop, dbg[2] = t3_epi, dbg[3] = t3_end, dbg[4] = hwid, dbg[5] = xcc, dbg[6] = KT;
-        }
-    }
-#endif
 }
 
 template <typename T, int WT, int EPI> int launch_fwd(const FwdArgs &a, int grid, hipStream_t st) {
@@ -942,9 +874,7 @@ extern "C" int xma_rocm_group_bwd_W(const void *DY, int64_t lddy, int dy_grouped
     hipStream_t st = (hipStream_t)stream;
     a.dy_div = make_fastdiv((uint32_t)dy_fan_out);
     a.x_div = make_fastdiv((uint32_t)x_fan_out);
-#ifndef XMA_EXP_TIMING3
     if (dy_scale) return launch_dw_scaled(a, dtype, (int)grid, st);
-#endif
     if (dtype == XMA_ROCM_BF16) return dispatch_dw<__bf16>(a, (int)grid, st);
     return dispatch_dw<_Float16>(a, (int)grid, st);
 }
