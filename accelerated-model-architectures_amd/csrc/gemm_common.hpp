@@ -36,6 +36,9 @@ struct FwdArgs {
     const uint16_t *scale;
     int64_t M;
     int N, K, E, fan_out, x_grouped, y_grouped;
+    float *partial;  // workspace for the K slices of the tiles of the last round, or NULL (no tile is split)
+    int split_cus;   // compute units of the device = tiles per round
+    int grid_main;   // workgroups that take whole tiles (an upper bound of the tile count); split_cus more follow
 };
 
 struct DwArgs {

@@ -219,21 +219,28 @@ template <int N> __device__ __forceinline__ void zero_acc(f32x16 (&acc)[N][N]) {
             for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.f;
 }
 
-// ------------------------------------------------------------------------------------------------
-// forward / dX kernel
-//   WT = 0: W[e] is (N, K) with K contiguous (x @ W^T)      -> P tile row-major
-//   WT = 1: W[e] is (K, N) with N contiguous (dy @ W)       -> P tile transposed source
-// ------------------------------------------------------------------------------------------------
-template <typename T, int WT, int EPI>
-__global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const FwdArgs a) {
-    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
-    __shared__ int s_sched[4];
-    u32x4 *tiles = (u32x4 *)smem;
+// Which tile a workgroup works on.
+struct TileSched {
+    int e, rows_valid, n0; // expert, valid rows of the row tile, first output column
+    int64_t row0;          // first grouped row
+    int part, parts;       // K slice of a split tile (parts == 1: the whole K range)
+    int tail_index;        // index of a split tile among the tiles of the last round
+};
+
+constexpr int SPLIT_MIN_STEPS = 8; // a K slice is at least this many K steps
+
+// Expert-major schedule: work[e] = ceil(rows_e / BM) * n_tiles, prefix sum over the experts in LDS, then the tile of
+// this workgroup.  With a workspace (a.partial) the tiles of the last, partial round of the launch - total mod
+// split_cus of them, the workgroups that would otherwise run while most CUs idle - are cut into `parts` K slices, each
+// taken by a workgroup of its own in a second launch of the kernel (ROLE_SLICES, at most split_cus workgroups); a
+// third launch (ROLE_FIXUP, workgroup b = split tile b) adds the slices.  ROLE_TILES takes all other tiles.  Returns
+// false if the workgroup has nothing to do.
+constexpr int ROLE_TILES = 0, ROLE_SLICES = 1, ROLE_FIXUP = 2;
+template <int ROLE>
+__device__ __forceinline__ bool locate_tile(const FwdArgs &a, unsigned char *smem, int *s_sched, TileSched &ts) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int NT = (a.N + BN - 1) / BN;
-
-    // ---- expert-major schedule: work[e] = ceil(rows_e / BM) * NT, prefix, locate this tile
     int *s_pre = (int *)smem; // [E + 1], dead before the first tile load
     if (tid == 0) s_sched[0] = -1;
     if (wave == 0) {
@@ -257,148 +264,61 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
         if (lane == 0) s_pre[a.E] = carry;
     }
     __syncthreads();
-    const int L = xcd_remap(blockIdx.x, gridDim.x);
+    const int total = __builtin_amdgcn_readfirstlane(s_pre[a.E]); // uniform: keep the whole schedule in scalar registers
+    int full = total, rest = 0, parts = 1;
+    if (a.partial) {
+        const int KT = (a.K + BK - 1) / BK;
+        full = total / a.split_cus * a.split_cus;
+        rest = total - full;
+        parts = rest ? a.split_cus / rest : 1;
+        if (parts > KT / SPLIT_MIN_STEPS) parts = KT / SPLIT_MIN_STEPS;
+        if (parts < 2) parts = 1, full = total, rest = 0;
+    }
+    int L, part = 0;
+    const int b = (int)blockIdx.x;
+    if (ROLE == ROLE_FIXUP) {
+        if (b >= rest) return false;
+        L = full + b;
+    } else if (ROLE == ROLE_SLICES) {
+        if (rest == 0) return false;
+        const int q = xcd_remap(b, a.split_cus); // neighbouring tiles of one slice index meet in one XCD's L2
+        part = q / rest;
+        if (part >= parts) return false;
+        L = full + q % rest;
+    } else {
+        L = xcd_remap(b, a.grid_main);
+        if (L >= full) return false; // beyond the last tile (the grid is an upper bound), or a tile that is split
+    }
     for (int e = tid; e < a.E; e += GEMM_THREADS)
         if (s_pre[e] <= L && L < s_pre[e + 1]) {
             s_sched[0] = e;
             s_sched[1] = L - s_pre[e];
         }
     __syncthreads();
-    const int e = s_sched[0];
-    if (e < 0) return; // beyond the last tile (the grid is an upper bound)
+    const int e = __builtin_amdgcn_readfirstlane(s_sched[0]);
+    const int local = __builtin_amdgcn_readfirstlane(s_sched[1]);
     const int64_t row_lo = e ? a.offs[e - 1] : 0, row_hi = a.offs[e];
     const int tiles_m = (int)((row_hi - row_lo + BM - 1) / BM);
-    const int m_tile = s_sched[1] % tiles_m, n_tile = s_sched[1] / tiles_m;
-    const int64_t row0 = row_lo + (int64_t)m_tile * BM;
-    const int rows_valid = (int)((row_hi - row0 < BM) ? row_hi - row0 : BM);
-    const int n0 = n_tile * BN;
+    const int m_tile = local % tiles_m, n_tile = local / tiles_m;
+    ts.e = e;
+    ts.row0 = row_lo + (int64_t)m_tile * BM;
+    ts.rows_valid = (int)((row_hi - ts.row0 < BM) ? row_hi - ts.row0 : BM);
+    ts.n0 = n_tile * BN;
+    ts.part = part;
+    ts.parts = (L >= full) ? parts : 1;
+    ts.tail_index = L - full;
     __syncthreads(); // s_pre is dead from here on
+    return true;
+}
 
-    // ---- loader set-up: one fixed per-lane global pointer per LDS-DMA piece (k = 0); a step adds a uniform offset
-    const uint16_t *zero = (const uint16_t *)g_zero_page;
-    const int KT = (a.K + BK - 1) / BK;
-    const bool k_tail = (a.K & (BK - 1)) != 0; // the last step has chunks past K: they are fetched from the zero page
-    const uint16_t *q_ptr[8], *p_ptr[8];
-    {
-        const int c = rowmajor_lane_chunk(lane);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            int r = wave * 64 + i * 8 + (lane >> 3);
-            if (r >= rows_valid) r = rows_valid - 1; // duplicates, masked at the store
-            const int64_t n = row0 + r;
-            const int64_t src = a.x_grouped ? n : a.idx[n] / a.fan_out;
-            q_ptr[i] = a.X + src * a.ldx + c * 8;
-        }
-        const uint16_t *We = a.W + (int64_t)e * a.w_es;
-        if (WT == 0) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                int r = n0 + wave * 64 + i * 8 + (lane >> 3);
-                if (r >= a.N) r = a.N - 1;
-                p_ptr[i] = We + (int64_t)r * a.ldw + c * 8;
-            }
-        } else {
-            const int max_chunk = ((a.N - n0) >> 3) - 1; // last valid 16-byte chunk of the tile's column range
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                int cj = transposed_lane_chunk(j, lane);
-                if (cj > max_chunk) cj = max_chunk; // columns past the edge are masked at the store
-                p_ptr[j] = We + (int64_t)(wave * 16 + 2 * j + (lane >> 5)) * a.ldw + n0 + cj * 8;
-            }
-        }
-    }
-    const int64_t p_step = (WT == 0) ? BK : (int64_t)BK * a.ldw; // elements per K step along the P pointers
-    const uint32_t lds0 = lds_addr_of(smem);
-
-    // piece 0..15 of K step kt -> stage kt & 1 (pieces 0..7 = Q tile, 8..15 = P tile).  FULL: the caller guarantees
-    // that step kt exists and has no chunk past K, so the piece is one M0 update, one 64-bit add and the load; a wave
-    // with a single instruction stream cannot afford more than a few instructions per MFMA.
-    auto issue_piece = [&](int kt, auto PIECE, auto FULL) {
-        constexpr int piece = PIECE.value;
-        constexpr int slot =
-            (piece >> 3) * OP_CHUNKS + ((piece < 8 || WT == 0) ? (piece & 7) * 64 : (piece & 7) * 64); // 1 KB per piece
-        if constexpr (!FULL.value) {
-            if (kt >= KT) return; // uniform
-        }
-        u32x4 *dst = tiles + (kt & 1) * STAGE_CHUNKS + slot + wave * 512; // a wave's 8 pieces are 8 KB apart per wave
-        const uint16_t *src = (piece < 8) ? q_ptr[piece] + (int64_t)kt * BK : p_ptr[piece - 8] + (int64_t)kt * p_step;
-        if constexpr (!FULL.value) {
-            if (k_tail && kt == KT - 1) { // uniform branch, taken by at most one step of a tile
-                asm volatile("" ::: "memory"); // keeps this rare path a branch instead of selects in every piece
-                if (piece < 8 || WT == 0) {
-                    if (kt * BK + rowmajor_lane_chunk(lane) * 8 >= a.K) src = zero;
-                } else {
-                    if (kt * BK + wave * 16 + 2 * (piece - 8) + (lane >> 5) >= a.K) src = zero;
-                }
-            }
-        }
-        lds_dma16(src, dst);
-    };
-
-    f32x16 acc[4][4];
-    zero_acc(acc);
+// ---- epilogue of one 256 x 256 tile (LDS is free: no wave reads operand tiles any more)
+template <typename T, int EPI>
+__device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4][4], unsigned char *smem, int64_t row0,
+                                              int rows_valid, int n0) {
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wq = (wave & 1) * 128, wp = (wave >> 1) * 128; // wave's 128 x 128 corner inside the tile
-    FragBase<0> qb;
-    FragBase<WT> pb;
-    make_frag_base<0>(qb, lds0, wq, lane);
-    make_frag_base<WT>(pb, lds0 + OP_CHUNKS * 16, wp, lane);
-
-    static_for<16>([&](auto P) { issue_piece(0, P, IC<0>{}); });
-    static_for<DMA_N0>([&](auto P) { issue_piece(1, P, IC<0>{}); });
-    // step 0 has landed in every wave (the first loads of step 1 may be in flight)
-    if (KT > 1)
-        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(DMA_N0) : "memory");
-    else
-        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
-    // Q blocks (32 rows) of this wave that hold valid rows: 4 except in an expert's last row tile.  A wave with fewer
-    // skips the MFMAs and fragment reads of the empty blocks (rounded up to 0, 1, 2 or 4 blocks); it still issues its
-    // share of the loads and meets every barrier.
-    const int q_blocks = (rows_valid > wq) ? (rows_valid - wq + 31) >> 5 : 0;
-    const int KT_full = a.K / BK; // steps without a chunk past K
-    auto main_loop = [&](auto NI_) {
-        constexpr int NI = NI_.value;
-        Frags f0, f1;
-        if constexpr (NI > 0) {
-            static_for<4>([&](auto I) { f0.p[I.value] = read_frag<WT, I.value, 0>(pb); });
-            static_for<NI>([&](auto I) { f0.q[I.value] = read_frag<0, I.value, 0>(qb); });
-        }
-        // one K step; FULL: steps kt + 1 and kt + 2 exist and are complete
-        auto k_step = [&](int kt, auto FULL) {
-            // rest of the loads of step kt + 1 (the first DMA_N0 went out behind the previous barrier)
-            mma_step<T, WT, 0, 1, NI>(f0, f1, pb, qb, acc, [&](auto G) {
-                if constexpr (G.value < DMA_N1) issue_piece(kt + 1, IC<DMA_N0 + G.value>{}, FULL);
-            });
-            mma_step<T, WT, 0, 2, NI>(f1, f0, pb, qb, acc, [&](auto G) {
-                if constexpr (G.value < DMA_N2) issue_piece(kt + 1, IC<DMA_N0 + DMA_N1 + G.value>{}, FULL);
-            });
-            mma_step<T, WT, 0, 3, NI>(f0, f1, pb, qb, acc, NoHook());
-            XMA_WAIT_LOADS_AND_BARRIER(); // step kt + 1 has landed; nobody reads this stage any more
-            flip_stage(pb);
-            flip_stage(qb);
-            // the stage just left is free: first loads of step kt + 2; fragments of sub-step 0 of step kt + 1
-            mma_step<T, WT, 0, 0, NI>(f1, f0, pb, qb, acc, [&](auto G) {
-                if constexpr (G.value < DMA_N0) issue_piece(kt + 2, G, FULL);
-                if constexpr (G.value + 8 < DMA_N0) issue_piece(kt + 2, IC<G.value + 8>{}, FULL);
-            });
-        };
-        int kt = 0;
-        if constexpr (NI == 4)
-            for (; kt + 2 < KT_full; ++kt) k_step(kt, IC<1>{});
-        for (; kt < KT; ++kt) k_step(kt, IC<0>{});
-    };
-    if (q_blocks > 2)
-        main_loop(IC<4>{});
-    else if (q_blocks == 2)
-        main_loop(IC<2>{});
-    else if (q_blocks == 1)
-        main_loop(IC<1>{});
-    else
-        main_loop(IC<0>{});
-    // every load has landed, every fragment read has returned (the last sub-step reads ahead into registers nobody
-    // uses), and no wave touches the operand tiles any more: LDS becomes the staging area of the epilogue
-    XMA_WAIT_LOADS_AND_BARRIER();
-
-    // ---- epilogue: lane owns row (lane & 31) of each 32-row block; quad g of tile (j, i) holds
+    // lane owns row (lane & 31) of each 32-row block; quad g of tile (j, i) holds
     //      columns n0 + wp + 32 j + 8 g + 4 (lane >> 5) + {0..3}
     const int lrow = lane & 31, lhalf = lane >> 5;
     if constexpr (EPI != XMA_ROCM_EPI_SWIGLU_BWD) {
@@ -554,6 +474,194 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
             wave_lds_sync(); // the next block overwrites the area
         }
     }
+}
+
+// ------------------------------------------------------------------------------------------------
+// forward / dX kernel
+//   WT = 0: W[e] is (N, K) with K contiguous (x @ W^T)      -> P tile row-major
+//   WT = 1: W[e] is (K, N) with N contiguous (dy @ W)       -> P tile transposed source
+// ------------------------------------------------------------------------------------------------
+template <typename T, int WT, int EPI, int ROLE>
+__global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const FwdArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    __shared__ int s_sched[4];
+    u32x4 *tiles = (u32x4 *)smem;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+
+    TileSched ts;
+    if (!locate_tile<ROLE>(a, smem, s_sched, ts)) return;
+    const int e = ts.e, rows_valid = ts.rows_valid, n0 = ts.n0;
+    const int64_t row0 = ts.row0;
+
+    // ---- loader set-up: one fixed per-lane global pointer per LDS-DMA piece (k = 0); a step adds a uniform offset
+    const uint16_t *zero = (const uint16_t *)g_zero_page;
+    const int KT = (a.K + BK - 1) / BK;
+    const bool k_tail = (a.K & (BK - 1)) != 0; // the last step has chunks past K: they are fetched from the zero page
+    // K steps [kt0, kt1) of this workgroup: all of them, or one of ts.parts slices of a tile of the last round.  kt0 is
+    // even, so step kt lives in stage kt & 1 in either case.
+    const int kt0 = (ROLE == ROLE_SLICES) ? ((ts.part * KT / ts.parts) & ~1) : 0;
+    const int kt1 = (ROLE == ROLE_SLICES && ts.part + 1 < ts.parts) ? (((ts.part + 1) * KT / ts.parts) & ~1) : KT;
+    const uint16_t *q_ptr[8], *p_ptr[8];
+    {
+        const int c = rowmajor_lane_chunk(lane);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            int r = wave * 64 + i * 8 + (lane >> 3);
+            if (r >= rows_valid) r = rows_valid - 1; // duplicates, masked at the store
+            const int64_t n = row0 + r;
+            const int64_t src = a.x_grouped ? n : a.idx[n] / a.fan_out;
+            q_ptr[i] = a.X + src * a.ldx + c * 8;
+        }
+        const uint16_t *We = a.W + (int64_t)e * a.w_es;
+        if (WT == 0) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                int r = n0 + wave * 64 + i * 8 + (lane >> 3);
+                if (r >= a.N) r = a.N - 1;
+                p_ptr[i] = We + (int64_t)r * a.ldw + c * 8;
+            }
+        } else {
+            const int max_chunk = ((a.N - n0) >> 3) - 1; // last valid 16-byte chunk of the tile's column range
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                int cj = transposed_lane_chunk(j, lane);
+                if (cj > max_chunk) cj = max_chunk; // columns past the edge are masked at the store
+                p_ptr[j] = We + (int64_t)(wave * 16 + 2 * j + (lane >> 5)) * a.ldw + n0 + cj * 8;
+            }
+        }
+    }
+    const int64_t p_step = (WT == 0) ? BK : (int64_t)BK * a.ldw; // elements per K step along the P pointers
+    const uint32_t lds0 = lds_addr_of(smem);
+
+    // piece 0..15 of K step kt -> stage kt & 1 (pieces 0..7 = Q tile, 8..15 = P tile).  FULL: the caller guarantees
+    // that step kt exists and has no chunk past K, so the piece is one M0 update, one 64-bit add and the load; a wave
+    // with a single instruction stream cannot afford more than a few instructions per MFMA.
+    auto issue_piece = [&](int kt, auto PIECE, auto FULL) {
+        constexpr int piece = PIECE.value;
+        constexpr int slot =
+            (piece >> 3) * OP_CHUNKS + ((piece < 8 || WT == 0) ? (piece & 7) * 64 : (piece & 7) * 64); // 1 KB per piece
+        if constexpr (!FULL.value) {
+            if (kt >= kt1) return; // uniform
+        }
+        u32x4 *dst = tiles + (kt & 1) * STAGE_CHUNKS + slot + wave * 512; // a wave's 8 pieces are 8 KB apart per wave
+        const uint16_t *src = (piece < 8) ? q_ptr[piece] + (int64_t)kt * BK : p_ptr[piece - 8] + (int64_t)kt * p_step;
+        if constexpr (!FULL.value) {
+            if (k_tail && kt == KT - 1) { // uniform branch, taken by at most one step of a tile
+                asm volatile("" ::: "memory"); // keeps this rare path a branch instead of selects in every piece
+                if (piece < 8 || WT == 0) {
+                    if (kt * BK + rowmajor_lane_chunk(lane) * 8 >= a.K) src = zero;
+                } else {
+                    if (kt * BK + wave * 16 + 2 * (piece - 8) + (lane >> 5) >= a.K) src = zero;
+                }
+            }
+        }
+        lds_dma16(src, dst);
+    };
+
+    f32x16 acc[4][4];
+    zero_acc(acc);
+    const int wq = (wave & 1) * 128, wp = (wave >> 1) * 128; // wave's 128 x 128 corner inside the tile
+    FragBase<0> qb;
+    FragBase<WT> pb;
+    make_frag_base<0>(qb, lds0, wq, lane);
+    make_frag_base<WT>(pb, lds0 + OP_CHUNKS * 16, wp, lane);
+
+    static_for<16>([&](auto P) { issue_piece(kt0, P, IC<0>{}); });
+    static_for<DMA_N0>([&](auto P) { issue_piece(kt0 + 1, P, IC<0>{}); });
+    // the first step has landed in every wave (the first loads of the second may be in flight)
+    if (kt1 - kt0 > 1)
+        asm volatile("s_waitcnt vmcnt(%0)\n\ts_barrier" ::"n"(DMA_N0) : "memory");
+    else
+        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+    // Q blocks (32 rows) of this wave that hold valid rows: 4 except in an expert's last row tile.  A wave with fewer
+    // skips the MFMAs and fragment reads of the empty blocks (rounded up to 0, 1, 2 or 4 blocks); it still issues its
+    // share of the loads and meets every barrier.
+    const int q_blocks = (rows_valid > wq) ? (rows_valid - wq + 31) >> 5 : 0;
+    const int KT_full = (a.K / BK < kt1) ? a.K / BK : kt1; // end of the steps without a chunk past K
+    auto main_loop = [&](auto NI_) {
+        constexpr int NI = NI_.value;
+        Frags f0, f1;
+        if constexpr (NI > 0) {
+            static_for<4>([&](auto I) { f0.p[I.value] = read_frag<WT, I.value, 0>(pb); });
+            static_for<NI>([&](auto I) { f0.q[I.value] = read_frag<0, I.value, 0>(qb); });
+        }
+        // one K step; FULL: steps kt + 1 and kt + 2 exist and are complete
+        auto k_step = [&](int kt, auto FULL) {
+            // rest of the loads of step kt + 1 (the first DMA_N0 went out behind the previous barrier)
+            mma_step<T, WT, 0, 1, NI>(f0, f1, pb, qb, acc, [&](auto G) {
+                if constexpr (G.value < DMA_N1) issue_piece(kt + 1, IC<DMA_N0 + G.value>{}, FULL);
+            });
+            mma_step<T, WT, 0, 2, NI>(f1, f0, pb, qb, acc, [&](auto G) {
+                if constexpr (G.value < DMA_N2) issue_piece(kt + 1, IC<DMA_N0 + DMA_N1 + G.value>{}, FULL);
+            });
+            mma_step<T, WT, 0, 3, NI>(f0, f1, pb, qb, acc, NoHook());
+            XMA_WAIT_LOADS_AND_BARRIER(); // step kt + 1 has landed; nobody reads this stage any more
+            flip_stage(pb);
+            flip_stage(qb);
+            // the stage just left is free: first loads of step kt + 2; fragments of sub-step 0 of step kt + 1
+            mma_step<T, WT, 0, 0, NI>(f1, f0, pb, qb, acc, [&](auto G) {
+                if constexpr (G.value < DMA_N0) issue_piece(kt + 2, G, FULL);
+                if constexpr (G.value + 8 < DMA_N0) issue_piece(kt + 2, IC<G.value + 8>{}, FULL);
+            });
+        };
+        int kt = kt0;
+        if constexpr (NI == 4)
+            for (; kt + 2 < KT_full; ++kt) k_step(kt, IC<1>{});
+        for (; kt < kt1; ++kt) k_step(kt, IC<0>{});
+    };
+    if (q_blocks > 2)
+        main_loop(IC<4>{});
+    else if (q_blocks == 2)
+        main_loop(IC<2>{});
+    else if (q_blocks == 1)
+        main_loop(IC<1>{});
+    else
+        main_loop(IC<0>{});
+    // every load has landed, every fragment read has returned (the last sub-step reads ahead into registers nobody
+    // uses), and no wave touches the operand tiles any more: LDS becomes the staging area of the epilogue
+    XMA_WAIT_LOADS_AND_BARRIER();
+
+    if constexpr (ROLE == ROLE_SLICES) {
+        // one K slice of a tile of the last round: the fp32 accumulators go to the workspace, 16 bytes per lane and
+        // consecutive lanes side by side; grouped_gemm_fixup_kernel adds the slices and runs the epilogue
+        float4 *dst = (float4 *)a.partial + (size_t)(ts.tail_index * ts.parts + ts.part) * (BM * BN / 4) + tid;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int g = 0; g < 4; ++g)
+                    dst[((j * 4 + i) * 4 + g) * GEMM_THREADS] =
+                        make_float4(acc[j][i][4 * g], acc[j][i][4 * g + 1], acc[j][i][4 * g + 2], acc[j][i][4 * g + 3]);
+    } else
+        tile_epilogue<T, EPI>(a, acc, smem, row0, rows_valid, n0);
+}
+
+// Sum of the K slices of the split tiles of the last round, then the epilogue of the GEMM kernel.  One workgroup per
+// split tile; the slices are added in a fixed order, so the result does not depend on timing.
+template <typename T, int EPI>
+__global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_fixup_kernel(const FwdArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    __shared__ int s_sched[4];
+    TileSched ts;
+    if (!locate_tile<ROLE_FIXUP>(a, smem, s_sched, ts)) return;
+    const int tid = threadIdx.x;
+    f32x16 acc[4][4];
+    zero_acc(acc);
+    for (int p = 0; p < ts.parts; ++p) {
+        const float4 *src = (const float4 *)a.partial + (size_t)(ts.tail_index * ts.parts + p) * (BM * BN / 4) + tid;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const float4 v = src[((j * 4 + i) * 4 + g) * GEMM_THREADS];
+                    acc[j][i][4 * g] += v.x, acc[j][i][4 * g + 1] += v.y, acc[j][i][4 * g + 2] += v.z, acc[j][i][4 * g + 3] += v.w;
+                }
+    }
+    tile_epilogue<T, EPI>(a, acc, smem, ts.row0, ts.rows_valid, ts.n0);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -738,11 +846,19 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
     }
 }
 
-template <typename T, int WT, int EPI> int launch_fwd(const FwdArgs &a, int grid, hipStream_t st) {
-    int rc = gemm_set_smem(grouped_gemm_kernel<T, WT, EPI>, GEMM_SMEM_BYTES);
+template <typename T, int WT, int EPI> int launch_fwd(const FwdArgs &a, hipStream_t st) {
+    int rc = gemm_set_smem(grouped_gemm_kernel<T, WT, EPI, ROLE_TILES>, GEMM_SMEM_BYTES);
     if (rc) return rc;
-    grouped_gemm_kernel<T, WT, EPI><<<grid, GEMM_THREADS, GEMM_SMEM_BYTES, st>>>(a);
-    return xma_check_launch("grouped_gemm_kernel");
+    grouped_gemm_kernel<T, WT, EPI, ROLE_TILES><<<a.grid_main, GEMM_THREADS, GEMM_SMEM_BYTES, st>>>(a);
+    if ((rc = xma_check_launch("grouped_gemm_kernel"))) return rc;
+    if (!a.partial) return XMA_ROCM_OK;
+    // the tiles of the last round as K slices (no epilogue: one instantiation serves all), then their sum + epilogue
+    if ((rc = gemm_set_smem(grouped_gemm_kernel<T, WT, XMA_ROCM_EPI_STORE, ROLE_SLICES>, GEMM_SMEM_BYTES))) return rc;
+    grouped_gemm_kernel<T, WT, XMA_ROCM_EPI_STORE, ROLE_SLICES><<<a.split_cus, GEMM_THREADS, GEMM_SMEM_BYTES, st>>>(a);
+    if ((rc = xma_check_launch("grouped_gemm_kernel (K slices)"))) return rc;
+    if ((rc = gemm_set_smem(grouped_gemm_fixup_kernel<T, EPI>, GEMM_SMEM_BYTES))) return rc;
+    grouped_gemm_fixup_kernel<T, EPI><<<a.split_cus, GEMM_THREADS, GEMM_SMEM_BYTES, st>>>(a);
+    return xma_check_launch("grouped_gemm_fixup_kernel");
 }
 
 template <typename T, int GQ, int GP> int launch_dw(const DwArgs &a, int grid, hipStream_t st) {
@@ -757,15 +873,39 @@ template <typename T> int dispatch_dw(const DwArgs &a, int grid, hipStream_t st)
     return a.x_grouped ? launch_dw<T, 1, 0>(a, grid, st) : launch_dw<T, 1, 1>(a, grid, st);
 }
 
-template <typename T> int dispatch_fwd(const FwdArgs &a, int wt, int epi, int grid, hipStream_t st) {
+template <typename T> int dispatch_fwd(const FwdArgs &a, int wt, int epi, hipStream_t st) {
     if (wt == 0) {
-        if (epi == XMA_ROCM_EPI_STORE) return launch_fwd<T, 0, XMA_ROCM_EPI_STORE>(a, grid, st);
-        if (epi == XMA_ROCM_EPI_SWIGLU) return launch_fwd<T, 0, XMA_ROCM_EPI_SWIGLU>(a, grid, st);
-        return launch_fwd<T, 0, XMA_ROCM_EPI_SWIGLU_BWD>(a, grid, st);
+        if (epi == XMA_ROCM_EPI_STORE) return launch_fwd<T, 0, XMA_ROCM_EPI_STORE>(a, st);
+        if (epi == XMA_ROCM_EPI_SWIGLU) return launch_fwd<T, 0, XMA_ROCM_EPI_SWIGLU>(a, st);
+        return launch_fwd<T, 0, XMA_ROCM_EPI_SWIGLU_BWD>(a, st);
     }
-    if (epi == XMA_ROCM_EPI_STORE) return launch_fwd<T, 1, XMA_ROCM_EPI_STORE>(a, grid, st);
-    if (epi == XMA_ROCM_EPI_SWIGLU) return launch_fwd<T, 1, XMA_ROCM_EPI_SWIGLU>(a, grid, st);
-    return launch_fwd<T, 1, XMA_ROCM_EPI_SWIGLU_BWD>(a, grid, st);
+    if (epi == XMA_ROCM_EPI_STORE) return launch_fwd<T, 1, XMA_ROCM_EPI_STORE>(a, st);
+    if (epi == XMA_ROCM_EPI_SWIGLU) return launch_fwd<T, 1, XMA_ROCM_EPI_SWIGLU>(a, st);
+    return launch_fwd<T, 1, XMA_ROCM_EPI_SWIGLU_BWD>(a, st);
+}
+
+// Compute units of the current device (tiles that run at the same time), looked up once per device.
+inline int device_cus() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+
+// Launches of fewer rounds than this may split the tiles of their last round over the idle CUs.
+constexpr int64_t SPLIT_MAX_ROUNDS = 12;
+
+inline size_t fwd_workspace_bytes(int64_t M, int32_t N, int32_t E) {
+    const int cus = device_cus();
+    if (cus <= 0) return 0;
+    const int64_t tiles = (M / BM + E) * ((N + BN - 1) / BN);
+    if (tiles > SPLIT_MAX_ROUNDS * cus) return 0;
+    return (size_t)cus * BM * BN * sizeof(float);
 }
 
 inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
@@ -779,7 +919,7 @@ extern "C" int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *
                                         const int64_t *expert_offsets, void *out, int64_t ldo, void *aux, int64_t ldaux,
                                         const void *row_scale, int64_t M, int32_t N, int32_t K, int32_t E,
                                         int32_t fan_out, int x_grouped, int y_grouped, int epilogue, int dtype,
-                                        void *stream) {
+                                        void *workspace, size_t workspace_bytes, void *stream) {
     XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED, "scatter2scatter: dtype %d", dtype);
     XMA_REQUIRE(epilogue >= XMA_ROCM_EPI_STORE && epilogue <= XMA_ROCM_EPI_SWIGLU_BWD, XMA_ROCM_EINVAL,
                 "scatter2scatter: epilogue %d", epilogue);
@@ -827,10 +967,26 @@ extern "C" int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *
     const int64_t NT = (N + BN - 1) / BN;
     const int64_t max_m_tiles = M / BM + E; // sum_e ceil(c_e / BM) <= floor(M / BM) + E
     const int64_t grid = max_m_tiles * NT;
-    XMA_REQUIRE(grid < ((int64_t)1 << 31), XMA_ROCM_EUNSUPPORTED, "scatter2scatter: grid too large");
+    XMA_REQUIRE(grid < ((int64_t)1 << 30), XMA_ROCM_EUNSUPPORTED, "scatter2scatter: grid too large");
+    a.grid_main = (int)grid;
+    a.partial = nullptr;
+    a.split_cus = 0;
+    const size_t ws_need = fwd_workspace_bytes(M, N, E);
+    if (workspace && ws_need) {
+        XMA_REQUIRE(workspace_bytes >= ws_need && aligned16(workspace), XMA_ROCM_EWORKSPACE,
+                    "scatter2scatter: workspace of %zu bytes, %zu needed (16-byte aligned)", workspace_bytes, ws_need);
+        a.partial = (float *)workspace;
+        a.split_cus = device_cus();
+    }
     hipStream_t st = (hipStream_t)stream;
-    if (dtype == XMA_ROCM_BF16) return dispatch_fwd<__bf16>(a, w_is_kn ? 1 : 0, epilogue, (int)grid, st);
-    return dispatch_fwd<_Float16>(a, w_is_kn ? 1 : 0, epilogue, (int)grid, st);
+    if (dtype == XMA_ROCM_BF16) return dispatch_fwd<__bf16>(a, w_is_kn ? 1 : 0, epilogue, st);
+    return dispatch_fwd<_Float16>(a, w_is_kn ? 1 : 0, epilogue, st);
+}
+
+extern "C" size_t xma_rocm_scatter2scatter_workspace_bytes(int64_t M, int32_t N, int32_t K, int32_t E) {
+    (void)K;
+    if (M <= 0 || N <= 0 || E <= 0) return 0;
+    return fwd_workspace_bytes(M, N, E);
 }
 
 extern "C" int xma_rocm_group_bwd_W(const void *DY, int64_t lddy, int dy_grouped, int32_t dy_fan_out,

@@ -124,11 +124,16 @@ def _scatter2scatter(X, W, idx, offs, out, aux, scale, fan_out, x_grouped, y_gro
     if scale is not None:
         assert scale.dtype == X.dtype and scale.is_contiguous()
     lib = get_library()
+    # scratch for the K slices of the tiles of a last, partial round (0 bytes for launches of many rounds); it comes from
+    # torch's caching allocator like every other buffer of the op
+    ws_bytes = lib.xma_rocm_scatter2scatter_workspace_bytes(M, N, K, W.size(0))
+    workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=X.device) if ws_bytes else None
     check(
         lib.xma_rocm_scatter2scatter(
             _ptr(X), _rows(X, "X"), _ptr(W), w_es, ldw, w_is_kn, _ptr(idx), _ptr(offs),
             _ptr(out), 0 if out is None else _rows(out, "out"), _ptr(aux), 0 if aux is None else _rows(aux, "aux"),
-            _ptr(scale), M, N, K, W.size(0), fan_out, int(x_grouped), int(y_grouped), epilogue, _code(X), _stream(X),
+            _ptr(scale), M, N, K, W.size(0), fan_out, int(x_grouped), int(y_grouped), epilogue, _code(X),
+            _ptr(workspace), ws_bytes, _stream(X),
         ),
         "xma_rocm_scatter2scatter",
     )

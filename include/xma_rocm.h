@@ -100,12 +100,18 @@ XMA_API int xma_rocm_route(const void *ids, int ids_are_int64, int64_t n, int32_
  *   EPI_STORE       out (M, N)
  *   EPI_SWIGLU      out (M, N) = z or NULL;  aux (M, N/2) = h
  *   EPI_SWIGLU_BWD  aux (M, 2N) = z (read, grouped order);  out (M, 2N) = dz;  requires y_grouped
+ * workspace (may be NULL): xma_rocm_scatter2scatter_workspace_bytes(M, N, K, E) bytes of scratch, 0 for launches of
+ * many rounds of tiles.  With it the tiles of the last, partial round (the workgroups that would run while most
+ * compute units idle) are split along K over the idle units and summed by a second kernel, in a fixed order: the
+ * result does not depend on timing.  Without it every tile is computed by one workgroup.
  */
+XMA_API size_t xma_rocm_scatter2scatter_workspace_bytes(int64_t M, int32_t N, int32_t K, int32_t num_experts);
 XMA_API int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *W, int64_t w_expert_stride, int64_t ldw,
                              int w_is_kn, const int64_t *sorted_scattered_idxs, const int64_t *expert_offsets,
                              void *out, int64_t ldo, void *aux, int64_t ldaux, const void *row_scale, int64_t M,
                              int32_t N, int32_t K, int32_t num_experts, int32_t fan_out, int x_grouped,
-                             int y_grouped, int epilogue, int dtype, void *stream);
+                             int y_grouped, int epilogue, int dtype, void *workspace,
+                             size_t workspace_bytes, void *stream);
 
 /*
  * Weight gradient of a grouped linear: for every expert e

@@ -92,6 +92,14 @@ def test_moe_many_tokens_ragged(dtype, act_name):
     _run_case(dtype, 2048, 4, 1, 128, 256, act_name)
 
 
+@pytest.mark.parametrize("act_name", ["swiglu_packed", "gelu"])
+def test_moe_tiles_split_along_k(act_name):
+    """Few tiles and a long K: the tiles of the only (partial) round are cut into K slices that a second kernel adds
+    up, in all three epilogues (up-projection K = H, dX2 K = H, down-projection K = I, dX1 K = 2 I)."""
+    _run_case(torch.bfloat16, 64, 2, 1, 1024, 1536, act_name)
+    _run_case(torch.float16, 300, 3, 2, 2048, 512, act_name, skew=1.0)
+
+
 def test_moe_plumbing_config_shape():
     """BASELINE configs[0] shape (T=512, H=256, I=512, E=8, top-2, SwiGLU, weights N(0, 0.02)) in bf16."""
     _run_case(torch.bfloat16, 512, 8, 2, 256, 512, "swiglu_packed", seed=0)

@@ -32,6 +32,8 @@ CASES = [
     (700, 8, 2, 256, 512, 1.5, (3,)),
     (1024, 2, 1, 64, 264, 0.0, ()),
     (513, 6, 4, 72, 40, 2.0, (0, 5)),
+    (100, 2, 1, 96, 136, 0.0, ()),  # about 50 rows per expert: two of a wave's four row blocks are computed
+    (300, 3, 2, 1096, 320, 0.0, ()),  # few tiles, long K (with a tail): tiles are split into K slices
 ]
 
 

@@ -49,7 +49,7 @@ def test_argument_errors_are_reported_before_any_launch():
     assert lib.xma_rocm_combine(None, 8, None, None, 8, 4, 2, 12, 0, None) == -1  # H % 8 != 0
     assert lib.xma_rocm_combine(None, 8, None, None, 8, 4, 2, 16, 7, None) == -2  # dtype
     rc = lib.xma_rocm_scatter2scatter(None, 64, None, 64 * 64, 64, 0, None, None, None, 64, None, 0, None, 16, 60, 64, 2, 1, 1, 1,
-                                      0, 0, None)
+                                      0, 0, None, 0, None)
     assert rc == -2 and b"multiples of 8" in lib.xma_rocm_last_error()
     # empty problems are accepted without touching a pointer
     assert lib.xma_rocm_combine(None, 8, None, None, 8, 0, 2, 16, 0, None) == 0
