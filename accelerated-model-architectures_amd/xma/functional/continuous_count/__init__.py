@@ -31,12 +31,10 @@ def continuous_count(x: torch.Tensor, bins: int, *, kernel_backend: KernelBacken
         assert kernel_backend.verify_accelerator()
 
     if kernel_backend == KernelBackend.rocm:
-        from ...rocm.ops import continuous_count_rocm, continuous_count_workspace_elements
+        from ...rocm.ops import continuous_count_rocm
 
         y = torch.zeros(bins, dtype=torch.uint32, device=x.device)
-        ws = continuous_count_workspace_elements(x.numel(), bins)
-        workspace = torch.empty(ws, dtype=torch.int32, device=x.device) if ws else None
-        continuous_count_rocm(x=x.contiguous(), y=y, workspace=workspace)
+        continuous_count_rocm(x=x.contiguous(), y=y, workspace=None)
     elif kernel_backend == KernelBackend.torch:
         y = x.bincount(minlength=bins).to(torch.uint32)
     else:

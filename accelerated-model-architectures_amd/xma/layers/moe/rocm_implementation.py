@@ -36,8 +36,7 @@ def route(selected_experts: torch.Tensor, num_experts: int):
     excl = torch.empty(num_experts, dtype=torch.int64, device=dev)
     sorted_expert_idxs = torch.empty_like(ids)
     sorted_scattered_idxs = torch.empty(n, dtype=torch.int64, device=dev)
-    workspace = torch.empty(ops.route_workspace_elements(n, num_experts), dtype=torch.int32, device=dev)
-    ops.route_rocm(ids, counts, incl, excl, sorted_expert_idxs, sorted_scattered_idxs, workspace)
+    ops.route_rocm(ids, counts, incl, excl, sorted_expert_idxs, sorted_scattered_idxs, None)
     return counts, incl, excl, sorted_expert_idxs, sorted_scattered_idxs
 
 

@@ -62,12 +62,16 @@ def continuous_count_workspace_elements(n: int, bins: int) -> int:
 def continuous_count_rocm(x: torch.Tensor, y: torch.Tensor, workspace: torch.Tensor | None) -> None:
     """y (uint32, zero-filled by the caller) += histogram of x
     (reference op: _continuous_count_cuda, continuous_count/cuda_implementation.py:171-197).  `workspace` (int32, from
-    continuous_count_workspace_elements) lets large inputs take the two-pass path."""
+    continuous_count_workspace_elements; None: taken from torch's allocator inside the op) lets large inputs take the
+    two-pass path."""
     assert x.is_cuda and y.is_cuda and x.dim() == 1 and x.is_contiguous() and y.is_contiguous()
     assert x.dtype in (torch.int32, torch.int64) and y.dtype == torch.uint32
-    if workspace is not None:
-        assert workspace.dtype == torch.int32 and workspace.is_contiguous() and workspace.is_cuda
     lib = get_library()
+    if workspace is None:  # allocated here, inside the op, so that a traced caller never sees the size query
+        ws = continuous_count_workspace_elements(x.numel(), y.numel())
+        workspace = torch.empty(ws, dtype=torch.int32, device=x.device) if ws else None
+    else:
+        assert workspace.dtype == torch.int32 and workspace.is_contiguous() and workspace.is_cuda
     check(
         lib.xma_rocm_continuous_count(
             _ptr(x), int(x.dtype == torch.int64), x.numel(), _ptr(y), y.numel(), _ptr(workspace),
@@ -93,7 +97,7 @@ def route_rocm(
     offsets_exclusive: torch.Tensor,
     sorted_expert_idxs: torch.Tensor,
     sorted_scattered_idxs: torch.Tensor,
-    workspace: torch.Tensor,
+    workspace: torch.Tensor | None,
 ) -> None:
     """counts / offsets / stable expert-major permutation of ``ids`` in one op
     (replaces sort + continuous_count + cumsum, moe/__init__.py:210-217)."""
@@ -103,8 +107,10 @@ def route_rocm(
     assert offsets_inclusive.numel() == E and offsets_exclusive.numel() == E
     assert sorted_expert_idxs.dtype == ids.dtype and sorted_expert_idxs.numel() == ids.numel()
     assert sorted_scattered_idxs.dtype == torch.int64 and sorted_scattered_idxs.numel() == ids.numel()
-    assert workspace.dtype == torch.int32 and workspace.is_contiguous()
     lib = get_library()
+    if workspace is None:  # allocated here, inside the op, so that a traced caller never sees the size query
+        workspace = torch.empty(route_workspace_elements(ids.numel(), E), dtype=torch.int32, device=ids.device)
+    assert workspace.dtype == torch.int32 and workspace.is_contiguous()
     check(
         lib.xma_rocm_route(
             _ptr(ids), int(ids.dtype == torch.int64), ids.numel(), E, _ptr(counts), _ptr(offsets_inclusive),

@@ -1,0 +1,102 @@
+"""The rocm path under torch.compile(fullgraph=True) and under HIP graph capture.
+
+The reference runs every op eager and compiled (tests/layers/moe_test.py:104-105 wraps the module in
+torch.compile(fullgraph=True)); its ops are traceable because they are registered custom ops that mutate
+caller-allocated outputs (xma/custom_op.py:72-108).  The same must hold here, and since the tile schedule is
+derived on the device from the offsets, a whole step must also be capturable in a graph and replayable."""
+
+import pytest
+import torch
+
+from tests.utils import nerr
+
+pytestmark = pytest.mark.gpu
+
+
+def _make(T=300, E=8, k=2, H=256, I=512, dtype=torch.bfloat16, seed=0):
+    from xma import set_seed
+    from xma.functional import swiglu_packed
+    from xma.layers import MoE
+
+    set_seed(seed)
+    moe = MoE(E, k, H, I, swiglu_packed, True, add_bias=False, std=0.02).to(dtype).cuda()
+    x = torch.randn(T, H, device="cuda").to(dtype)
+    return moe, x
+
+
+def test_compiled_module_matches_eager():
+    from xma import KernelBackend
+
+    moe, x = _make()
+    print("compile: eager run", flush=True)
+    xe = x.clone().requires_grad_()
+    ye, _ = moe(xe, kernel_backend=KernelBackend.rocm)
+    ye.sum().backward()
+    want = {"y": ye.detach().clone(), "dx": xe.grad.clone(), "dw_fc": moe.c_fc.weight.grad.clone(),
+            "dw_proj": moe.c_proj.weight.grad.clone(), "dgate": moe.gate.weight.grad.clone()}
+    for p in moe.parameters():
+        p.grad = None
+    print("compile: compiled run (fullgraph)", flush=True)
+    cmoe = torch.compile(moe, fullgraph=True, backend="aot_eager")
+    xc = x.clone().requires_grad_()
+    yc, _ = cmoe(xc, kernel_backend=KernelBackend.rocm)
+    yc.sum().backward()
+    torch.cuda.synchronize()
+    got = {"y": yc, "dx": xc.grad, "dw_fc": moe.c_fc.weight.grad, "dw_proj": moe.c_proj.weight.grad,
+           "dgate": moe.gate.weight.grad}
+    for name in want:
+        # same kernels on the same inputs: bit-identical
+        assert torch.equal(got[name], want[name]), name
+
+
+def test_graph_capture_and_replay():
+    """fwd + bwd of the expert computation captured once and replayed on new inputs (new routing included); every
+    replay is checked against an eager run, with eager work and synchronisations in between."""
+    from xma import KernelBackend
+
+    E, k = 8, 2
+    moe, x = _make(E=E, k=k)
+    T, H = x.shape
+    g = torch.Generator(device="cuda").manual_seed(1)
+
+    def inputs():
+        logits = torch.randn(T, E, device="cuda", generator=g)
+        vals, sel = logits.topk(k, dim=-1)
+        rw = torch.softmax(vals, dim=-1).to(x.dtype)
+        xx = torch.randn(T, H, device="cuda", generator=g).to(x.dtype)
+        gy = torch.randn(T, H, device="cuda", generator=g).to(x.dtype)
+        return xx, rw, sel, gy
+
+    def step(xx, rw, sel, gy):
+        xx = xx.detach().requires_grad_()
+        rw = rw.detach().requires_grad_()
+        for p in (moe.c_fc.weight, moe.c_proj.weight):
+            p.grad = None
+        y = moe._compute_experts(xx, rw, sel, kernel_backend=KernelBackend.rocm)
+        y.backward(gy)
+        return y.detach(), xx.grad, rw.grad, moe.c_fc.weight.grad, moe.c_proj.weight.grad
+
+    sx, srw, ssel, sgy = inputs()
+    print("graph: warm-up on a side stream", flush=True)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step(sx, srw, ssel, sgy)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    print("graph: capture", flush=True)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = step(sx, srw, ssel, sgy)
+    for it in range(3):
+        nx, nrw, nsel, ngy = inputs()
+        print(f"graph: replay {it}", flush=True)
+        sx.copy_(nx), srw.copy_(nrw), ssel.copy_(nsel), sgy.copy_(ngy)
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [o.clone() for o in outs]
+        want = step(nx, nrw, nsel, ngy)  # eager, same kernels
+        torch.cuda.synchronize()
+        for a, b, name in zip(got, want, ("y", "dx", "d_router_weights", "dw_fc", "dw_proj")):
+            assert torch.equal(a, b), f"replay {it}: {name} differs, nerr {nerr(a, b):.2e}"
