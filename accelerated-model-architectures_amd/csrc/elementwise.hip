@@ -2,6 +2,7 @@
 // weight gradient), the gather copy `group`, and stand-alone packed SwiGLU.
 // All move 16 bytes per lane per access and accumulate in fp32.
 #include "common.hpp"
+#include "fp32.hpp"
 
 namespace {
 
@@ -150,13 +151,14 @@ inline int grid_for(int64_t work) { return (int)((work + EW_THREADS - 1) / EW_TH
 
 extern "C" int xma_rocm_combine(const void *expert_out, int64_t ld_in, const void *w, void *y, int64_t ldy, int64_t T,
                                 int32_t k, int32_t H, int dtype, void *stream) {
-    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED, "combine: dtype %d", dtype);
+    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16 || dtype == XMA_ROCM_F32, XMA_ROCM_EUNSUPPORTED, "combine: dtype %d", dtype);
     XMA_REQUIRE(T >= 0 && k >= 1 && H >= 8 && H % 8 == 0 && ld_in % 8 == 0 && ldy % 8 == 0, XMA_ROCM_EINVAL,
                 "combine: T=%lld k=%d H=%d ld_in=%lld ldy=%lld (H, ld %% 8 == 0)", (long long)T, k, H, (long long)ld_in,
                 (long long)ldy);
     XMA_REQUIRE(T == 0 || (expert_out && y && aligned16(expert_out) && aligned16(y)), XMA_ROCM_EINVAL,
                 "combine: null or misaligned pointer");
     if (T == 0) return XMA_ROCM_OK;
+    if (dtype == XMA_ROCM_F32) return f32_combine(expert_out, ld_in, w, y, ldy, T, k, H, (hipStream_t)stream);
     const int cpr = H / 8;
     XMA_REQUIRE(T * cpr < ((int64_t)1 << 31) * EW_THREADS, XMA_ROCM_EUNSUPPORTED, "combine: too large");
     hipStream_t st = (hipStream_t)stream;
@@ -167,12 +169,13 @@ extern "C" int xma_rocm_combine(const void *expert_out, int64_t ld_in, const voi
 
 extern "C" int xma_rocm_combine_bwd(const void *expert_out, int64_t ld_in, const void *dy, int64_t lddy, void *d_w,
                                     int64_t T, int32_t k, int32_t H, int dtype, void *stream) {
-    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED, "combine_bwd: dtype %d", dtype);
+    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16 || dtype == XMA_ROCM_F32, XMA_ROCM_EUNSUPPORTED, "combine_bwd: dtype %d", dtype);
     XMA_REQUIRE(T >= 0 && k >= 1 && H >= 8 && H % 8 == 0 && ld_in % 8 == 0 && lddy % 8 == 0, XMA_ROCM_EINVAL,
                 "combine_bwd: T=%lld k=%d H=%d", (long long)T, k, H);
     XMA_REQUIRE(T == 0 || (expert_out && dy && d_w && aligned16(expert_out) && aligned16(dy)), XMA_ROCM_EINVAL,
                 "combine_bwd: null or misaligned pointer");
     if (T == 0) return XMA_ROCM_OK;
+    if (dtype == XMA_ROCM_F32) return f32_combine_bwd(expert_out, ld_in, dy, lddy, d_w, T, k, H, (hipStream_t)stream);
     const int64_t rows = T * k;
     const int64_t blocks = (rows + (EW_THREADS / WAVE) - 1) / (EW_THREADS / WAVE);
     XMA_REQUIRE(blocks < ((int64_t)1 << 31), XMA_ROCM_EUNSUPPORTED, "combine_bwd: too large");
@@ -184,12 +187,13 @@ extern "C" int xma_rocm_combine_bwd(const void *expert_out, int64_t ld_in, const
 
 extern "C" int xma_rocm_group(const void *A, int64_t lda, const int64_t *idx, void *out, int64_t ldo, const void *coeff,
                               int64_t M, int32_t K, int32_t fan_out, int dtype, void *stream) {
-    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED, "group: dtype %d", dtype);
+    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16 || dtype == XMA_ROCM_F32, XMA_ROCM_EUNSUPPORTED, "group: dtype %d", dtype);
     XMA_REQUIRE(M >= 0 && K >= 8 && K % 8 == 0 && lda % 8 == 0 && ldo % 8 == 0 && fan_out >= 1, XMA_ROCM_EINVAL,
                 "group: M=%lld K=%d fan_out=%d", (long long)M, K, fan_out);
     XMA_REQUIRE(M == 0 || (A && idx && out && aligned16(A) && aligned16(out)), XMA_ROCM_EINVAL,
                 "group: null or misaligned pointer");
     if (M == 0) return XMA_ROCM_OK;
+    if (dtype == XMA_ROCM_F32) return f32_group(A, lda, idx, out, ldo, coeff, M, K, fan_out, (hipStream_t)stream);
     const int cpr = K / 8;
     hipStream_t st = (hipStream_t)stream;
     DISPATCH_T(dtype, (group_kernel<ET><<<grid_for(M * cpr), EW_THREADS, 0, st>>>(
@@ -199,12 +203,13 @@ extern "C" int xma_rocm_group(const void *A, int64_t lda, const int64_t *idx, vo
 
 extern "C" int xma_rocm_swiglu_packed_forward(const void *x, int64_t ldx, void *y, int64_t ldy, int64_t rows,
                                               int32_t cols_out, int dtype, void *stream) {
-    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED, "swiglu_packed: dtype %d", dtype);
+    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16 || dtype == XMA_ROCM_F32, XMA_ROCM_EUNSUPPORTED, "swiglu_packed: dtype %d", dtype);
     XMA_REQUIRE(rows >= 0 && cols_out >= 8 && cols_out % 8 == 0 && ldx % 8 == 0 && ldy % 8 == 0, XMA_ROCM_EINVAL,
                 "swiglu_packed: rows=%lld cols_out=%d (cols_out %% 8 == 0)", (long long)rows, cols_out);
     XMA_REQUIRE(rows == 0 || (x && y && aligned16(x) && aligned16(y)), XMA_ROCM_EINVAL,
                 "swiglu_packed: null or misaligned pointer");
     if (rows == 0) return XMA_ROCM_OK;
+    if (dtype == XMA_ROCM_F32) return f32_swiglu_packed_forward(x, ldx, y, ldy, rows, cols_out, (hipStream_t)stream);
     const int cpr = cols_out / 8;
     hipStream_t st = (hipStream_t)stream;
     DISPATCH_T(dtype, (swiglu_packed_fwd_kernel<ET><<<grid_for(rows * cpr), EW_THREADS, 0, st>>>(
@@ -214,13 +219,14 @@ extern "C" int xma_rocm_swiglu_packed_forward(const void *x, int64_t ldx, void *
 
 extern "C" int xma_rocm_swiglu_packed_backward(const void *x, int64_t ldx, const void *dy, int64_t lddy, void *dx,
                                                int64_t lddx, int64_t rows, int32_t cols_out, int dtype, void *stream) {
-    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED, "swiglu_packed_bwd: dtype %d",
+    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16 || dtype == XMA_ROCM_F32, XMA_ROCM_EUNSUPPORTED, "swiglu_packed_bwd: dtype %d",
                 dtype);
     XMA_REQUIRE(rows >= 0 && cols_out >= 8 && cols_out % 8 == 0 && ldx % 8 == 0 && lddy % 8 == 0 && lddx % 8 == 0,
                 XMA_ROCM_EINVAL, "swiglu_packed_bwd: rows=%lld cols_out=%d", (long long)rows, cols_out);
     XMA_REQUIRE(rows == 0 || (x && dy && dx && aligned16(x) && aligned16(dy) && aligned16(dx)), XMA_ROCM_EINVAL,
                 "swiglu_packed_bwd: null or misaligned pointer");
     if (rows == 0) return XMA_ROCM_OK;
+    if (dtype == XMA_ROCM_F32) return f32_swiglu_packed_backward(x, ldx, dy, lddy, dx, lddx, rows, cols_out, (hipStream_t)stream);
     const int cpr = cols_out / 8;
     hipStream_t st = (hipStream_t)stream;
     DISPATCH_T(dtype, (swiglu_packed_bwd_kernel<ET><<<grid_for(rows * cpr), EW_THREADS, 0, st>>>(

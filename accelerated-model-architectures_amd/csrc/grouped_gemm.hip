@@ -31,6 +31,7 @@
 //
 // Tiles never straddle experts: the schedule is expert-major, derived on the device from the inclusive expert
 // offsets in each workgroup's prologue (no host read of the counts).
+#include "fp32.hpp"
 #include "gemm_common.hpp"
 
 namespace xma_rocm {
@@ -920,7 +921,8 @@ extern "C" int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *
                                         const void *row_scale, int64_t M, int32_t N, int32_t K, int32_t E,
                                         int32_t fan_out, int x_grouped, int y_grouped, int epilogue, int dtype,
                                         void *workspace, size_t workspace_bytes, void *stream) {
-    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED, "scatter2scatter: dtype %d", dtype);
+    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16 || dtype == XMA_ROCM_F32, XMA_ROCM_EUNSUPPORTED,
+                "scatter2scatter: dtype %d", dtype);
     XMA_REQUIRE(epilogue >= XMA_ROCM_EPI_STORE && epilogue <= XMA_ROCM_EPI_SWIGLU_BWD, XMA_ROCM_EINVAL,
                 "scatter2scatter: epilogue %d", epilogue);
     XMA_REQUIRE(M >= 0 && M < ((int64_t)1 << 31) && N >= 8 && K >= 8 && E >= 1 && fan_out >= 1, XMA_ROCM_EINVAL,
@@ -964,6 +966,10 @@ extern "C" int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *
     a.fan_out = fan_out;
     a.x_grouped = x_grouped;
     a.y_grouped = y_grouped;
+    a.partial = nullptr;
+    a.split_cus = 0;
+    a.grid_main = 0;
+    if (dtype == XMA_ROCM_F32) return f32_scatter2scatter(a, w_is_kn ? 1 : 0, epilogue, (hipStream_t)stream);
     const int64_t NT = (N + BN - 1) / BN;
     const int64_t max_m_tiles = M / BM + E; // sum_e ceil(c_e / BM) <= floor(M / BM) + E
     const int64_t grid = max_m_tiles * NT;
@@ -994,7 +1000,8 @@ extern "C" int xma_rocm_group_bwd_W(const void *DY, int64_t lddy, int dy_grouped
                                     const int64_t *sorted_scattered_idxs, const int64_t *expert_offsets, void *DW,
                                     int64_t dw_expert_stride, int64_t lddw, int32_t N_out, int32_t K_in, int32_t E,
                                     int dtype, void *stream) {
-    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED, "group_bwd_W: dtype %d", dtype);
+    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16 || dtype == XMA_ROCM_F32, XMA_ROCM_EUNSUPPORTED,
+                "group_bwd_W: dtype %d", dtype);
     XMA_REQUIRE(N_out >= 8 && K_in >= 8 && E >= 1 && dy_fan_out >= 1 && x_fan_out >= 1, XMA_ROCM_EINVAL,
                 "group_bwd_W: N_out=%d K_in=%d E=%d", N_out, K_in, E);
     XMA_REQUIRE(N_out % 8 == 0 && K_in % 8 == 0 && lddy % 8 == 0 && ldx % 8 == 0 && lddw % 8 == 0 &&
@@ -1030,6 +1037,7 @@ extern "C" int xma_rocm_group_bwd_W(const void *DY, int64_t lddy, int dy_grouped
     hipStream_t st = (hipStream_t)stream;
     a.dy_div = make_fastdiv((uint32_t)dy_fan_out);
     a.x_div = make_fastdiv((uint32_t)x_fan_out);
+    if (dtype == XMA_ROCM_F32) return f32_group_bwd_W(a, st);
     if (dy_scale) return launch_dw_scaled(a, dtype, (int)grid, st);
     if (dtype == XMA_ROCM_BF16) return dispatch_dw<__bf16>(a, (int)grid, st);
     return dispatch_dw<_Float16>(a, (int)grid, st);

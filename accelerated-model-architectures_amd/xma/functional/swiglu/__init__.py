@@ -73,10 +73,10 @@ def swiglu_packed(x: torch.Tensor, *, kernel_backend: KernelBackend | None = Non
 
     kernel_backend = _resolve(kernel_backend, x)
     if kernel_backend == KernelBackend.rocm:
-        if x.dtype not in (torch.bfloat16, torch.float16) or H % 8 != 0:
+        if x.dtype not in (torch.bfloat16, torch.float16, torch.float32) or H % 8 != 0:
             raise NotImplementedError(
-                f"swiglu_packed on KernelBackend.rocm covers bf16/fp16 with an output width that is a multiple of 8 "
-                f"(got {x.dtype}, {H})"
+                f"swiglu_packed on KernelBackend.rocm covers bf16/fp16/fp32 with an output width that is a multiple of "
+                f"8 (got {x.dtype}, {H})"
             )
         y = _SwigluPackedROCm.apply(x.flatten(0, -2))
     elif kernel_backend == KernelBackend.torch:

@@ -16,7 +16,7 @@ import torch
 from .loader import check, get_library
 
 
-_DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1}
+_DTYPE_CODE = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
 
 EPI_STORE, EPI_SWIGLU, EPI_SWIGLU_BWD = 0, 1, 2
 
@@ -31,7 +31,7 @@ def _ptr(t: torch.Tensor | None) -> int | None:
 
 def _code(t: torch.Tensor) -> int:
     if t.dtype not in _DTYPE_CODE:
-        raise NotImplementedError(f"KernelBackend.rocm covers bfloat16 and float16, got {t.dtype}")
+        raise NotImplementedError(f"KernelBackend.rocm covers bfloat16, float16 and float32, got {t.dtype}")
     return _DTYPE_CODE[t.dtype]
 
 

@@ -12,7 +12,7 @@
  *     detected before anything is launched; launch errors come from
  *     hipGetLastError right after the launch); xma_rocm_last_error() gives the
  *     message of the calling thread's last failure;
- *   - `dtype` is XMA_ROCM_BF16 or XMA_ROCM_F16 (fp32 accumulation in both);
+ *   - `dtype` is XMA_ROCM_BF16, XMA_ROCM_F16 or XMA_ROCM_F32 (fp32 accumulation in all);
  *   - leading dimensions (ld*) and expert strides are in ELEMENTS;
  *   - "grouped" order = position n in the expert-sorted list; "scattered" order
  *     = row sorted_scattered_idxs[n] of the flattened (T, k) selection.
@@ -42,6 +42,7 @@ extern "C" {
 
 #define XMA_ROCM_BF16 0
 #define XMA_ROCM_F16 1
+#define XMA_ROCM_F32 2 /* exact fp32 kernels (v_mfma_f32_32x32x2_f32): parity runs and the fp32 points of the reference's test grid */
 
 /* epilogues of xma_rocm_scatter2scatter */
 #define XMA_ROCM_EPI_STORE 0      /* out = acc (optionally * row_scale) */

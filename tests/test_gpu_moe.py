@@ -16,6 +16,7 @@ from tests.utils import nerr
 pytestmark = pytest.mark.gpu
 
 TOL = 1e-2
+TOL_F32 = 5e-5  # fp32 kernels against the fp32 oracle: summation order and exp/rcp approximations only
 
 
 def _act(name):
@@ -61,13 +62,13 @@ def _run_case(dtype, T, E, k, H, I, act_name, skew=0.0, empty=(), seed=42):
         assert torch.isfinite(g).all(), name
         e = nerr(g, w)
         print(f"   {name}: nerr={e:.2e}", flush=True)
-        assert e <= TOL, f"{name}: {e}"
+        assert e <= (TOL_F32 if dtype == torch.float32 else TOL), f"{name}: {e}"
     # experts without tokens: zero weight gradient slices
     for e in empty:
         assert (moe.c_fc.weight.grad[e] == 0).all() and (moe.c_proj.weight.grad[e] == 0).all()
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("E", [2, 4, 6, 8])
 @pytest.mark.parametrize("k", [2, 4])
 @pytest.mark.parametrize("act_name", ["swiglu_packed", "glu", "gelu"])
@@ -101,8 +102,15 @@ def test_moe_tiles_split_along_k(act_name):
 
 
 def test_moe_plumbing_config_shape():
-    """BASELINE configs[0] shape (T=512, H=256, I=512, E=8, top-2, SwiGLU, weights N(0, 0.02)) in bf16."""
+    """BASELINE configs[0] (T=512, H=256, I=512, E=8, top-2, SwiGLU, weights N(0, 0.02)) in fp32, as stated, and bf16."""
+    _run_case(torch.float32, 512, 8, 2, 256, 512, "swiglu_packed", seed=0)
     _run_case(torch.bfloat16, 512, 8, 2, 256, 512, "swiglu_packed", seed=0)
+
+
+@pytest.mark.parametrize("act_name", ["swiglu_packed", "gelu"])
+def test_moe_fp32_ragged(act_name):
+    _run_case(torch.float32, 777, 16, 4, 264, 136, act_name, skew=2.0, empty=(0, 15))
+    _run_case(torch.float32, 300, 3, 2, 1024, 512, act_name, skew=1.0)
 
 
 def test_moe_forward_module_and_state_dict():

@@ -1,6 +1,6 @@
 """GPU parity of the MoE ops (grouped GEMMs, dW, group, combine) through the C ABI against the
 op-level oracle.  Tolerance: max-abs-normalised error <= 1e-2 for bf16/fp16 results with fp32
-accumulation (the bar of the north star); operands are bit-identical on both sides."""
+accumulation (the bar of the north star), <= 2e-5 for the fp32 kernels; operands are bit-identical on both sides."""
 
 import pytest
 import torch
@@ -11,6 +11,11 @@ from tests.utils import nerr
 pytestmark = pytest.mark.gpu
 
 TOL = 1e-2
+TOL_F32 = 2e-5  # fp32 kernels: fp32 operands and accumulators, only the summation order differs from the oracle's
+
+
+def _tol(dtype):
+    return TOL_F32 if dtype == torch.float32 else TOL
 
 
 def _routing(T, E, k, seed, skew=0.0, empty=()):
@@ -37,7 +42,7 @@ CASES = [
 ]
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("case", CASES)
 @pytest.mark.parametrize("w_kn", [False, True])
 @pytest.mark.parametrize("x_grouped,y_grouped", [(False, True), (True, False), (True, True), (False, False)])
@@ -63,10 +68,10 @@ def test_scatter2scatter(dtype, case, w_kn, x_grouped, y_grouped):
                           None if rs is None else rs.cuda())
         torch.cuda.synchronize()
         assert torch.isfinite(out).all()
-        assert nerr(out, want) <= TOL
+        assert nerr(out, want) <= _tol(dtype)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("case", CASES)
 def test_group_bwd_W(dtype, case):
     from xma.rocm import ops
@@ -92,18 +97,18 @@ def test_group_bwd_W(dtype, case):
 
     # both grouped (the reference op), x gathered (dW1), dy gathered and scaled (dW2)
     want = oracle.group_bwd_W(dy_grp, x_grp, offs, E)
-    assert nerr(run(dy_grp, x_grp, None, 0, 0), want) <= TOL
+    assert nerr(run(dy_grp, x_grp, None, 0, 0), want) <= _tol(dtype)
     want = oracle.group_bwd_W(dy_grp, oracle.group(x_tok, ss, None, k), offs, E)
-    assert nerr(run(dy_grp, x_tok, None, 0, k), want) <= TOL
+    assert nerr(run(dy_grp, x_tok, None, 0, k), want) <= _tol(dtype)
     want = oracle.group_bwd_W(oracle.group(dy_tok, ss, scale, k), x_grp, offs, E)
-    assert nerr(run(dy_tok, x_grp, scale, k, 0), want) <= TOL
+    assert nerr(run(dy_tok, x_grp, scale, k, 0), want) <= _tol(dtype)
     # experts without rows get an all-zero slice
     got = run(dy_grp, x_grp, None, 0, 0)
     for e in empty:
         assert (got[e] == 0).all()
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_group_and_combine(dtype):
     from xma.layers.moe import rocm_implementation as R
     from xma.rocm import ops
@@ -124,13 +129,13 @@ def test_group_and_combine(dtype):
         for ww in (None, w):
             y = torch.empty(T, H, dtype=dtype, device="cuda")
             ops.combine_rocm(eo.cuda(), None if ww is None else ww.cuda(), y, k)
-            assert nerr(y, oracle.combine(eo, ww, k)) <= TOL
+            assert nerr(y, oracle.combine(eo, ww, k)) <= _tol(dtype)
         d_w = torch.empty(T, k, dtype=dtype, device="cuda")
         ops.combine_bwd_rocm(eo.cuda(), dy.cuda(), d_w)
-        assert nerr(d_w, oracle.combine_bwd(eo, dy, k)) <= TOL
+        assert nerr(d_w, oracle.combine_bwd(eo, dy, k)) <= _tol(dtype)
 
 
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_swiglu_packed_standalone(dtype):
     from xma import KernelBackend
     from xma.functional import swiglu_packed
@@ -142,7 +147,7 @@ def test_swiglu_packed_standalone(dtype):
         xd = x.cuda().requires_grad_()
         y = swiglu_packed(xd, kernel_backend=KernelBackend.rocm)
         y.backward(dy.cuda())
-        assert nerr(y, oracle.swiglu_packed(x.float())) <= TOL
+        assert nerr(y, oracle.swiglu_packed(x.float())) <= _tol(dtype)
         dg, du = oracle.swiglu_backward(x[..., 0::2].float(), x[..., 1::2].float(), dy.float())
         want = torch.stack([dg, du], dim=-1).flatten(-2)
-        assert nerr(xd.grad, want) <= TOL
+        assert nerr(xd.grad, want) <= _tol(dtype)
