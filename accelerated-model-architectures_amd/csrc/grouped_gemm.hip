@@ -242,63 +242,92 @@ __device__ __forceinline__ bool locate_tile(const FwdArgs &a, unsigned char *sme
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int NT = (a.N + BN - 1) / BN;
-    int *s_pre = (int *)smem; // [E + 1], dead before the first tile load
-    if (tid == 0) s_sched[0] = -1;
-    if (wave == 0) {
-        int carry = 0;
-        for (int b = 0; b < a.E; b += WAVE) {
-            const int e = b + lane;
-            int v = 0;
-            if (e < a.E) {
-                const int64_t cnt = a.offs[e] - (e ? a.offs[e - 1] : 0);
-                v = (int)((cnt + BM - 1) / BM) * NT;
-            }
-            int s = v;
+    int full = 0, rest = 0, parts = 1, part = 0, L = 0;
+    // from the number of tiles: which one is this workgroup's (false: none)
+    auto pick = [&](int total) -> bool {
+        full = total;
+        if (a.partial) {
+            const int KT = (a.K + BK - 1) / BK;
+            full = total / a.split_cus * a.split_cus;
+            rest = total - full;
+            parts = rest ? a.split_cus / rest : 1;
+            if (parts > KT / SPLIT_MIN_STEPS) parts = KT / SPLIT_MIN_STEPS;
+            if (parts < 2) parts = 1, full = total, rest = 0;
+        }
+        const int b = (int)blockIdx.x;
+        if (ROLE == ROLE_FIXUP) {
+            if (b >= rest) return false;
+            L = full + b;
+        } else if (ROLE == ROLE_SLICES) {
+            if (rest == 0) return false;
+            const int q = xcd_remap(b, a.split_cus); // neighbouring tiles of one slice index meet in one XCD's L2
+            part = q / rest;
+            if (part >= parts) return false;
+            L = full + q % rest;
+        } else {
+            L = xcd_remap(b, a.grid_main);
+            if (L >= full) return false; // beyond the last tile (the grid is an upper bound), or a tile that is split
+        }
+        return true;
+    };
+    int e, local;
+    int64_t row_lo, row_hi;
+    if (a.E <= WAVE) {
+        // every wave scans the experts in registers: lane = expert; no LDS, no barrier, one load per lane
+        const int64_t hi = a.offs[lane < a.E ? lane : a.E - 1];
+        int64_t lo = __shfl_up(hi, 1);
+        if (lane == 0) lo = 0;
+        const int v = (int)((hi - lo + BM - 1) / BM) * NT; // 0 for the lanes past E
+        int s = v;
 #pragma unroll
-            for (int d = 1; d < WAVE; d <<= 1) {
-                const int t = __shfl_up(s, d);
-                if (lane >= d) s += t;
-            }
-            if (e < a.E) s_pre[e] = carry + s - v;
-            carry += __shfl(s, WAVE - 1);
+        for (int d = 1; d < WAVE; d <<= 1) {
+            const int t = __shfl_up(s, d);
+            if (lane >= d) s += t;
         }
-        if (lane == 0) s_pre[a.E] = carry;
-    }
-    __syncthreads();
-    const int total = __builtin_amdgcn_readfirstlane(s_pre[a.E]); // uniform: keep the whole schedule in scalar registers
-    int full = total, rest = 0, parts = 1;
-    if (a.partial) {
-        const int KT = (a.K + BK - 1) / BK;
-        full = total / a.split_cus * a.split_cus;
-        rest = total - full;
-        parts = rest ? a.split_cus / rest : 1;
-        if (parts > KT / SPLIT_MIN_STEPS) parts = KT / SPLIT_MIN_STEPS;
-        if (parts < 2) parts = 1, full = total, rest = 0;
-    }
-    int L, part = 0;
-    const int b = (int)blockIdx.x;
-    if (ROLE == ROLE_FIXUP) {
-        if (b >= rest) return false;
-        L = full + b;
-    } else if (ROLE == ROLE_SLICES) {
-        if (rest == 0) return false;
-        const int q = xcd_remap(b, a.split_cus); // neighbouring tiles of one slice index meet in one XCD's L2
-        part = q / rest;
-        if (part >= parts) return false;
-        L = full + q % rest;
+        if (!pick(__builtin_amdgcn_readlane(s, WAVE - 1))) return false;
+        const uint64_t hit = __ballot(s - v <= L && L < s); // exactly one lane
+        e = __builtin_ctzll(hit);
+        local = L - __builtin_amdgcn_readlane(s - v, e);
+        row_lo = ((int64_t)__builtin_amdgcn_readlane((int)(lo >> 32), e) << 32) |
+                 (uint32_t)__builtin_amdgcn_readlane((int)lo, e);
+        row_hi = ((int64_t)__builtin_amdgcn_readlane((int)(hi >> 32), e) << 32) |
+                 (uint32_t)__builtin_amdgcn_readlane((int)hi, e);
     } else {
-        L = xcd_remap(b, a.grid_main);
-        if (L >= full) return false; // beyond the last tile (the grid is an upper bound), or a tile that is split
-    }
-    for (int e = tid; e < a.E; e += GEMM_THREADS)
-        if (s_pre[e] <= L && L < s_pre[e + 1]) {
-            s_sched[0] = e;
-            s_sched[1] = L - s_pre[e];
+        int *s_pre = (int *)smem; // [E + 1], dead before the first tile load
+        if (wave == 0) {
+            int carry = 0;
+            for (int b = 0; b < a.E; b += WAVE) {
+                const int x = b + lane;
+                int v = 0;
+                if (x < a.E) {
+                    const int64_t cnt = a.offs[x] - (x ? a.offs[x - 1] : 0);
+                    v = (int)((cnt + BM - 1) / BM) * NT;
+                }
+                int s = v;
+#pragma unroll
+                for (int d = 1; d < WAVE; d <<= 1) {
+                    const int t = __shfl_up(s, d);
+                    if (lane >= d) s += t;
+                }
+                if (x < a.E) s_pre[x] = carry + s - v;
+                carry += __shfl(s, WAVE - 1);
+            }
+            if (lane == 0) s_pre[a.E] = carry;
         }
-    __syncthreads();
-    const int e = __builtin_amdgcn_readfirstlane(s_sched[0]);
-    const int local = __builtin_amdgcn_readfirstlane(s_sched[1]);
-    const int64_t row_lo = e ? a.offs[e - 1] : 0, row_hi = a.offs[e];
+        __syncthreads();
+        if (!pick(__builtin_amdgcn_readfirstlane(s_pre[a.E]))) return false;
+        for (int x = tid; x < a.E; x += GEMM_THREADS)
+            if (s_pre[x] <= L && L < s_pre[x + 1]) {
+                s_sched[0] = x;
+                s_sched[1] = L - s_pre[x];
+            }
+        __syncthreads();
+        e = __builtin_amdgcn_readfirstlane(s_sched[0]);
+        local = __builtin_amdgcn_readfirstlane(s_sched[1]);
+        row_lo = e ? a.offs[e - 1] : 0;
+        row_hi = a.offs[e];
+        __syncthreads(); // s_pre is dead from here on
+    }
     const int tiles_m = (int)((row_hi - row_lo + BM - 1) / BM);
     const int m_tile = local % tiles_m, n_tile = local / tiles_m;
     ts.e = e;
@@ -308,7 +337,6 @@ __device__ __forceinline__ bool locate_tile(const FwdArgs &a, unsigned char *sme
     ts.part = part;
     ts.parts = (L >= full) ? parts : 1;
     ts.tail_index = L - full;
-    __syncthreads(); // s_pre is dead from here on
     return true;
 }
 
@@ -504,23 +532,15 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
     const int kt0 = (ROLE == ROLE_SLICES) ? ((ts.part * KT / ts.parts) & ~1) : 0;
     const int kt1 = (ROLE == ROLE_SLICES && ts.part + 1 < ts.parts) ? (((ts.part + 1) * KT / ts.parts) & ~1) : KT;
     const uint16_t *q_ptr[8], *p_ptr[8];
+    const int c_lane = rowmajor_lane_chunk(lane);
     {
-        const int c = rowmajor_lane_chunk(lane);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            int r = wave * 64 + i * 8 + (lane >> 3);
-            if (r >= rows_valid) r = rows_valid - 1; // duplicates, masked at the store
-            const int64_t n = row0 + r;
-            const int64_t src = a.x_grouped ? n : a.idx[n] / a.fan_out;
-            q_ptr[i] = a.X + src * a.ldx + c * 8;
-        }
         const uint16_t *We = a.W + (int64_t)e * a.w_es;
         if (WT == 0) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 int r = n0 + wave * 64 + i * 8 + (lane >> 3);
                 if (r >= a.N) r = a.N - 1;
-                p_ptr[i] = We + (int64_t)r * a.ldw + c * 8;
+                p_ptr[i] = We + (int64_t)r * a.ldw + c_lane * 8;
             }
         } else {
             const int max_chunk = ((a.N - n0) >> 3) - 1; // last valid 16-byte chunk of the tile's column range
@@ -568,7 +588,18 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
     make_frag_base<0>(qb, lds0, wq, lane);
     make_frag_base<WT>(pb, lds0 + OP_CHUNKS * 16, wp, lane);
 
-    static_for<16>([&](auto P) { issue_piece(kt0, P, IC<0>{}); });
+    // The weight pieces of the first step go out before the activation rows are known: their addresses need only
+    // the schedule, while the rows of a gathered tile take another dependent load (the scattered index).
+    static_for<8>([&](auto P) { issue_piece(kt0, IC<8 + P.value>{}, IC<0>{}); });
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        int r = wave * 64 + i * 8 + (lane >> 3);
+        if (r >= rows_valid) r = rows_valid - 1; // duplicates, masked at the store
+        const int64_t n = row0 + r;
+        const int64_t src = a.x_grouped ? n : a.idx[n] / a.fan_out;
+        q_ptr[i] = a.X + src * a.ldx + c_lane * 8;
+    }
+    static_for<8>([&](auto P) { issue_piece(kt0, P, IC<0>{}); });
     static_for<DMA_N0>([&](auto P) { issue_piece(kt0 + 1, P, IC<0>{}); });
     // the first step has landed in every wave (the first loads of the second may be in flight)
     if (kt1 - kt0 > 1)
