@@ -158,25 +158,48 @@ __device__ __forceinline__ void load_frags(Frags &f, const FragBase<PTR> &pb, co
     });
 }
 
-// The 16 MFMAs of one k16 sub-step on `cur` as 8 pinned slots (NI < 4: only the first NI of the wave's four 32-wide Q
-// blocks hold valid rows; the MFMAs and fragment reads of the others are left out).  Slot g: two MFMAs; for g < 4 one P and one Q fragment
-// read of sub-step KK (of the stage pb/qb point at) into `nxt`; then `hook(IC<g>)`, which the callers use to issue one
-// LDS-DMA load per slot.  A wave issues in order, so anything not placed between MFMAs would leave the matrix pipe idle
-// for as long as it takes to issue; all fragment reads sit in the first half so that the second half covers their
-// latency.
+// The 16 MFMAs of one k16 sub-step on `cur` in pinned slots of MMA_GROUP MFMAs, each followed by its share of the other
+// instructions: the 8 fragment reads of sub-step KK (of the stage pb/qb point at) into `nxt` during the first half of
+// the sub-step, so that the second half covers their latency, and the 8 calls `hook(IC<0..7>)`, which the callers use
+// to issue one LDS-DMA or index load each.  A wave issues in order, so anything not placed between MFMAs would leave the
+// matrix pipe idle for as long as it takes to issue.  Pairs of MFMAs measured best in the kernels (single MFMAs 2-3 %
+// slower, although an isolated instruction-mix benchmark prefers them).  NI < 4: only the first NI of the wave's four
+// 32-wide Q blocks hold valid rows; the MFMAs and fragment reads of the others are left out.
+constexpr int MMA_GROUP = 2;
 template <typename T, int PTR, int QTR, int KK, int NI = 4, typename Hook>
 __device__ __forceinline__ void mma_step(Frags &cur, Frags &nxt, const FragBase<PTR> &pb, const FragBase<QTR> &qb,
                                          f32x16 (&acc)[4][4], Hook hook) {
     wait_frags(cur); // issued at least 8 MFMAs ago
-    static_for<8>([&](auto G) {
-        constexpr int g = G.value, j = g >> 1, i0 = (g & 1) * 2;
+    constexpr int SLOTS = 16 / MMA_GROUP;
+    static_for<SLOTS>([&](auto S) {
+        constexpr int t = S.value;
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (i0 < NI) acc[j][i0] = Elem<T>::mfma(cur.p[j], cur.q[i0], acc[j][i0]);
-        if constexpr (i0 + 1 < NI) acc[j][i0 + 1] = Elem<T>::mfma(cur.p[j], cur.q[i0 + 1], acc[j][i0 + 1]);
+        static_for<MMA_GROUP>([&](auto M) {
+            constexpr int m = t * MMA_GROUP + M.value, j = m >> 2, i = m & 3;
+            if constexpr (i < NI) acc[j][i] = Elem<T>::mfma(cur.p[j], cur.q[i], acc[j][i]);
+        });
         __builtin_amdgcn_sched_barrier(0);
-        if constexpr (g < 4 && NI > 0) nxt.p[g] = read_frag<PTR, g, KK>(pb);
-        if constexpr (g < NI) nxt.q[g] = read_frag<QTR, g, KK>(qb);
-        hook(G);
+        // fragment reads: 8 (4 P, 4 Q) over the first SLOTS / 2 slots
+        constexpr int RPS = 16 / SLOTS; // reads per slot of the first half
+        if constexpr (t < SLOTS / 2) {
+            static_for<RPS>([&](auto R) {
+                constexpr int r = t * RPS + R.value, f = r >> 1;
+                if constexpr ((r & 1) == 0) {
+                    if constexpr (NI > 0) nxt.p[f] = read_frag<PTR, f, KK>(pb);
+                } else {
+                    if constexpr (f < NI) nxt.q[f] = read_frag<QTR, f, KK>(qb);
+                }
+            });
+        }
+        // hooks: 8 over all slots (two per slot for groups of 4, every other slot for single MFMAs)
+        if constexpr (SLOTS == 4) {
+            hook(IC<2 * t>{});
+            hook(IC<2 * t + 1>{});
+        } else if constexpr (SLOTS == 8) {
+            hook(S);
+        } else if constexpr ((t & 1) == 1) {
+            hook(IC<t / 2>{});
+        }
     });
     __builtin_amdgcn_sched_barrier(0);
 }
@@ -566,7 +589,11 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
             if (kt >= kt1) return; // uniform
         }
         u32x4 *dst = tiles + (kt & 1) * STAGE_CHUNKS + slot + wave * 512; // a wave's 8 pieces are 8 KB apart per wave
-        const uint16_t *src = (piece < 8) ? q_ptr[piece] + (int64_t)kt * BK : p_ptr[piece - 8] + (int64_t)kt * p_step;
+        const uint16_t *src;
+        if constexpr (piece < 8)
+            src = q_ptr[piece] + (int64_t)kt * BK;
+        else
+            src = p_ptr[piece - 8] + (int64_t)kt * p_step;
         if constexpr (!FULL.value) {
             if (k_tail && kt == KT - 1) { // uniform branch, taken by at most one step of a tile
                 asm volatile("" ::: "memory"); // keeps this rare path a branch instead of selects in every piece
@@ -620,12 +647,17 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
         }
         // one K step; FULL: steps kt + 1 and kt + 2 exist and are complete
         auto k_step = [&](int kt, auto FULL) {
+            // The step numbers of the loads are made opaque: otherwise the compiler turns "pointer + kt * step" into 16
+            // running pointers and advances all of them with 64-bit vector adds in one lump at the end of the loop body,
+            // where nothing hides them.
+            int kt_a = kt + 1, kt_b = kt + 2;
+            asm volatile("" : "+s"(kt_a), "+s"(kt_b));
             // rest of the loads of step kt + 1 (the first DMA_N0 went out behind the previous barrier)
             mma_step<T, WT, 0, 1, NI>(f0, f1, pb, qb, acc, [&](auto G) {
-                if constexpr (G.value < DMA_N1) issue_piece(kt + 1, IC<DMA_N0 + G.value>{}, FULL);
+                if constexpr (G.value < DMA_N1) issue_piece(kt_a, IC<DMA_N0 + G.value>{}, FULL);
             });
             mma_step<T, WT, 0, 2, NI>(f1, f0, pb, qb, acc, [&](auto G) {
-                if constexpr (G.value < DMA_N2) issue_piece(kt + 1, IC<DMA_N0 + DMA_N1 + G.value>{}, FULL);
+                if constexpr (G.value < DMA_N2) issue_piece(kt_a, IC<DMA_N0 + DMA_N1 + G.value>{}, FULL);
             });
             mma_step<T, WT, 0, 3, NI>(f0, f1, pb, qb, acc, NoHook());
             XMA_WAIT_LOADS_AND_BARRIER(); // step kt + 1 has landed; nobody reads this stage any more
@@ -633,8 +665,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
             flip_stage(qb);
             // the stage just left is free: first loads of step kt + 2; fragments of sub-step 0 of step kt + 1
             mma_step<T, WT, 0, 0, NI>(f1, f0, pb, qb, acc, [&](auto G) {
-                if constexpr (G.value < DMA_N0) issue_piece(kt + 2, G, FULL);
-                if constexpr (G.value + 8 < DMA_N0) issue_piece(kt + 2, IC<G.value + 8>{}, FULL);
+                if constexpr (G.value < DMA_N0) issue_piece(kt_b, G, FULL);
+                if constexpr (G.value + 8 < DMA_N0) issue_piece(kt_b, IC<G.value + 8>{}, FULL);
             });
         };
         int kt = kt0;

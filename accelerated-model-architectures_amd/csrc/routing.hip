@@ -142,30 +142,40 @@ __global__ __launch_bounds__(ROUTE_THREADS) void route_unit_hist_kernel(const Id
     }
 }
 
+// inclusive scan of one value per thread over the workgroup: wave scans by shuffles, then the wave totals
+__device__ __forceinline__ uint32_t block_inclusive_scan(uint32_t v, uint32_t *s_wave /* [ROUTE_WAVES] */, int tid) {
+    const int lane = tid % WAVE, wave = tid / WAVE;
+    uint32_t s = v;
+#pragma unroll
+    for (int d = 1; d < WAVE; d <<= 1) {
+        const uint32_t t = __shfl_up(s, d);
+        if (lane >= d) s += t;
+    }
+    if (lane == WAVE - 1) s_wave[wave] = s;
+    __syncthreads();
+    uint32_t before = 0;
+#pragma unroll
+    for (int w = 0; w < ROUTE_WAVES; ++w)
+        if (w < wave) before += s_wave[w];
+    return s + before;
+}
+
 __global__ __launch_bounds__(ROUTE_THREADS) void route_scan_kernel(uint32_t *__restrict__ unit_hist, int64_t num_units,
                                                                    int E, uint32_t *__restrict__ counts) {
-    __shared__ uint32_t s_part[ROUTE_THREADS];
+    __shared__ uint32_t s_wave[ROUTE_WAVES];
     const int e = blockIdx.x, tid = threadIdx.x;
     const int64_t per = (num_units + ROUTE_THREADS - 1) / ROUTE_THREADS;
     const int64_t u0 = tid * per, u1 = (u0 + per < num_units) ? u0 + per : num_units;
     uint32_t sum = 0;
     for (int64_t u = u0; u < u1; ++u) sum += unit_hist[u * E + e];
-    s_part[tid] = sum;
-    __syncthreads();
-    // Hillis-Steele inclusive scan over the 256 partial sums
-    for (int d = 1; d < ROUTE_THREADS; d <<= 1) {
-        uint32_t v = (tid >= d) ? s_part[tid - d] : 0;
-        __syncthreads();
-        s_part[tid] += v;
-        __syncthreads();
-    }
-    uint32_t run = s_part[tid] - sum; // exclusive prefix of this thread's range
+    const uint32_t incl = block_inclusive_scan(sum, s_wave, tid);
+    uint32_t run = incl - sum; // exclusive prefix of this thread's range
     for (int64_t u = u0; u < u1; ++u) {
         uint32_t c = unit_hist[u * E + e];
         unit_hist[u * E + e] = run;
         run += c;
     }
-    if (tid == ROUTE_THREADS - 1) counts[e] = s_part[tid];
+    if (tid == ROUTE_THREADS - 1) counts[e] = incl;
 }
 
 template <typename IdT>
@@ -235,16 +245,9 @@ __global__ __launch_bounds__(ROUTE_THREADS) void route_scatter_kernel(
     uint32_t mine = 0;
     for (int e = e0; e < e1; ++e)
         for (int w = 0; w < ROUTE_WAVES; ++w) mine += s_ctr[w * E + e];
-    s_scan[tid] = mine;
-    __syncthreads();
-    for (int d = 1; d < ROUTE_THREADS; d <<= 1) {
-        const uint32_t v = (tid >= d) ? s_scan[tid - d] : 0;
-        __syncthreads();
-        s_scan[tid] += v;
-        __syncthreads();
-    }
-    const uint32_t total = s_scan[ROUTE_THREADS - 1]; // ids of this unit that are in range
-    uint32_t run = s_scan[tid] - mine;
+    const uint32_t incl = block_inclusive_scan(mine, s_scan, tid);
+    if (tid == ROUTE_THREADS - 1) s_scan[ROUTE_WAVES] = incl;
+    uint32_t run = incl - mine;
     for (int e = e0; e < e1; ++e) {
         s_gbase[e] -= run; // destination of local sorted position j of expert e = s_gbase[e] + j
         for (int w = 0; w < ROUTE_WAVES; ++w) {
@@ -254,6 +257,7 @@ __global__ __launch_bounds__(ROUTE_THREADS) void route_scatter_kernel(
         }
     }
     __syncthreads();
+    const uint32_t total = s_scan[ROUTE_WAVES]; // ids of this unit that are in range
 
     // phase 3: stable ranks, unit sorted into LDS.  ds_add_rtn_u32 applies the lanes of one wave instruction that hit
     // the same address in lane order (verified on gfx950 over 5e7 lane operations against the ballot formulation below,
