@@ -183,6 +183,9 @@ def run_moe(args, cfg, name):
         "unit": "TFLOP/s",
         "frac": round(gemms[dom]["tflops"] / PEAK_BF16_TFLOPS, 4),
         "traffic": MEASURED_TRAFFIC_BYTES.get(name) if dom.startswith("up_swiglu") else None,
+        # measured on this hardware: independent bf16 MFMAs alone, random operands, no memory traffic (power-limited clock);
+        # with all-zero operands the same stream reaches 2475
+        "mfma_only_random_operands_tflops": 1700.0,
         "all_gemms_tflops": round(total_flops / total_ms / 1e9, 1),
         "all_gemms_frac": round(total_flops / total_ms / 1e9 / PEAK_BF16_TFLOPS, 4),
     }
