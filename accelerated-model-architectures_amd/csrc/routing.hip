@@ -108,7 +108,7 @@ __global__ __launch_bounds__(HIST_THREADS) void histogram_global_kernel(const Id
 }
 
 // ------------------------------------------------------------------------------------------------
-// route: a unit is the ROUTE_CHUNK consecutive ids of one workgroup (4 waves x 1024).
+// route: a unit is the ROUTE_CHUNK consecutive ids of one workgroup (8 waves x 512).
 //   pass 1  unit_hist[u][e]               (LDS atomics)
 //   pass 2  block e: exclusive prefix over units of column e (in place) and counts[e]
 //   pass 3  per unit: per-wave counts -> local offsets; stable rank of every id inside its wave (64 ids per step,
@@ -116,10 +116,10 @@ __global__ __launch_bounds__(HIST_THREADS) void histogram_global_kernel(const Id
 //           order; XMA_ROUTE_BALLOT_RANKS selects ranks from log2(E) ballots instead); the unit is sorted into LDS
 //           and leaves as one contiguous run per expert.
 // ------------------------------------------------------------------------------------------------
-constexpr int ROUTE_THREADS = 256;
+constexpr int ROUTE_THREADS = 512;
 constexpr int ROUTE_WAVES = ROUTE_THREADS / WAVE;
-constexpr int ROUTE_WAVE_IDS = 1024;
-constexpr int ROUTE_STEPS = ROUTE_WAVE_IDS / WAVE;          // 16 ids per lane
+constexpr int ROUTE_WAVE_IDS = 512;
+constexpr int ROUTE_STEPS = ROUTE_WAVE_IDS / WAVE;          // 8 ids per lane
 constexpr int ROUTE_CHUNK = ROUTE_WAVES * ROUTE_WAVE_IDS;   // 4096 ids per workgroup
 constexpr int ROUTE_MAX_E = 2048;
 
