@@ -233,9 +233,23 @@ __global__ __launch_bounds__(ROUTE_THREADS) void route_scatter_kernel(
         }
         key[s] = k;
     }
+    // Counting and ranking in one pass: ds_add_rtn_u32 applies the lanes of one wave instruction that hit the same
+    // address in lane order (verified on gfx950 over 5e7 lane operations against the ballot formulation below, and by
+    // the bit-exact stability tests), and a wave's LDS instructions execute in program order, so the value returned
+    // from the wave-private counter is the stable rank of the id among the wave's ids of the same expert, and the
+    // counter ends up as their number.  XMA_ROUTE_BALLOT_RANKS selects the formulation that does not rely on that.
+#ifndef XMA_ROUTE_BALLOT_RANKS
+    uint32_t rank[ROUTE_STEPS];
+#pragma unroll
+    for (int s = 0; s < ROUTE_STEPS; ++s) {
+        rank[s] = 0;
+        if (key[s] != 0xffffffffu) rank[s] = atomicAdd(&my_ctr[key[s]], 1u);
+    }
+#else
 #pragma unroll
     for (int s = 0; s < ROUTE_STEPS; ++s)
         if (key[s] != 0xffffffffu) atomicAdd(&my_ctr[key[s]], 1u);
+#endif
     __syncthreads();
 
     // phase 2: local start of every (wave, expert) run: experts major, waves minor.  Thread t owns experts
@@ -259,15 +273,12 @@ __global__ __launch_bounds__(ROUTE_THREADS) void route_scatter_kernel(
     __syncthreads();
     const uint32_t total = s_scan[ROUTE_WAVES]; // ids of this unit that are in range
 
-    // phase 3: stable ranks, unit sorted into LDS.  ds_add_rtn_u32 applies the lanes of one wave instruction that hit
-    // the same address in lane order (verified on gfx950 over 5e7 lane operations against the ballot formulation below,
-    // and by the bit-exact stability tests), and a wave's LDS instructions execute in program order: the returned
-    // value is the stable position.  XMA_ROUTE_BALLOT_RANKS selects the formulation that does not rely on that.
+    // phase 3: the unit sorted into LDS: local position = start of the (wave, expert) run + rank
 #ifndef XMA_ROUTE_BALLOT_RANKS
 #pragma unroll
     for (int s = 0; s < ROUTE_STEPS; ++s) {
         if (key[s] != 0xffffffffu) {
-            const uint32_t pos = atomicAdd(&my_ctr[key[s]], 1u);
+            const uint32_t pos = my_ctr[key[s]] + rank[s];
             s_idx[pos] = (uint16_t)(wave * ROUTE_WAVE_IDS + s * WAVE + lane);
             s_exp[pos] = (uint16_t)key[s];
         }
