@@ -102,7 +102,7 @@ def test_moe_tiles_split_along_k(act_name):
 
 
 def test_moe_plumbing_config_shape():
-    """BASELINE configs[0] (T=512, H=256, I=512, E=8, top-2, SwiGLU, weights N(0, 0.02)) in fp32, as stated, and bf16."""
+    """The small plumbing configuration (T=512, H=256, I=512, E=8, top-2, SwiGLU, weights N(0, 0.02)) in fp32 and in bf16."""
     _run_case(torch.float32, 512, 8, 2, 256, 512, "swiglu_packed", seed=0)
     _run_case(torch.bfloat16, 512, 8, 2, 256, 512, "swiglu_packed", seed=0)
 

@@ -58,7 +58,7 @@ def test_continuous_count_edge_cases():
 @pytest.mark.parametrize("dist", ["uniform", "zipf", "sorted"])
 @pytest.mark.parametrize("dtype", [torch.int32, torch.int64])
 def test_continuous_count_4m(dist, dtype):
-    """BASELINE configs[1]: 4 Mi ids over E = 64, uniform and Zipf(s = 1.1); also the sorted input the MoE feeds."""
+    """The routing benchmark configuration: 4 Mi ids over E = 64, uniform and Zipf(s = 1.1); also the sorted input the MoE feeds."""
     from xma.functional import continuous_count
 
     n, E = 4 * 1024 * 1024, 64
@@ -100,7 +100,7 @@ def test_route_small_and_ragged(dtype):
 
 @pytest.mark.parametrize("dist", ["uniform", "zipf"])
 def test_route_4m(dist):
-    """BASELINE configs[1] at full size: bit-exact against the oracle plus the size-independent properties
+    """The routing benchmark configuration at full size: bit-exact against the oracle plus the size-independent properties
     (permutation, sortedness, stability, offsets identities)."""
     from xma.layers.moe import rocm_implementation as R
 
