@@ -279,8 +279,8 @@ __device__ __forceinline__ bool locate_tile(const FwdArgs &a, unsigned char *sme
         }
         const int b = (int)blockIdx.x;
         if (ROLE == ROLE_FIXUP) {
-            if (b >= rest) return false;
-            L = full + b;
+            if ((b >> 2) >= rest) return false; // four workgroups per split tile
+            L = full + (b >> 2);
         } else if (ROLE == ROLE_SLICES) {
             if (rest == 0) return false;
             const int q = xcd_remap(b, a.split_cus); // neighbouring tiles of one slice index meet in one XCD's L2
@@ -366,7 +366,8 @@ __device__ __forceinline__ bool locate_tile(const FwdArgs &a, unsigned char *sme
 // ---- epilogue of one 256 x 256 tile (LDS is free: no wave reads operand tiles any more)
 template <typename T, int EPI>
 __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4][4], unsigned char *smem, int64_t row0,
-                                              int rows_valid, int n0) {
+                                              int rows_valid, int n0, int only_i = -1) {
+    // only_i >= 0: just the 32-row block only_i of every wave (the fix-up kernel spreads a tile over four workgroups)
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wq = (wave & 1) * 128, wp = (wave >> 1) * 128; // wave's 128 x 128 corner inside the tile
@@ -418,6 +419,7 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             if (wq + i * 32 >= rows_valid) break; // wave-uniform
+            if (only_i >= 0 && i != only_i) continue;
             const int dst = dst_i[i];
             const float sc = sc_i[i];
 #pragma unroll
@@ -490,13 +492,15 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
                 if (col_ok) zin[it] = *(const u32x4 *)(a.aux + (row0 + r) * a.ldaux + cz);
             }
         };
-        if (wq < rows_valid) load_block(0);
+        const int i_first = only_i >= 0 ? only_i : 0, i_last = only_i >= 0 ? only_i : 3;
+        if (wq + i_first * 32 < rows_valid) load_block(i_first);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             if (wq + i * 32 >= rows_valid) break; // wave-uniform
+            if (i < i_first || i > i_last) continue;
 #pragma unroll
             for (int it = 0; it < 16; ++it) *(u32x4 *)(row_io + 2 * it * EPI_BWD_STRIDE) = zin[it];
-            if (i < 3 && wq + (i + 1) * 32 < rows_valid) load_block(i + 1);
+            if (i < i_last && wq + (i + 1) * 32 < rows_valid) load_block(i + 1);
             wave_lds_sync();
             const float sc = sc_i[i];
 #pragma unroll
@@ -702,8 +706,10 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
         tile_epilogue<T, EPI>(a, acc, smem, row0, rows_valid, n0);
 }
 
-// Sum of the K slices of the split tiles of the last round, then the epilogue of the GEMM kernel.  One workgroup per
-// split tile; the slices are added in a fixed order, so the result does not depend on timing.
+// Sum of the K slices of the split tiles of the last round, then the epilogue of the GEMM kernel.  Four workgroups
+// per split tile, one per 32-row block of the waves' corners (a quarter of the loads each: the kernel is a chain of
+// dependent round trips, so it is as fast as it is parallel); the slices are added in a fixed order, so the result does
+// not depend on timing.
 template <typename T, int EPI>
 __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_fixup_kernel(const FwdArgs a) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
@@ -711,6 +717,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_fixup_kernel(con
     TileSched ts;
     if (!locate_tile<ROLE_FIXUP>(a, smem, s_sched, ts)) return;
     const int tid = threadIdx.x;
+    const int iblk = blockIdx.x & 3;
     f32x16 acc[4][4];
     zero_acc(acc);
     for (int p = 0; p < ts.parts; ++p) {
@@ -718,14 +725,16 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_fixup_kernel(con
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
-            for (int i = 0; i < 4; ++i)
+            for (int i = 0; i < 4; ++i) {
+                if (i != iblk) continue;
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
                     const float4 v = src[((j * 4 + i) * 4 + g) * GEMM_THREADS];
                     acc[j][i][4 * g] += v.x, acc[j][i][4 * g + 1] += v.y, acc[j][i][4 * g + 2] += v.z, acc[j][i][4 * g + 3] += v.w;
                 }
+            }
     }
-    tile_epilogue<T, EPI>(a, acc, smem, ts.row0, ts.rows_valid, ts.n0);
+    tile_epilogue<T, EPI>(a, acc, smem, ts.row0, ts.rows_valid, ts.n0, iblk);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -837,11 +846,13 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
         FragBase<1> qb, pb;
         make_frag_base<1>(qb, lds0, wq, lane);
         make_frag_base<1>(pb, lds0 + OP_CHUNKS * 16, wp, lane);
-        if (GATHER) {
-            load_idx(0);
-            use_idx();
-        }
-        static_for<16>([&](auto P) { issue_piece(0, P, IC<0>{}); });
+        // the operand that is not gathered needs no index: its first step goes out while the indices are on their way
+        if (GATHER) load_idx(0);
+        if (!GQ) static_for<8>([&](auto P) { issue_piece(0, P, IC<0>{}); });
+        if (!GP) static_for<8>([&](auto P) { issue_piece(0, IC<8 + P.value>{}, IC<0>{}); });
+        if (GATHER) use_idx();
+        if (GQ) static_for<8>([&](auto P) { issue_piece(0, P, IC<0>{}); });
+        if (GP) static_for<8>([&](auto P) { issue_piece(0, IC<8 + P.value>{}, IC<0>{}); });
         __builtin_amdgcn_sched_barrier(0);
         if (GATHER) {
             load_idx(1);
@@ -921,7 +932,7 @@ template <typename T, int WT, int EPI> int launch_fwd(const FwdArgs &a, hipStrea
     grouped_gemm_kernel<T, WT, XMA_ROCM_EPI_STORE, ROLE_SLICES><<<a.split_cus, GEMM_THREADS, GEMM_SMEM_BYTES, st>>>(a);
     if ((rc = xma_check_launch("grouped_gemm_kernel (K slices)"))) return rc;
     if ((rc = gemm_set_smem(grouped_gemm_fixup_kernel<T, EPI>, GEMM_SMEM_BYTES))) return rc;
-    grouped_gemm_fixup_kernel<T, EPI><<<a.split_cus, GEMM_THREADS, GEMM_SMEM_BYTES, st>>>(a);
+    grouped_gemm_fixup_kernel<T, EPI><<<4 * a.split_cus, GEMM_THREADS, GEMM_SMEM_BYTES, st>>>(a);
     return xma_check_launch("grouped_gemm_fixup_kernel");
 }
 
