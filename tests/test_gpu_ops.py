@@ -151,3 +151,41 @@ def test_swiglu_packed_standalone(dtype):
         dg, du = oracle.swiglu_backward(x[..., 0::2].float(), x[..., 1::2].float(), dy.float())
         want = torch.stack([dg, du], dim=-1).flatten(-2)
         assert nerr(xd.grad, want) <= _tol(dtype)
+
+
+def test_scatter2scatter_with_and_without_workspace():
+    """The same launch through the C ABI with the scratch for splitting the last round of tiles along K and without
+    it (every tile by one workgroup): both within tolerance of the oracle; the workspace query and its error code."""
+    from xma.rocm.loader import get_library
+
+    lib = get_library()
+    T, E, k, K, N = 300, 3, 2, 2048, 320
+    dtype = torch.bfloat16
+    sel, se, ss, offs = _routing(T, E, k, 0)
+    g = torch.Generator().manual_seed(3)
+    M = T * k
+    X = torch.randn(M, K, generator=g).to(dtype)
+    W = (torch.randn(E, N, K, generator=g) * 0.1).to(dtype)
+    want = oracle.scatter2scatter(X, W.permute(0, 2, 1), se, ss, k, True, True, None)
+    Xd, Wd, ssd, offsd = X.cuda(), W.cuda(), ss.cuda(), offs.cuda()
+    st = torch.cuda.current_stream().cuda_stream
+    need = lib.xma_rocm_scatter2scatter_workspace_bytes(M, N, K, E)
+    assert need > 0  # a handful of tiles: a last (and only) round that can be split
+    ws = torch.empty(need // 4, dtype=torch.float32, device="cuda")
+
+    def run(wptr, wbytes):
+        out = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+        rc = lib.xma_rocm_scatter2scatter(Xd.data_ptr(), K, Wd.data_ptr(), N * K, K, 0, ssd.data_ptr(), offsd.data_ptr(),
+                                          out.data_ptr(), N, None, 0, None, M, N, K, E, k, 1, 1, 0, 0, wptr, wbytes, st)
+        torch.cuda.synchronize()
+        return rc, out
+
+    rc, split = run(ws.data_ptr(), need)
+    assert rc == 0 and nerr(split, want) <= TOL
+    rc, whole = run(None, 0)
+    assert rc == 0 and nerr(whole, want) <= TOL
+    assert nerr(split, whole) <= 2e-3  # the two differ only in the order of the fp32 summation over K
+    rc, _ = run(ws.data_ptr(), need - 16)
+    assert rc == -3 and b"workspace" in lib.xma_rocm_last_error()
+    # launches of many rounds of tiles never split: no scratch asked for
+    assert lib.xma_rocm_scatter2scatter_workspace_bytes(16384, 28672, 4096, 8) == 0
