@@ -416,6 +416,8 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
                 dst_i[i] = (int)(row0 + r);
             }
         }
+        // two copies of the loop: without a row scale the 256 multiplications by one are left out
+        auto blocks = [&](auto SCALED) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             if (wq + i * 32 >= rows_valid) break; // wave-uniform
@@ -426,8 +428,9 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
             for (int j = 0; j < 4; ++j) {
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const float v0 = acc[j][i][4 * g] * sc, v1 = acc[j][i][4 * g + 1] * sc;
-                    const float v2 = acc[j][i][4 * g + 2] * sc, v3 = acc[j][i][4 * g + 3] * sc;
+                    float v0 = acc[j][i][4 * g], v1 = acc[j][i][4 * g + 1];
+                    float v2 = acc[j][i][4 * g + 2], v3 = acc[j][i][4 * g + 3];
+                    if constexpr (SCALED.value) v0 *= sc, v1 *= sc, v2 *= sc, v3 *= sc;
                     const uint32_t z0 = Elem<T>::pack(v0, v1), z1 = Elem<T>::pack(v2, v3);
                     u32x2 o = {z0, z1};
                     *(u32x2 *)(z_w + (j * 32 + g * 8) * 2) = o;
@@ -463,6 +466,11 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
             }
             wave_lds_sync(); // the next block overwrites the area
         }
+        };
+        if (a.scale)
+            blocks(IC<1>{});
+        else
+            blocks(IC<0>{});
     } else {
         // SwiGLU backward: the accumulators are d h for the wave's 128 columns; z and dz have twice as many (gate, up
         // interleaved).  Each 32-row block of z comes in as whole rows (2 rows of 512 bytes per instruction) through
