@@ -30,7 +30,12 @@
 //   dW           :  Q = dY columns (out features),    P = X columns (in features), K = tokens
 //
 // Tiles never straddle experts: the schedule is expert-major, derived on the device from the inclusive expert
-// offsets in each workgroup's prologue (no host read of the counts).
+// offsets in each workgroup's prologue (no host read of the counts).  With a workspace, the tiles of a last, partial
+// round of a launch are computed as K slices by a second launch and summed by grouped_gemm_fixup_kernel.
+//
+// Epilogues (plain store with optional row scale and scatter, SwiGLU forward, SwiGLU backward) stage every 32-row block
+// of a wave's corner in wave-private LDS and write whole rows: in the accumulator layout a store instruction would
+// touch 32 rows with 16 bytes each.
 #include "fp32.hpp"
 #include "gemm_common.hpp"
 
