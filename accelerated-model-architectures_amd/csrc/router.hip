@@ -1,0 +1,307 @@
+// Router of the MoE layer behind the gate GEMM: top-k selection over each row of expert logits, fp32 softmax over the
+// k selected values and the selected expert ids in one pass (xma/layers/moe/__init__.py:186-193 and :256-262), and the
+// backward of that chain (gradient of the logits from the gradient of the router weights).
+//
+// A row is held in registers by a group of G = min(64, next power of two >= E) lanes of a wave, VPL = ceil(E / G)
+// values per lane (element e lives in lane e % G), so a wave takes 64 / G rows.  Selection is k rounds of "largest
+// remaining value, lowest index among equals" by a butterfly over the group; round r leaves its winner in lane r, so
+// the k results of a row come out of k neighbouring lanes.  HBM traffic is the logits once in, (weights, ids) once out.
+#include "common.hpp"
+
+namespace {
+
+constexpr int RT_THREADS = 256;
+constexpr int RT_MAX_E = 2048, RT_MAX_K = 64;
+
+// monotone map float -> uint32 (a larger value has a larger key).  NaN is the largest value, as in torch.topk;
+// -0 and +0 are equal; every key is > 0, so 0 marks "not a candidate".
+__device__ __forceinline__ uint32_t order_key(float v) {
+    uint32_t u = __builtin_bit_cast(uint32_t, v);
+    if (v != v) return 0xffffffffu;
+    if (u == 0x80000000u) u = 0;
+    return (u & 0x80000000u) ? ~u : (u | 0x80000000u);
+}
+__device__ __forceinline__ float key_value(uint32_t key) {
+    if (key == 0xffffffffu) return __builtin_nanf("");
+    const uint32_t u = (key & 0x80000000u) ? (key ^ 0x80000000u) : ~key;
+    return __builtin_bit_cast(float, u);
+}
+
+template <int DT> struct Scalar;
+template <> struct Scalar<XMA_ROCM_BF16> {
+    typedef uint16_t type;
+    static __device__ __forceinline__ float load(const void *p, int64_t i) {
+        return Elem<__bf16>::lo((uint32_t)((const uint16_t *)p)[i]);
+    }
+    static __device__ __forceinline__ void store(void *p, int64_t i, float v) {
+        ((uint16_t *)p)[i] = (uint16_t)(Elem<__bf16>::pack(v, 0.f) & 0xffffu);
+    }
+};
+template <> struct Scalar<XMA_ROCM_F16> {
+    typedef uint16_t type;
+    static __device__ __forceinline__ float load(const void *p, int64_t i) {
+        return Elem<_Float16>::lo((uint32_t)((const uint16_t *)p)[i]);
+    }
+    static __device__ __forceinline__ void store(void *p, int64_t i, float v) {
+        ((uint16_t *)p)[i] = (uint16_t)(Elem<_Float16>::pack(v, 0.f) & 0xffffu);
+    }
+};
+template <> struct Scalar<XMA_ROCM_F32> {
+    typedef float type;
+    static __device__ __forceinline__ float load(const void *p, int64_t i) { return ((const float *)p)[i]; }
+    static __device__ __forceinline__ void store(void *p, int64_t i, float v) { ((float *)p)[i] = v; }
+};
+
+// Exchange with the lane whose group-local index differs in bit log2(M) (or, for 4 and 8, with the mirrored lane of
+// the 8- or 16-lane block, which lies in the other half just the same): cross-lane moves inside a row of 16 lanes
+// are DPP operands of the VALU, 16 is an LDS-crossbar swizzle, only 32 needs a general permute.
+template <int M> __device__ __forceinline__ uint32_t lane_exchange(uint32_t v) {
+    const int x = (int)v;
+    if constexpr (M == 1) return (uint32_t)__builtin_amdgcn_update_dpp(x, x, 0xB1, 0xf, 0xf, false);  // quad_perm 1,0,3,2
+    if constexpr (M == 2) return (uint32_t)__builtin_amdgcn_update_dpp(x, x, 0x4E, 0xf, 0xf, false);  // quad_perm 2,3,0,1
+    if constexpr (M == 4) return (uint32_t)__builtin_amdgcn_update_dpp(x, x, 0x141, 0xf, 0xf, false); // row_half_mirror
+    if constexpr (M == 8) return (uint32_t)__builtin_amdgcn_update_dpp(x, x, 0x140, 0xf, 0xf, false); // row_mirror
+    if constexpr (M == 16) return (uint32_t)__builtin_amdgcn_ds_swizzle(x, 0x401F);                   // lane ^ 16
+    return (uint32_t)__shfl_xor(x, 32);
+}
+template <int M> __device__ __forceinline__ float lane_exchange(float v) {
+    return __builtin_bit_cast(float, lane_exchange<M>(__builtin_bit_cast(uint32_t, v)));
+}
+
+// all-reduce over the G lanes of a group; op(a, b) must be commutative and associative
+template <int G, int M = 1, typename V, typename Op> __device__ __forceinline__ V group_reduce(V v, Op op) {
+    if constexpr (M < G) {
+        v = op(v, lane_exchange<M>(v));
+        return group_reduce<G, M * 2>(v, op);
+    } else
+        return v;
+}
+template <int G> __device__ __forceinline__ float group_sum(float v) {
+    return group_reduce<G>(v, [](float a, float b) { return a + b; });
+}
+
+// softmax over the values held by lanes 0..k-1 of a group; lane 0 holds the largest (NaN propagates like in torch)
+template <int G> __device__ __forceinline__ float group_softmax(float my_val, int g, int k, int group_lane0) {
+    const float vmax = __shfl(my_val, group_lane0);
+    const float ex = (g < k) ? expf(my_val - vmax) : 0.f;
+    return ex / group_sum<G>(ex);
+}
+
+// A candidate of the selection: larger value first, lower expert index among equal values.  16-bit logits have
+// 16-bit keys, so key and inverted index share one word and the butterfly is a plain integer maximum; fp32 logits
+// carry the index in a second word.  The all-zero candidate loses against every real one.
+template <int DT> struct Cand {
+    uint32_t packed; // key16 << 16 | (0xffff - index)
+    static __device__ __forceinline__ Cand none() { return {0u}; }
+    static __device__ __forceinline__ Cand make(const void *row, int e) {
+        const uint32_t b = ((const uint16_t *)row)[e];
+        const uint32_t inf = (DT == XMA_ROCM_BF16) ? 0x7f80u : 0x7c00u;
+        uint32_t key;
+        if ((b & 0x7fffu) > inf)
+            key = 0xffffu;
+        else if (b == 0x8000u)
+            key = 0x8000u;
+        else
+            key = (b & 0x8000u) ? (~b & 0xffffu) : (b | 0x8000u);
+        return {(key << 16) | (0xffffu - (uint32_t)e)};
+    }
+    __device__ __forceinline__ bool beats(const Cand &o) const { return packed > o.packed; }
+    __device__ __forceinline__ bool is_none() const { return packed == 0u; }
+    __device__ __forceinline__ int index() const { return (int)(0xffffu - (packed & 0xffffu)); }
+    __device__ __forceinline__ float value() const {
+        const uint32_t key = packed >> 16;
+        const uint32_t b = (key == 0xffffu) ? 0x7fffu : ((key & 0x8000u) ? (key ^ 0x8000u) : (~key & 0xffffu));
+        return (DT == XMA_ROCM_BF16) ? Elem<__bf16>::lo(b) : Elem<_Float16>::lo(b);
+    }
+    template <int G> __device__ __forceinline__ Cand group_best() const {
+        return {group_reduce<G>(packed, [](uint32_t a, uint32_t b) { return a > b ? a : b; })};
+    }
+};
+template <> struct Cand<XMA_ROCM_F32> {
+    uint32_t key;
+    int idx;
+    static __device__ __forceinline__ Cand none() { return {0u, 0x7fffffff}; }
+    static __device__ __forceinline__ Cand make(const void *row, int e) { return {order_key(((const float *)row)[e]), e}; }
+    __device__ __forceinline__ bool beats(const Cand &o) const { return key > o.key || (key == o.key && idx < o.idx); }
+    __device__ __forceinline__ bool is_none() const { return key == 0u; }
+    __device__ __forceinline__ int index() const { return idx; }
+    __device__ __forceinline__ float value() const { return key_value(key); }
+    template <int G, int M = 1> __device__ __forceinline__ Cand group_best() const {
+        if constexpr (M < G) {
+            const Cand o = {lane_exchange<M>(key), (int)lane_exchange<M>((uint32_t)idx)};
+            const Cand w = o.beats(*this) ? o : *this;
+            return w.template group_best<G, M * 2>();
+        } else
+            return *this;
+    }
+};
+
+template <int DT, int G, int VPL>
+__global__ __launch_bounds__(RT_THREADS) void router_topk_kernel(const void *__restrict__ logits, int64_t ld, int64_t T,
+                                                                int E, int k, void *__restrict__ weights,
+                                                                void *__restrict__ ids, int ids_i64) {
+    const int lane = threadIdx.x & 63;
+    const int g = lane & (G - 1);
+    const int64_t wave = (int64_t)blockIdx.x * (RT_THREADS / 64) + (threadIdx.x >> 6);
+    const int64_t t = wave * (64 / G) + lane / G;
+    const bool live = t < T; // the same for all lanes of a group; dead groups still take part in the exchanges
+    const void *row = (const char *)logits + (live ? t : 0) * ld * (int64_t)sizeof(typename Scalar<DT>::type);
+    Cand<DT> c[VPL];
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) {
+        const int e = g + v * G;
+        c[v] = (live && e < E) ? Cand<DT>::make(row, e) : Cand<DT>::none();
+    }
+    Cand<DT> mine = Cand<DT>::none();
+    for (int r = 0; r < k; ++r) {
+        Cand<DT> best = c[0];
+#pragma unroll
+        for (int v = 1; v < VPL; ++v)
+            if (c[v].beats(best)) best = c[v];
+        best = best.template group_best<G>();
+        const int be = best.index();
+#pragma unroll
+        for (int v = 0; v < VPL; ++v)
+            if (g + v * G == be && !best.is_none()) c[v] = Cand<DT>::none(); // taken
+        if (g == r) mine = best;
+    }
+    const float w = group_softmax<G>(mine.value(), g, k, lane - g);
+    if (live && g < k) {
+        Scalar<DT>::store(weights, t * k + g, w);
+        if (ids_i64)
+            ((int64_t *)ids)[t * k + g] = mine.index();
+        else
+            ((int32_t *)ids)[t * k + g] = mine.index();
+    }
+}
+
+// d_logits[t, :] = 0 except d_logits[t, ids[t, j]] = w_j * (d_w[t, j] - sum_i w_i d_w[t, i]), w = the fp32 softmax of
+// the selected logits, recomputed exactly as in the forward kernel.  Writes every element of d_logits.
+template <int DT, int G, int VPL>
+__global__ __launch_bounds__(RT_THREADS) void router_topk_bwd_kernel(const void *__restrict__ logits, int64_t ld,
+                                                                    int64_t T, int E, int k,
+                                                                    const void *__restrict__ ids, int ids_i64,
+                                                                    const void *__restrict__ d_w,
+                                                                    void *__restrict__ d_logits, int64_t ldd) {
+    const int lane = threadIdx.x & 63;
+    const int g = lane & (G - 1);
+    const int64_t wave = (int64_t)blockIdx.x * (RT_THREADS / 64) + (threadIdx.x >> 6);
+    const int64_t t = wave * (64 / G) + lane / G;
+    const bool live = t < T;
+    int my_idx = -1;
+    float my_val = 0.f, my_dw = 0.f;
+    if (live && g < k) {
+        my_idx = ids_i64 ? (int)((const int64_t *)ids)[t * k + g] : ((const int32_t *)ids)[t * k + g];
+        my_idx = my_idx < 0 ? 0 : (my_idx >= E ? E - 1 : my_idx); // ids come from the forward; never read outside the row
+        my_val = key_value(order_key(Scalar<DT>::load(logits, t * ld + my_idx)));
+        my_dw = Scalar<DT>::load(d_w, t * k + g);
+    }
+    const float w = group_softmax<G>(my_val, g, k, lane - g);
+    const float dot = group_sum<G>((g < k) ? w * my_dw : 0.f);
+    const float dv = w * (my_dw - dot);
+    float out[VPL];
+#pragma unroll
+    for (int v = 0; v < VPL; ++v) out[v] = 0.f;
+    for (int j = 0; j < k; ++j) {
+        const int ej = __shfl(my_idx, lane - g + j);
+        const float dj = __shfl(dv, lane - g + j);
+#pragma unroll
+        for (int v = 0; v < VPL; ++v)
+            if (g + v * G == ej) out[v] = dj;
+    }
+    if (live) {
+#pragma unroll
+        for (int v = 0; v < VPL; ++v) {
+            const int e = g + v * G;
+            if (e < E) Scalar<DT>::store(d_logits, t * ldd + e, out[v]);
+        }
+    }
+}
+
+struct RouterShape {
+    int G, vpl;
+    int64_t blocks;
+};
+
+int router_shape(const char *what, int64_t T, int E, int k, int dtype, RouterShape &s) {
+    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16 || dtype == XMA_ROCM_F32, XMA_ROCM_EUNSUPPORTED,
+                "%s: dtype %d", what, dtype);
+    XMA_REQUIRE(T >= 0 && E >= 1 && k >= 1 && k <= E, XMA_ROCM_EINVAL, "%s: T=%lld E=%d k=%d (1 <= k <= E)", what,
+                (long long)T, E, k);
+    XMA_REQUIRE(E <= RT_MAX_E && k <= RT_MAX_K, XMA_ROCM_EUNSUPPORTED, "%s: E=%d k=%d (E <= %d, k <= %d)", what, E, k,
+                RT_MAX_E, RT_MAX_K);
+    int G = 1;
+    while (G < E && G < 64) G <<= 1;
+    int vpl = 1;
+    while (G * vpl < E) vpl <<= 1;
+    s.G = G;
+    s.vpl = vpl;
+    const int64_t rows_per_block = (int64_t)(RT_THREADS / 64) * (64 / G);
+    s.blocks = (T + rows_per_block - 1) / rows_per_block;
+    XMA_REQUIRE(s.blocks < ((int64_t)1 << 31), XMA_ROCM_EUNSUPPORTED, "%s: too many rows", what);
+    return XMA_ROCM_OK;
+}
+
+#define ROUTER_CASE(g_, v_, CALL)   \
+    {                               \
+        constexpr int G = g_;       \
+        constexpr int VPL = v_;     \
+        CALL;                       \
+    }                               \
+    break;
+#define ROUTER_DISPATCH_SHAPE(s, CALL)        \
+    switch ((s).G * (s).vpl) {                \
+    case 1: ROUTER_CASE(1, 1, CALL)           \
+    case 2: ROUTER_CASE(2, 1, CALL)           \
+    case 4: ROUTER_CASE(4, 1, CALL)           \
+    case 8: ROUTER_CASE(8, 1, CALL)           \
+    case 16: ROUTER_CASE(16, 1, CALL)         \
+    case 32: ROUTER_CASE(32, 1, CALL)         \
+    case 64: ROUTER_CASE(64, 1, CALL)         \
+    case 128: ROUTER_CASE(64, 2, CALL)        \
+    case 256: ROUTER_CASE(64, 4, CALL)        \
+    case 512: ROUTER_CASE(64, 8, CALL)        \
+    case 1024: ROUTER_CASE(64, 16, CALL)      \
+    default: ROUTER_CASE(64, 32, CALL)        \
+    }
+#define ROUTER_DISPATCH(dtype, s, CALL)           \
+    if (dtype == XMA_ROCM_BF16) {                 \
+        constexpr int DT = XMA_ROCM_BF16;         \
+        ROUTER_DISPATCH_SHAPE(s, CALL)            \
+    } else if (dtype == XMA_ROCM_F16) {           \
+        constexpr int DT = XMA_ROCM_F16;          \
+        ROUTER_DISPATCH_SHAPE(s, CALL)            \
+    } else {                                      \
+        constexpr int DT = XMA_ROCM_F32;          \
+        ROUTER_DISPATCH_SHAPE(s, CALL)            \
+    }
+
+} // namespace
+
+extern "C" int xma_rocm_router_topk(const void *logits, int64_t ld, int64_t T, int32_t E, int32_t k, int dtype,
+                                    void *weights, void *ids, int ids_is_i64, void *stream) {
+    RouterShape s;
+    if (int rc = router_shape("router_topk", T, E, k, dtype, s)) return rc;
+    XMA_REQUIRE(ld >= E, XMA_ROCM_EINVAL, "router_topk: ld=%lld < E=%d", (long long)ld, E);
+    XMA_REQUIRE(T == 0 || (logits && weights && ids), XMA_ROCM_EINVAL, "router_topk: null pointer");
+    if (T == 0) return XMA_ROCM_OK;
+    hipStream_t st = (hipStream_t)stream;
+    ROUTER_DISPATCH(dtype, s, (router_topk_kernel<DT, G, VPL><<<(int)s.blocks, RT_THREADS, 0, st>>>(
+                                  logits, ld, T, E, k, weights, ids, ids_is_i64)));
+    return xma_check_launch("router_topk_kernel");
+}
+
+extern "C" int xma_rocm_router_topk_bwd(const void *logits, int64_t ld, int64_t T, int32_t E, int32_t k, int dtype,
+                                        const void *ids, int ids_is_i64, const void *d_weights, void *d_logits,
+                                        int64_t ldd, void *stream) {
+    RouterShape s;
+    if (int rc = router_shape("router_topk_bwd", T, E, k, dtype, s)) return rc;
+    XMA_REQUIRE(ld >= E && ldd >= E, XMA_ROCM_EINVAL, "router_topk_bwd: ld=%lld ldd=%lld < E=%d", (long long)ld,
+                (long long)ldd, E);
+    XMA_REQUIRE(T == 0 || (logits && ids && d_weights && d_logits), XMA_ROCM_EINVAL, "router_topk_bwd: null pointer");
+    if (T == 0) return XMA_ROCM_OK;
+    hipStream_t st = (hipStream_t)stream;
+    ROUTER_DISPATCH(dtype, s, (router_topk_bwd_kernel<DT, G, VPL><<<(int)s.blocks, RT_THREADS, 0, st>>>(
+                                  logits, ld, T, E, k, ids, ids_is_i64, d_weights, d_logits, ldd)));
+    return xma_check_launch("router_topk_bwd_kernel");
+}

@@ -93,13 +93,23 @@ class MoE(nn.Module):
     def forward(self, x: torch.Tensor, *, kernel_backend: KernelBackend | None = None) -> tuple[torch.Tensor, torch.Tensor]:
         original_shape = x.shape
         x = x.view(-1, self.hidden_size)
-        router_logits, router_weights, selected_experts = self._compute_routing_weights(x)
+        router_logits, router_weights, selected_experts = self._compute_routing_weights(x, kernel_backend=kernel_backend)
         x = self._compute_experts(x, router_weights, selected_experts, kernel_backend=kernel_backend)
         return x.view(original_shape), router_logits
 
-    def _compute_routing_weights(self, x: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    def _compute_routing_weights(
+        self, x: torch.Tensor, *, kernel_backend: KernelBackend | None = None
+    ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
         # (T, H) -> logits (T, E), weights (T, k) = fp32 softmax over the k selected logits, experts (T, k)
         router_logits = self.gate(x)
+        if kernel_backend is None:
+            kernel_backend = Accelerator.get_kernel_backend()
+        if kernel_backend == KernelBackend.rocm and router_logits.is_cuda:
+            from . import rocm_implementation as R
+
+            # top-k, softmax and the cast in one kernel; equal logits go to the lower expert index
+            router_weights, selected_experts = R.router_topk(router_logits, self.top_k)
+            return router_logits, router_weights, selected_experts
         router_weights, selected_experts = self._get_topk(router_logits)
         router_weights = F.softmax(router_weights.float(), dim=-1).type_as(x)
         return router_logits, router_weights, selected_experts

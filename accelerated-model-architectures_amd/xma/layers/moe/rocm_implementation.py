@@ -4,7 +4,7 @@ Mirrors the op-level interface of the reference's Triton implementation
 (xma/layers/moe/triton_implementation/__init__.py): ``scatter2scatter``,
 ``group``, ``group_bwd_W`` and the two autograd Functions behind
 ``up_projection_experts`` / ``down_projection_experts``; adds ``route`` (one op
-for sort + histogram + offsets) and ``fused_swiglu_experts`` (the whole expert
+for sort + histogram + offsets), ``router_topk`` (top-k + softmax behind the gate) and ``fused_swiglu_experts`` (the whole expert
 computation with SwiGLU folded into the GEMM epilogues).
 
 Differences from the reference's data flow, all of which remove HBM passes:
@@ -38,6 +38,33 @@ def route(selected_experts: torch.Tensor, num_experts: int):
     sorted_scattered_idxs = torch.empty(n, dtype=torch.int64, device=dev)
     ops.route_rocm(ids, counts, incl, excl, sorted_expert_idxs, sorted_scattered_idxs, None)
     return counts, incl, excl, sorted_expert_idxs, sorted_scattered_idxs
+
+
+class _RouterTopK(torch.autograd.Function):
+    """top-k + fp32 softmax over the selected logits + cast, and the gradient of the logits
+    (xma/layers/moe/__init__.py:186-193, 256-262)"""
+
+    @staticmethod
+    def forward(ctx, router_logits: torch.Tensor, top_k: int):
+        T = router_logits.size(0)
+        weights = torch.empty(T, top_k, dtype=router_logits.dtype, device=router_logits.device)
+        ids = torch.empty(T, top_k, dtype=torch.int64, device=router_logits.device)
+        ops.router_topk_rocm(router_logits, weights, ids)
+        ctx.save_for_backward(router_logits, ids)
+        ctx.mark_non_differentiable(ids)
+        return weights, ids
+
+    @staticmethod
+    def backward(ctx, d_weights: torch.Tensor, _d_ids):
+        router_logits, ids = ctx.saved_tensors
+        d_logits = torch.empty_like(router_logits, memory_format=torch.contiguous_format)
+        ops.router_topk_bwd_rocm(router_logits, ids, d_weights.contiguous(), d_logits)
+        return d_logits, None
+
+
+def router_topk(router_logits: torch.Tensor, top_k: int):
+    """(router weights (T, k) in the logits' dtype, selected experts int64 (T, k)); differentiable in the logits."""
+    return _RouterTopK.apply(router_logits, top_k)
 
 
 # ----------------------------------------------------------------------------------------- op mirrors

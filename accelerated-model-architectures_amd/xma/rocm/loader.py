@@ -48,6 +48,8 @@ SIGNATURES = {
     "xma_rocm_combine_bwd": (_int, [_p, _i64, _p, _i64, _p, _i64, _i32, _i32, _int, _p]),
     "xma_rocm_swiglu_packed_forward": (_int, [_p, _i64, _p, _i64, _i64, _i32, _int, _p]),
     "xma_rocm_swiglu_packed_backward": (_int, [_p, _i64, _p, _i64, _p, _i64, _i64, _i32, _int, _p]),
+    "xma_rocm_router_topk": (_int, [_p, _i64, _i64, _i32, _i32, _int, _p, _p, _int, _p]),
+    "xma_rocm_router_topk_bwd": (_int, [_p, _i64, _i64, _i32, _i32, _int, _p, _int, _p, _p, _i64, _p]),
 }
 
 

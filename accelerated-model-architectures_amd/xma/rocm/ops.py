@@ -306,3 +306,37 @@ def swiglu_packed_backward_rocm(x: torch.Tensor, dy: torch.Tensor, dx: torch.Ten
                                             rows, cols, _code(x), _stream(x)),
         "xma_rocm_swiglu_packed_backward",
     )
+
+
+# --------------------------------------------------------------------------- router behind the gate GEMM
+@torch.library.custom_op("xma_rocm::router_topk", mutates_args={"weights", "ids"})
+def router_topk_rocm(logits: torch.Tensor, weights: torch.Tensor, ids: torch.Tensor) -> None:
+    """weights[t], ids[t] = softmax over / indices of the k largest logits of row t, k = weights.size(1)
+    (xma/layers/moe/__init__.py:186-193, 256-262)."""
+    T, E = logits.shape
+    k = weights.size(1)
+    assert weights.shape == (T, k) and ids.shape == (T, k) and weights.is_contiguous() and ids.is_contiguous()
+    assert weights.dtype == logits.dtype and ids.dtype in (torch.int32, torch.int64)
+    lib = get_library()
+    check(
+        lib.xma_rocm_router_topk(_ptr(logits), _rows(logits, "logits"), T, E, k, _code(logits), _ptr(weights), _ptr(ids),
+                                 int(ids.dtype == torch.int64), _stream(logits)),
+        "xma_rocm_router_topk",
+    )
+
+
+@torch.library.custom_op("xma_rocm::router_topk_bwd", mutates_args={"d_logits"})
+def router_topk_bwd_rocm(logits: torch.Tensor, ids: torch.Tensor, d_weights: torch.Tensor, d_logits: torch.Tensor) -> None:
+    """d_logits = gradient of the logits through top-k and softmax, every element written."""
+    T, E = logits.shape
+    k = ids.size(1)
+    assert ids.shape == (T, k) and d_weights.shape == (T, k) and d_logits.shape == (T, E)
+    assert ids.is_contiguous() and d_weights.is_contiguous() and ids.dtype in (torch.int32, torch.int64)
+    assert d_weights.dtype == logits.dtype == d_logits.dtype
+    lib = get_library()
+    check(
+        lib.xma_rocm_router_topk_bwd(_ptr(logits), _rows(logits, "logits"), T, E, k, _code(logits), _ptr(ids),
+                                     int(ids.dtype == torch.int64), _ptr(d_weights), _ptr(d_logits),
+                                     _rows(d_logits, "d_logits"), _stream(logits)),
+        "xma_rocm_router_topk_bwd",
+    )

@@ -139,6 +139,15 @@ def _kernel_table(moe, x, rw, sel, grad, cfg, iters):
     mem("combine_bwd", lambda: ops.combine_bwd_rocm(eo, grad, d_rw), Tk * H * esz + T * H * esz + T * k * esz)
     mem("group(dy*w)", lambda: ops.group_rocm(grad, ss, gdy, flat_w, k), T * H * esz + Tk * H * esz + Tk * (8 + esz))
     mem("route", lambda: R.route(sel, E), Tk * 8 + Tk * 8 + Tk * 8 + E * 20)
+    # the router behind the gate GEMM (outside the timed step, which starts from the router's outputs)
+    lg = torch.randn(T, E, device=dev, dtype=torch.float32).to(x.dtype)
+    r_w = torch.empty(T, k, device=dev, dtype=x.dtype)
+    r_ids = torch.empty(T, k, device=dev, dtype=torch.int64)
+    d_lg = torch.empty_like(lg)
+    mem("router_topk(top-k+softmax+ids)", lambda: ops.router_topk_rocm(lg, r_w, r_ids), T * E * esz + T * k * (esz + 8))
+    mem("router_topk_bwd", lambda: ops.router_topk_bwd_rocm(lg, r_ids, r_w, d_lg), 2 * T * E * esz + T * k * (esz + 8))
+    mem("router_torch(topk+softmax+cast)", lambda: torch.softmax(lg.topk(k, dim=-1).values.float(), -1).to(x.dtype),
+        T * E * esz + T * k * (esz + 8))
     return table
 
 

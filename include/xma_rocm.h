@@ -166,6 +166,24 @@ XMA_API int xma_rocm_swiglu_packed_forward(const void *x, int64_t ldx, void *y, 
 XMA_API int xma_rocm_swiglu_packed_backward(const void *x, int64_t ldx, const void *dy, int64_t lddy, void *dx,
                                     int64_t lddx, int64_t rows, int32_t cols_out, int dtype, void *stream);
 
+/*
+ * Router behind the gate GEMM: for each of T rows of E expert logits, the k largest values in descending order
+ * (equal values: lowest expert index first; NaN counts as the largest value), the fp32 softmax over those k values
+ * cast to `dtype`, and their expert ids (int64 if ids_is_i64, else int32), all (T, k) row-major.
+ * Replaces topk / max + softmax + type_as of xma/layers/moe/__init__.py:186-193 and :256-262 (three ATen launches
+ * and an fp32 round trip).  E <= 2048, k <= min(E, 64); `ld` = row stride of the logits in elements.
+ */
+XMA_API int xma_rocm_router_topk(const void *logits, int64_t ld, int64_t T, int32_t E, int32_t k, int dtype, void *weights,
+                         void *ids, int ids_is_i64, void *stream);
+/*
+ * Backward of xma_rocm_router_topk: with w = softmax of the selected logits (fp32, recomputed),
+ *     d_logits[t, ids[t, j]] = w_j * (d_weights[t, j] - sum_i w_i * d_weights[t, i]),  0 elsewhere.
+ * Writes all T x E elements of d_logits (row stride ldd), so the caller need not clear it.  Replaces the autograd
+ * chain of the same lines (type_as, softmax, float, topk backward with its zero fill and scatter).
+ */
+XMA_API int xma_rocm_router_topk_bwd(const void *logits, int64_t ld, int64_t T, int32_t E, int32_t k, int dtype, const void *ids,
+                             int ids_is_i64, const void *d_weights, void *d_logits, int64_t ldd, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

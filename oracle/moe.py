@@ -62,6 +62,17 @@ def routing_weights(router_logits: torch.Tensor, top_k: int, out_dtype: torch.dt
     return w, idx
 
 
+def routing_topk(router_logits: torch.Tensor, top_k: int, out_dtype: torch.dtype):
+    """routing_weights with the order among equal logits spelled out, which torch.topk leaves open: the k largest
+    values in descending order, the lower expert index first among equals (a stable descending sort; NaN counts as
+    the largest value, -0 equals +0).  On rows without equal values it is routing_weights.  Differentiable in the
+    logits (moe/__init__.py:186-193, 256-262)."""
+    idx = torch.sort(router_logits.detach().float(), dim=-1, descending=True, stable=True).indices[:, :top_k].contiguous()
+    vals = router_logits.gather(-1, idx)
+    w = F.softmax(vals.float(), dim=-1).to(out_dtype)
+    return w, idx
+
+
 # --------------------------------------------------------------------------- experts
 def experts_forward(
     x: torch.Tensor,  # (T, H)

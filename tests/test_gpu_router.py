@@ -1,0 +1,143 @@
+"""GPU parity of the fused router (top-k + fp32 softmax + expert ids behind the gate, and its backward)
+against the CPU oracle's restatement of xma/layers/moe/__init__.py:186-193, 256-262.
+
+Expert ids: bit-exact, also among equal logits (16-bit logits tie often; the rule is "lower expert index first",
+oracle.routing_topk).  Router weights and the logits' gradient: fp32 softmax on both sides, so the difference is the
+exp/division rounding before the cast: at most one unit in the last place of the result dtype."""
+
+import pytest
+import torch
+
+from oracle import moe as oracle
+
+pytestmark = pytest.mark.gpu
+
+ULP = {torch.float32: 2.0**-22, torch.bfloat16: 2.0**-8, torch.float16: 2.0**-11}  # weights are <= 1
+
+CASES = [  # T, E, k
+    (7, 8, 2),
+    (1000, 8, 2),
+    (513, 64, 6),
+    (300, 128, 8),
+    (33, 1, 1),
+    (50, 5, 5),
+    (64, 100, 1),
+    (257, 3, 2),
+    (40, 200, 7),
+    (19, 2048, 64),
+    (8192, 8, 2),
+    (130, 65, 33),
+]
+
+
+def _logits(T, E, dtype, seed=0, coarse=False):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(T, E, generator=g)
+    if coarse:  # few distinct values: every row has equal logits
+        x = (x * 2).round() / 2
+    return x.to(dtype)
+
+
+def _run_fwd(logits, k, id_dtype=torch.int64):
+    from xma.rocm import ops
+
+    d = logits.cuda()
+    w = torch.empty(d.size(0), k, dtype=d.dtype, device="cuda")
+    ids = torch.empty(d.size(0), k, dtype=id_dtype, device="cuda")
+    ops.router_topk_rocm(d, w, ids)
+    torch.cuda.synchronize()
+    return w.cpu(), ids.cpu()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("T,E,k", CASES)
+@pytest.mark.parametrize("coarse", [False, True])
+def test_router_topk_forward(dtype, T, E, k, coarse):
+    print(f"router fwd {dtype} T={T} E={E} k={k} coarse={coarse}", flush=True)
+    logits = _logits(T, E, dtype, seed=T + E + k, coarse=coarse)
+    want_w, want_ids = oracle.routing_topk(logits, k, dtype)
+    w, ids = _run_fwd(logits, k)
+    assert torch.equal(ids, want_ids)
+    assert (w.float() - want_w.float()).abs().max().item() <= ULP[dtype]
+    if not coarse and dtype == torch.float32:  # no equal values: the library routine gives the same selection
+        lib_w, lib_ids = oracle.routing_weights(logits, k, dtype)
+        assert torch.equal(ids, lib_ids)
+
+
+def test_router_topk_int32_ids_strided_rows_and_special_values():
+    logits = _logits(200, 16, torch.float32, seed=5)
+    logits[3, 4] = float("nan")
+    logits[4, :] = float("-inf")
+    logits[4, 9] = 1.0
+    logits[5, 2] = float("inf")
+    logits[6, 1], logits[6, 7] = 0.0, -0.0
+    logits[6, [0, 2, 3, 4, 5, 6]] = -1.0
+    want_w, want_ids = oracle.routing_topk(logits, 3, torch.float32)
+    w, ids = _run_fwd(logits, 3, torch.int32)
+    assert ids.dtype == torch.int32 and torch.equal(ids.long(), want_ids)
+    torch.testing.assert_close(w, want_w, rtol=0, atol=ULP[torch.float32], equal_nan=True)
+    # rows of a wider buffer (row stride 24)
+    wide = torch.zeros(200, 24)
+    wide[:, :16] = logits
+    from xma.rocm import ops
+
+    d = wide.cuda()[:, :16]
+    w2 = torch.empty(200, 3, device="cuda")
+    ids2 = torch.empty(200, 3, dtype=torch.int64, device="cuda")
+    ops.router_topk_rocm(d, w2, ids2)
+    assert torch.equal(ids2.cpu(), want_ids)
+    torch.testing.assert_close(w2.cpu(), want_w, rtol=0, atol=ULP[torch.float32], equal_nan=True)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("T,E,k", CASES)
+def test_router_topk_backward(dtype, T, E, k):
+    from xma.layers.moe import rocm_implementation as R
+
+    print(f"router bwd {dtype} T={T} E={E} k={k}", flush=True)
+    logits = _logits(T, E, dtype, seed=3 * T + E)
+    dw = torch.randn(T, k, generator=torch.Generator().manual_seed(1)).to(dtype)
+    lg = logits.clone().requires_grad_()
+    w, _ = oracle.routing_topk(lg, k, dtype)
+    w.backward(dw)
+    d = logits.cuda().requires_grad_()
+    wd, ids = R.router_topk(d, k)
+    assert not ids.requires_grad
+    wd.backward(dw.cuda())
+    got = d.grad.cpu()
+    assert got.dtype == dtype and got.shape == (T, E)
+    mask = torch.zeros(T, E, dtype=torch.bool).scatter_(1, ids.cpu(), True)
+    assert (got[~mask] == 0).all()  # exact zeros outside the selection
+    scale = max(dw.float().abs().max().item(), 1.0)
+    assert (got.float() - lg.grad.float()).abs().max().item() <= 2 * ULP[dtype] * scale
+
+
+def test_router_in_the_layer_forward_and_gate_gradient():
+    """MoE.forward on the rocm backend routes through the fused router: logits, selection (taken from the device
+    logits) and the gate's gradient against the oracle"""
+    from xma import KernelBackend, set_seed
+    from xma.functional import swiglu_packed
+    from xma.layers import MoE
+    from tests.utils import nerr
+
+    set_seed(3)
+    T, H, I, E, k = 192, 256, 128, 16, 4
+    moe = MoE(E, k, H, I, swiglu_packed, True, add_bias=False, std=0.02).to(torch.bfloat16).cuda()
+    x = torch.randn(T, H, device="cuda", dtype=torch.bfloat16)
+    grad = torch.randn(T, H, device="cuda", dtype=torch.bfloat16)
+    y, logits = moe(x, kernel_backend=KernelBackend.rocm)
+    y.backward(grad)
+    # oracle: the gate in fp32; selection and softmax from the device's bf16 logits
+    xc = x.float().cpu()
+    wg = moe.gate.weight.detach().float().cpu().requires_grad_()
+    dev_logits = logits.detach().float().cpu()
+    lg = xc @ wg.t()
+    assert (lg.detach() - dev_logits).abs().max().item() <= 2.0**-8 * max(1.0, dev_logits.abs().max().item())
+    lg = lg + (dev_logits - lg).detach()  # the device's values, the fp32 chain's gradient
+    _, sel = oracle.routing_topk(dev_logits, k, torch.float32)
+    rw = torch.softmax(lg.gather(-1, sel), -1)
+    want = oracle.experts_forward(xc, rw, sel, moe.c_fc.weight.detach().float().cpu(),
+                                  moe.c_proj.weight.detach().float().cpu(), oracle.swiglu_packed)
+    want.backward(grad.float().cpu())
+    assert nerr(y, want.detach()) <= 1e-2
+    assert nerr(moe.gate.weight.grad, wg.grad) <= 2e-2  # bf16 router weights and a bf16 gate GEMM in the chain

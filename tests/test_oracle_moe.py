@@ -54,6 +54,42 @@ def test_routing_weights_brute_force():
         assert torch.allclose(w.sum(-1), torch.ones(9), atol=1e-6)
 
 
+def test_routing_topk_tie_rule_and_agreement_with_topk():
+    """the restatement with the spelled-out tie rule: equals torch.topk on rows without equal values, picks the
+    lowest expert indices among equal values (brute force), NaN first, k = E gives the full softmax, and its
+    gradient is the softmax Jacobian scattered to the selected columns"""
+    torch.manual_seed(2)
+    logits = torch.randn(64, 10)
+    for k in (1, 3, 10):
+        w0, i0 = oracle.routing_weights(logits, k, torch.float32)
+        w1, i1 = oracle.routing_topk(logits, k, torch.float32)
+        assert torch.equal(i0, i1) and torch.equal(w0, w1)
+    # heavy ties: values from a set of 3
+    tied = torch.randint(0, 3, (50, 7)).float()
+    tied[0, :] = 1.0
+    tied[1, 3] = float("nan")
+    tied[2, 2], tied[2, 5] = 0.0, -0.0
+    for k in (1, 2, 5, 7):
+        w, idx = oracle.routing_topk(tied, k, torch.float32)
+        for t in range(50):
+            row = tied[t].tolist()
+            key = lambda e: (0 if math.isnan(row[e]) else 1, -row[e] if not math.isnan(row[e]) else 0.0, e)
+            assert idx[t].tolist() == sorted(range(7), key=key)[:k], (t, k)
+        ok = ~torch.isnan(w).any(-1)
+        assert torch.allclose(w[ok].sum(-1), torch.ones(int(ok.sum())), atol=1e-6)
+    w, idx = oracle.routing_topk(logits, 10, torch.float32)
+    full = torch.softmax(logits, -1)
+    assert torch.allclose(w, full.gather(-1, idx), rtol=1e-6, atol=1e-7)
+    # gradient: d_logits[t, idx_j] = w_j (dw_j - sum_i w_i dw_i), zero elsewhere
+    lg = logits.clone().requires_grad_()
+    w, idx = oracle.routing_topk(lg, 3, torch.float32)
+    dw = torch.randn(64, 3)
+    w.backward(dw)
+    wd = w.detach()
+    want = torch.zeros(64, 10).scatter_(1, idx, wd * (dw - (wd * dw).sum(-1, keepdim=True)))
+    assert torch.allclose(lg.grad, want, rtol=1e-5, atol=1e-7)
+
+
 def _random_case(T, E, k, H, I, dtype=torch.float64, seed=0, glu=True):
     g = torch.Generator().manual_seed(seed)
     x = torch.randn(T, H, generator=g, dtype=dtype)
