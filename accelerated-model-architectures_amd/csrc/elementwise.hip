@@ -58,24 +58,38 @@ __global__ __launch_bounds__(EW_THREADS) void combine_bwd_kernel(const uint16_t 
     if (lane == 0) d_w[row] = (uint16_t)(Elem<ET>::pack(acc, 0.f) & 0xffffu);
 }
 
-// out[n, :] = A[idx[n] / fan_out, :] * coeff[idx[n]]
+// out[n, :] = A[idx[n] / fan_out, :] * coeff[idx[n]].  A thread moves one 16-byte chunk of GROUP_ROWS consecutive
+// output rows: the index, coefficient and data loads of the rows are independent, so each of the three dependent
+// round trips is paid once per thread, not once per chunk.
+constexpr int GROUP_ROWS = 4;
 template <typename ET>
 __global__ __launch_bounds__(EW_THREADS) void group_kernel(const uint16_t *__restrict__ A, int64_t lda,
                                                            const int64_t *__restrict__ idx, uint16_t *__restrict__ out,
                                                            int64_t ldo, const uint16_t *__restrict__ coeff, int64_t M,
                                                            int chunks_per_row, int fan_out) {
     const int64_t g = (int64_t)blockIdx.x * EW_THREADS + threadIdx.x;
-    if (g >= M * chunks_per_row) return;
-    const int64_t n = g / chunks_per_row;
+    const int64_t n0 = g / chunks_per_row * GROUP_ROWS;
+    if (n0 >= M) return;
     const int c = (int)(g % chunks_per_row) * 8;
-    const int64_t s = idx[n];
-    u32x4 v = *(const u32x4 *)(A + (s / fan_out) * lda + c);
-    if (coeff) {
-        const float f = Elem<ET>::lo((uint32_t)coeff[s]);
+    int64_t s[GROUP_ROWS];
 #pragma unroll
-        for (int q = 0; q < 4; ++q) v[q] = Elem<ET>::pack(f * Elem<ET>::lo(v[q]), f * Elem<ET>::hi(v[q]));
+    for (int r = 0; r < GROUP_ROWS; ++r) s[r] = idx[n0 + r < M ? n0 + r : M - 1];
+    float f[GROUP_ROWS];
+    u32x4 v[GROUP_ROWS];
+#pragma unroll
+    for (int r = 0; r < GROUP_ROWS; ++r) {
+        f[r] = coeff ? Elem<ET>::lo((uint32_t)coeff[s[r]]) : 1.0f;
+        v[r] = *(const u32x4 *)(A + (s[r] / fan_out) * lda + c);
     }
-    *(u32x4 *)(out + n * ldo + c) = v;
+#pragma unroll
+    for (int r = 0; r < GROUP_ROWS; ++r) {
+        if (n0 + r >= M) break;
+        if (coeff) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[r][q] = Elem<ET>::pack(f[r] * Elem<ET>::lo(v[r][q]), f[r] * Elem<ET>::hi(v[r][q]));
+        }
+        *(u32x4 *)(out + (n0 + r) * ldo + c) = v[r];
+    }
 }
 
 // y[r, c..c+7] from x[r, 2c..2c+15]
@@ -196,7 +210,7 @@ extern "C" int xma_rocm_group(const void *A, int64_t lda, const int64_t *idx, vo
     if (dtype == XMA_ROCM_F32) return f32_group(A, lda, idx, out, ldo, coeff, M, K, fan_out, (hipStream_t)stream);
     const int cpr = K / 8;
     hipStream_t st = (hipStream_t)stream;
-    DISPATCH_T(dtype, (group_kernel<ET><<<grid_for(M * cpr), EW_THREADS, 0, st>>>(
+    DISPATCH_T(dtype, (group_kernel<ET><<<grid_for((M + GROUP_ROWS - 1) / GROUP_ROWS * cpr), EW_THREADS, 0, st>>>(
                           (const uint16_t *)A, lda, idx, (uint16_t *)out, ldo, (const uint16_t *)coeff, M, cpr, fan_out)));
     return xma_check_launch("group_kernel");
 }
