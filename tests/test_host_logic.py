@@ -51,6 +51,15 @@ def test_argument_errors_are_reported_before_any_launch():
     rc = lib.xma_rocm_scatter2scatter(None, 64, None, 64 * 64, 64, 0, None, None, None, 64, None, 0, None, 16, 60, 64, 2, 1, 1, 1,
                                       0, 0, None, 0, None)
     assert rc == -2 and b"multiples of 8" in lib.xma_rocm_last_error()
+    # router: k > E, E and k beyond what a wave holds, row stride shorter than a row, dtype
+    assert lib.xma_rocm_router_topk(None, 8, 4, 8, 9, 0, None, None, 1, None) == -1 and b"k <= E" in lib.xma_rocm_last_error()
+    assert lib.xma_rocm_router_topk(None, 4096, 4, 4096, 2, 0, None, None, 1, None) == -2
+    assert lib.xma_rocm_router_topk(None, 128, 4, 128, 65, 0, None, None, 1, None) == -2
+    assert lib.xma_rocm_router_topk(None, 4, 4, 8, 2, 0, None, None, 1, None) == -1
+    assert lib.xma_rocm_router_topk(None, 8, 4, 8, 2, 5, None, None, 1, None) == -2
+    assert lib.xma_rocm_router_topk(None, 8, 4, 8, 2, 0, None, None, 1, None) == -1  # null pointers with T > 0
+    assert lib.xma_rocm_router_topk_bwd(None, 8, 4, 8, 2, 0, None, 1, None, None, 4, None) == -1  # ldd < E
+    assert lib.xma_rocm_router_topk(None, 8, 0, 8, 2, 0, None, None, 1, None) == 0
     # empty problems are accepted without touching a pointer
     assert lib.xma_rocm_combine(None, 8, None, None, 8, 0, 2, 16, 0, None) == 0
     assert lib.xma_rocm_continuous_count(None, 0, 0, ctypes.c_void_p(16), 4, None, 0, None) == 0
