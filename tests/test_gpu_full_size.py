@@ -1,0 +1,124 @@
+"""The MoE path at the full sizes of the benchmark configurations, where the CPU oracle cannot run a whole step in
+seconds: (1) tokens are independent, so the oracle is run in fp32 on a sample of tokens (first and last rows of every
+expert's group, rows next to tile boundaries, random ones) and compared with those rows of the full-size device
+result (y, dx, d_router_weights); (2) with one weight matrix shared by all experts the layer is a dense MLP scaled by
+the sum of the router weights whatever the routing, so the full result - the weight gradients summed over the experts
+included - is compared with the dense computation by the stock GEMM.
+Tolerance: max-abs-normalised error <= 1e-2 (bf16 results, fp32 accumulation), as for the small cases."""
+
+import pytest
+import torch
+
+from oracle import moe as oracle
+from tests.utils import nerr
+
+pytestmark = pytest.mark.gpu
+
+TOL = 1e-2
+
+CONFIGS = {  # T, H, I, E, k, bias of the router logits (skew)
+    "c3": (8192, 4096, 14336, 8, 2, 0.0),
+    "c4": (16384, 2048, 1408, 64, 6, 1.5),
+    "c5": (32768, 2048, 768, 128, 8, 0.0),
+}
+
+
+def _inputs(name, shared_weights=False):
+    from xma import set_seed
+    from xma.functional import swiglu_packed
+    from xma.layers import MoE
+
+    T, H, I, E, k, bias = CONFIGS[name]
+    set_seed(7)
+    g = torch.Generator(device="cuda").manual_seed(7)
+    with torch.device("meta"):
+        moe = MoE(E, k, H, I, swiglu_packed, True, add_bias=False, std=0.02)
+    moe = moe.to_empty(device="cuda").to(torch.bfloat16)
+    with torch.no_grad():
+        for p in (moe.c_fc.weight, moe.c_proj.weight):
+            if shared_weights:
+                p.copy_((torch.randn(p.shape[1:], generator=g, device="cuda") * 0.02).to(p.dtype).expand_as(p))
+            else:
+                p.copy_((torch.randn(p.shape, generator=g, device="cuda") * 0.02).to(p.dtype))
+    x = torch.randn(T, H, generator=g, device="cuda").to(torch.bfloat16)
+    logits = torch.randn(T, E, generator=g, device="cuda")
+    if bias:
+        logits = logits + bias * torch.randn(E, generator=g, device="cuda")
+    rw, sel = oracle.routing_weights(logits, k, torch.bfloat16)
+    grad = torch.randn(T, H, generator=g, device="cuda").to(torch.bfloat16)
+    return moe, x, rw, sel, grad
+
+
+def _run(moe, x, rw, sel, grad):
+    from xma import KernelBackend
+
+    xd = x.clone().requires_grad_()
+    rwd = rw.clone().requires_grad_()
+    y = moe._compute_experts(xd, rwd, sel, kernel_backend=KernelBackend.rocm)
+    y.backward(grad)
+    torch.cuda.synchronize()
+    return y.detach(), xd.grad, rwd.grad
+
+
+@pytest.mark.parametrize("name", ["c3", "c4", "c5"])
+def test_full_size_sampled_tokens_against_oracle(name):
+    from xma.layers.moe import rocm_implementation as R
+
+    print(f"full size {name}: sampled tokens", flush=True)
+    T, H, I, E, k, _ = CONFIGS[name]
+    moe, x, rw, sel, grad = _inputs(name)
+    y, dx, d_rw = _run(moe, x, rw, sel, grad)
+    assert torch.isfinite(y).all() and torch.isfinite(dx).all() and torch.isfinite(d_rw).all()
+
+    # sample: per expert the first and last row of its group and the rows around every 256-row tile boundary of the
+    # first two tiles, plus random tokens
+    counts, incl, excl, _, ss = R.route(sel, E)
+    incl, excl, ss = incl.cpu(), excl.cpu(), ss.cpu()
+    rows = []
+    for e in range(E):
+        lo, hi = int(excl[e]), int(incl[e])
+        for r in (lo, lo + 255, lo + 256, lo + 511, lo + 512, hi - 1):
+            if lo <= r < hi:
+                rows.append(r)
+    rows = rows[:: max(1, len(rows) // 96)]  # about a hundred rows
+    tokens = set((ss[rows] // k).tolist())
+    gen = torch.Generator().manual_seed(0)
+    tokens |= set(torch.randint(0, T, (32,), generator=gen).tolist())
+    tok = torch.tensor(sorted(tokens))
+    print(f"   {len(tok)} tokens", flush=True)
+
+    xs = x[tok.cuda()].float().cpu().requires_grad_()
+    rws = rw[tok.cuda()].float().cpu().requires_grad_()
+    want = oracle.experts_forward(xs, rws, sel[tok.cuda()].cpu(), moe.c_fc.weight.detach().float().cpu(),
+                                  moe.c_proj.weight.detach().float().cpu(), oracle.swiglu_packed)
+    want.backward(grad[tok.cuda()].float().cpu())
+    for label, got, ref in (("y", y, want.detach()), ("dx", dx, xs.grad), ("d_router_weights", d_rw, rws.grad)):
+        e = nerr(got[tok.cuda()], ref)
+        print(f"   {label}: nerr={e:.2e}", flush=True)
+        assert e <= TOL, f"{name} {label}: {e}"
+
+
+def test_full_size_shared_weights_equal_dense_mlp():
+    """Mixtral-shaped configuration with one weight pair shared by all experts"""
+    print("full size c3: shared weights against the dense MLP", flush=True)
+    T, H, I, E, k, _ = CONFIGS["c3"]
+    moe, x, rw, sel, grad = _inputs("c3", shared_weights=True)
+    y, dx, d_rw = _run(moe, x, rw, sel, grad)
+    dw_fc = moe.c_fc.weight.grad.float().sum(0)
+    dw_proj = moe.c_proj.weight.grad.float().sum(0)
+    moe.c_fc.weight.grad = None
+    moe.c_proj.weight.grad = None
+
+    s = rw.float().sum(-1, keepdim=True)
+    xr = x.clone().requires_grad_()
+    w1 = moe.c_fc.weight[0].detach().clone().requires_grad_()
+    w2 = moe.c_proj.weight[0].detach().clone().requires_grad_()
+    o = oracle.swiglu_packed(xr @ w1.t()) @ w2.t()  # the stock GEMM, bf16 with fp32 accumulation
+    want = (s * o.float()).to(torch.bfloat16)
+    want.backward(grad)
+    want_d_rw = (o.detach().float() * grad.float()).sum(-1, keepdim=True).expand(T, k)
+    for label, got, ref in (("y", y, want.detach()), ("dx", dx, xr.grad), ("d_router_weights", d_rw, want_d_rw),
+                            ("sum of dw_fc", dw_fc, w1.grad), ("sum of dw_proj", dw_proj, w2.grad)):
+        e = nerr(got, ref)
+        print(f"   {label}: nerr={e:.2e}", flush=True)
+        assert e <= TOL, f"{label}: {e}"
