@@ -3,7 +3,8 @@ seconds: (1) tokens are independent, so the oracle is run in fp32 on a sample of
 expert's group, rows next to tile boundaries, random ones) and compared with those rows of the full-size device
 result (y, dx, d_router_weights); (2) with one weight matrix shared by all experts the layer is a dense MLP scaled by
 the sum of the router weights whatever the routing, so the full result - the weight gradients summed over the experts
-included - is compared with the dense computation by the stock GEMM.
+included - is compared with the dense computation by the stock GEMM.  Two further shapes put byte offsets past 2^32
+inside one tensor and 2^20 rows into the grouped order.
 Tolerance: max-abs-normalised error <= 1e-2 (bf16 results, fp32 accumulation), as for the small cases."""
 
 import pytest
@@ -20,6 +21,10 @@ CONFIGS = {  # T, H, I, E, k, bias of the router logits (skew)
     "c3": (8192, 4096, 14336, 8, 2, 0.0),
     "c4": (16384, 2048, 1408, 64, 6, 1.5),
     "c5": (32768, 2048, 768, 128, 8, 0.0),
+    # not a benchmark configuration: 2^18 grouped rows whose pre-activations (and their gradient) take 4.3 GB each, so
+    # that byte offsets inside one tensor pass 2^32; and 2^20 grouped rows of small matrices
+    "over_4_gib": (65536, 512, 4096, 8, 4, 0.0),
+    "many_rows": (262144, 256, 128, 16, 4, 1.0),
 }
 
 
@@ -60,7 +65,7 @@ def _run(moe, x, rw, sel, grad):
     return y.detach(), xd.grad, rwd.grad
 
 
-@pytest.mark.parametrize("name", ["c3", "c4", "c5"])
+@pytest.mark.parametrize("name", ["c3", "c4", "c5", "over_4_gib", "many_rows"])
 def test_full_size_sampled_tokens_against_oracle(name):
     from xma.layers.moe import rocm_implementation as R
 
