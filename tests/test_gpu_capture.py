@@ -50,8 +50,9 @@ def test_compiled_module_matches_eager():
 
 
 def test_graph_capture_and_replay():
-    """fwd + bwd of the expert computation captured once and replayed on new inputs (new routing included); every
-    replay is checked against an eager run, with eager work and synchronisations in between."""
+    """fwd + bwd of the router (behind the gate) and of the expert computation captured once and replayed on new
+    inputs (new routing included); every replay is checked against an eager run, with eager work and synchronisations
+    in between."""
     from xma import KernelBackend
 
     E, k = 8, 2
@@ -60,43 +61,44 @@ def test_graph_capture_and_replay():
     g = torch.Generator(device="cuda").manual_seed(1)
 
     def inputs():
-        logits = torch.randn(T, E, device="cuda", generator=g)
-        vals, sel = logits.topk(k, dim=-1)
-        rw = torch.softmax(vals, dim=-1).to(x.dtype)
+        logits = torch.randn(T, E, device="cuda", generator=g).to(x.dtype)
         xx = torch.randn(T, H, device="cuda", generator=g).to(x.dtype)
         gy = torch.randn(T, H, device="cuda", generator=g).to(x.dtype)
-        return xx, rw, sel, gy
+        return xx, logits, gy
 
-    def step(xx, rw, sel, gy):
+    def step(xx, logits, gy):
+        from xma.layers.moe import rocm_implementation as R
+
         xx = xx.detach().requires_grad_()
-        rw = rw.detach().requires_grad_()
+        logits = logits.detach().requires_grad_()
         for p in (moe.c_fc.weight, moe.c_proj.weight):
             p.grad = None
+        rw, sel = R.router_topk(logits, k)  # top-k + softmax + ids: part of the captured sequence
         y = moe._compute_experts(xx, rw, sel, kernel_backend=KernelBackend.rocm)
         y.backward(gy)
-        return y.detach(), xx.grad, rw.grad, moe.c_fc.weight.grad, moe.c_proj.weight.grad
+        return y.detach(), xx.grad, logits.grad, moe.c_fc.weight.grad, moe.c_proj.weight.grad
 
-    sx, srw, ssel, sgy = inputs()
+    sx, slg, sgy = inputs()
     print("graph: warm-up on a side stream", flush=True)
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
         for _ in range(2):
-            step(sx, srw, ssel, sgy)
+            step(sx, slg, sgy)
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     print("graph: capture", flush=True)
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
-        outs = step(sx, srw, ssel, sgy)
+        outs = step(sx, slg, sgy)
     for it in range(3):
-        nx, nrw, nsel, ngy = inputs()
+        nx, nlg, ngy = inputs()
         print(f"graph: replay {it}", flush=True)
-        sx.copy_(nx), srw.copy_(nrw), ssel.copy_(nsel), sgy.copy_(ngy)
+        sx.copy_(nx), slg.copy_(nlg), sgy.copy_(ngy)
         graph.replay()
         torch.cuda.synchronize()
         got = [o.clone() for o in outs]
-        want = step(nx, nrw, nsel, ngy)  # eager, same kernels
+        want = step(nx, nlg, ngy)  # eager, same kernels
         torch.cuda.synchronize()
-        for a, b, name in zip(got, want, ("y", "dx", "d_router_weights", "dw_fc", "dw_proj")):
+        for a, b, name in zip(got, want, ("y", "dx", "d_router_logits", "dw_fc", "dw_proj")):
             assert torch.equal(a, b), f"replay {it}: {name} differs, nerr {nerr(a, b):.2e}"
