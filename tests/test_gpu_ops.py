@@ -39,6 +39,7 @@ CASES = [
     (513, 6, 4, 72, 40, 2.0, (0, 5)),
     (100, 2, 1, 96, 136, 0.0, ()),  # about 50 rows per expert: two of a wave's four row blocks are computed
     (300, 3, 2, 1096, 320, 0.0, ()),  # few tiles, long K (with a tail): tiles are split into K slices
+    (400, 100, 3, 128, 264, 1.0, (7, 99)),  # more experts than lanes of a wave: the schedule is scanned through LDS
 ]
 
 
