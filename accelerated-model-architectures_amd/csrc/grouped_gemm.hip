@@ -265,9 +265,17 @@ constexpr int SPLIT_MIN_STEPS = 8; // a K slice is at least this many K steps
 // third launch (ROLE_FIXUP, workgroup b = split tile b) adds the slices.  ROLE_TILES takes all other tiles.  Returns
 // false if the workgroup has nothing to do.
 constexpr int ROLE_TILES = 0, ROLE_SLICES = 1, ROLE_FIXUP = 2;
+// Which launches are persistent (one workgroup per compute unit walking its tiles) instead of one workgroup per tile:
+// the dX of the down-projection with its long SwiGLU-backward epilogue measured 3-4 % faster that way on all three
+// benchmark shapes; the up-projection gains or loses about 1 % depending on the shape and the plain-store launches
+// lose 1 % (their tail is cut into K slices by a launch of its own), so those stay as they are.
+__host__ __device__ constexpr bool fwd_persistent(int epi, int role) {
+    return role == ROLE_TILES && epi == XMA_ROCM_EPI_SWIGLU_BWD;
+}
 template <int ROLE>
-__device__ __forceinline__ bool locate_tile(const FwdArgs &a, unsigned char *smem, int *s_sched, TileSched &ts) {
-    const int tid = threadIdx.x, lane = tid & 63;
+__device__ __forceinline__ bool locate_tile(const FwdArgs &a, unsigned char *smem, int *s_sched, TileSched &ts,
+                                            int b, int tid) {
+    const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int NT = (a.N + BN - 1) / BN;
     int full = 0, rest = 0, parts = 1, part = 0, L = 0;
@@ -282,7 +290,6 @@ __device__ __forceinline__ bool locate_tile(const FwdArgs &a, unsigned char *sme
             if (parts > KT / SPLIT_MIN_STEPS) parts = KT / SPLIT_MIN_STEPS;
             if (parts < 2) parts = 1, full = total, rest = 0;
         }
-        const int b = (int)blockIdx.x;
         if (ROLE == ROLE_FIXUP) {
             if ((b >> 2) >= rest) return false; // four workgroups per split tile
             L = full + (b >> 2);
@@ -371,9 +378,9 @@ __device__ __forceinline__ bool locate_tile(const FwdArgs &a, unsigned char *sme
 // ---- epilogue of one 256 x 256 tile (LDS is free: no wave reads operand tiles any more)
 template <typename T, int EPI>
 __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4][4], unsigned char *smem, int64_t row0,
-                                              int rows_valid, int n0, int only_i = -1) {
+                                              int rows_valid, int n0, int tid, int only_i = -1) {
     // only_i >= 0: just the 32-row block only_i of every wave (the fix-up kernel spreads a tile over four workgroups)
-    const int tid = threadIdx.x, lane = tid & 63;
+    const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int wq = (wave & 1) * 128, wp = (wave >> 1) * 128; // wave's 128 x 128 corner inside the tile
     // lane owns row (lane & 31) of each 32-row block; quad g of tile (j, i) holds
@@ -555,11 +562,20 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     __shared__ int s_sched[4];
     u32x4 *tiles = (u32x4 *)smem;
-    const int tid = threadIdx.x, lane = tid & 63;
+    // A persistent launch has one workgroup per compute unit, which walks the tiles b, b + gridDim.x, ... of the launch.
+    const int b_end = fwd_persistent(EPI, ROLE) ? a.grid_main : (int)blockIdx.x + 1;
+    for (int b = blockIdx.x; b < b_end; b += gridDim.x) {
+    if (b != (int)blockIdx.x) __syncthreads(); // the staging areas of the last epilogue are dead in every wave
+    // Everything derived from the thread index is derived again for every tile (the compiler cannot see through the
+    // empty statement): hoisted out of the tile loop, those values would live across the main loop, which has no
+    // register to spare, and be spilled.
+    int tid = threadIdx.x;
+    asm volatile("" : "+v"(tid));
+    const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
     TileSched ts;
-    if (!locate_tile<ROLE>(a, smem, s_sched, ts)) return;
+    if (!locate_tile<ROLE>(a, smem, s_sched, ts, b, tid)) continue;
     const int e = ts.e, rows_valid = ts.rows_valid, n0 = ts.n0;
     const int64_t row0 = ts.row0;
 
@@ -715,8 +731,12 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
                 for (int g = 0; g < 4; ++g)
                     dst[((j * 4 + i) * 4 + g) * GEMM_THREADS] =
                         make_float4(acc[j][i][4 * g], acc[j][i][4 * g + 1], acc[j][i][4 * g + 2], acc[j][i][4 * g + 3]);
-    } else
-        tile_epilogue<T, EPI>(a, acc, smem, row0, rows_valid, n0);
+    } else {
+        int tid_e = threadIdx.x;
+        asm volatile("" : "+v"(tid_e));
+        tile_epilogue<T, EPI>(a, acc, smem, row0, rows_valid, n0, tid_e);
+    }
+    }
 }
 
 // Sum of the K slices of the split tiles of the last round, then the epilogue of the GEMM kernel.  Four workgroups
@@ -728,7 +748,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_fixup_kernel(con
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     __shared__ int s_sched[4];
     TileSched ts;
-    if (!locate_tile<ROLE_FIXUP>(a, smem, s_sched, ts)) return;
+    if (!locate_tile<ROLE_FIXUP>(a, smem, s_sched, ts, (int)blockIdx.x, (int)threadIdx.x)) return;
     const int tid = threadIdx.x;
     const int iblk = blockIdx.x & 3;
     f32x16 acc[4][4];
@@ -747,7 +767,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_fixup_kernel(con
                 }
             }
     }
-    tile_epilogue<T, EPI>(a, acc, smem, ts.row0, ts.rows_valid, ts.n0, iblk);
+    tile_epilogue<T, EPI>(a, acc, smem, ts.row0, ts.rows_valid, ts.n0, (int)threadIdx.x, iblk);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -934,10 +954,16 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
     }
 }
 
+inline int device_cus();
 template <typename T, int WT, int EPI> int launch_fwd(const FwdArgs &a, hipStream_t st) {
     int rc = gemm_set_smem(grouped_gemm_kernel<T, WT, EPI, ROLE_TILES>, GEMM_SMEM_BYTES);
     if (rc) return rc;
-    grouped_gemm_kernel<T, WT, EPI, ROLE_TILES><<<a.grid_main, GEMM_THREADS, GEMM_SMEM_BYTES, st>>>(a);
+    int launch_grid = a.grid_main;
+    if (fwd_persistent(EPI, ROLE_TILES)) {
+        const int cus = device_cus();
+        if (cus > 0 && cus < launch_grid) launch_grid = cus;
+    }
+    grouped_gemm_kernel<T, WT, EPI, ROLE_TILES><<<launch_grid, GEMM_THREADS, GEMM_SMEM_BYTES, st>>>(a);
     if ((rc = xma_check_launch("grouped_gemm_kernel"))) return rc;
     if (!a.partial) return XMA_ROCM_OK;
     // the tiles of the last round as K slices (no epilogue: one instantiation serves all), then their sum + epilogue
