@@ -131,3 +131,32 @@ def test_moe_forward_module_and_state_dict():
     assert nerr(y.view(-1, 256), want) <= TOL
     y2, _ = moe(x, kernel_backend=KernelBackend.torch)
     assert nerr(y2.view(-1, 256), want) <= 2e-2  # the torch path accumulates the k terms in bf16
+
+
+def test_moe_results_are_bitwise_reproducible():
+    """no float atomics anywhere: every output of two runs on the same inputs is identical, also where tiles are split
+    along K (the slices are added in a fixed order) and under skewed routing"""
+    from xma import KernelBackend, set_seed
+    from xma.layers import MoE
+
+    set_seed(11)
+    T, E, k, H, I = 1500, 8, 2, 1096, 320
+    moe = MoE(E, k, H, I, _act("swiglu_packed"), True, add_bias=False, std=0.02).to(torch.bfloat16).cuda()
+    x = torch.randn(T, H, device="cuda").to(torch.bfloat16)
+    logits = torch.randn(T, E, device="cuda") + 1.5 * torch.randn(E, device="cuda")
+    rw, sel = oracle.routing_weights(logits, k, torch.bfloat16)
+    grad = torch.randn(T, H, device="cuda").to(torch.bfloat16)
+
+    def run():
+        for p in moe.parameters():
+            p.grad = None
+        xd, rwd = x.clone().requires_grad_(), rw.clone().requires_grad_()
+        y = moe._compute_experts(xd, rwd, sel, kernel_backend=KernelBackend.rocm)
+        y.backward(grad)
+        torch.cuda.synchronize()
+        return [t.clone() for t in (y.detach(), xd.grad, rwd.grad, moe.c_fc.weight.grad, moe.c_proj.weight.grad)]
+
+    first = run()
+    for _ in range(3):
+        for a, b, name in zip(first, run(), ("y", "dx", "d_router_weights", "dw_fc", "dw_proj")):
+            assert torch.equal(a, b), name
