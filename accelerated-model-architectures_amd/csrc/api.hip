@@ -1,6 +1,10 @@
 // Error slot and version query of the C ABI.
 #include <stdarg.h>
 
+#include <mutex>
+#include <set>
+#include <utility>
+
 #include "common.hpp"
 
 namespace {
@@ -18,6 +22,24 @@ int xma_check_launch(const char *what) {
     hipError_t err = hipGetLastError();
     if (err == hipSuccess) return XMA_ROCM_OK;
     xma_set_error("%s: %s", what, hipGetErrorString(err));
+    return XMA_ROCM_ELAUNCH;
+}
+
+int xma_set_max_lds_once(const void *kernel, int bytes) {
+    static std::mutex lock;
+    static std::set<std::pair<const void *, int>> done; // (kernel, device) pairs whose limit has been raised
+    int dev = 0;
+    hipError_t err = hipGetDevice(&dev);
+    if (err == hipSuccess) {
+        std::lock_guard<std::mutex> guard(lock);
+        if (done.count({kernel, dev})) return XMA_ROCM_OK;
+        err = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (err == hipSuccess) {
+            done.insert({kernel, dev});
+            return XMA_ROCM_OK;
+        }
+    }
+    xma_set_error("hipFuncSetAttribute(max dynamic LDS = %d): %s", bytes, hipGetErrorString(err));
     return XMA_ROCM_ELAUNCH;
 }
 

@@ -19,6 +19,8 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 // ---------------------------------------------------------------- error slot
 void xma_set_error(const char *fmt, ...);
 int xma_check_launch(const char *what);
+// hipFuncSetAttribute(MaxDynamicSharedMemorySize) on the first call per (kernel, device); later calls only look it up
+int xma_set_max_lds_once(const void *kernel, int bytes);
 
 #define XMA_REQUIRE(cond, code, ...)   \
     do {                               \

@@ -64,14 +64,8 @@ __device__ __forceinline__ int xcd_remap(int bid, int grid) {
     return (bid & ~255) + (w & 7) * 32 + (w >> 3);
 }
 
-template <typename K> inline int gemm_set_smem(K kernel, int bytes) {
-    hipError_t err = hipFuncSetAttribute((const void *)kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-    if (err != hipSuccess) {
-        xma_set_error("hipFuncSetAttribute(max dynamic LDS = %d): %s", bytes, hipGetErrorString(err));
-        return XMA_ROCM_ELAUNCH;
-    }
-    return XMA_ROCM_OK;
-}
+// Raises a kernel's dynamic-LDS limit; the attribute belongs to (kernel, device) and is set on the first launch only.
+template <typename K> inline int gemm_set_smem(K kernel, int bytes) { return xma_set_max_lds_once((const void *)kernel, bytes); }
 
 // dW with a per-token scale on dY (register-staged loader, grouped_gemm_staged.hip)
 int launch_dw_scaled(const DwArgs &a, int dtype, int grid, hipStream_t st);

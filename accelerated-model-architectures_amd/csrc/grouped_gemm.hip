@@ -36,6 +36,8 @@
 // Epilogues (plain store with optional row scale and scatter, SwiGLU forward, SwiGLU backward) stage every 32-row block
 // of a wave's corner in wave-private LDS and write whole rows: in the accumulator layout a store instruction would
 // touch 32 rows with 16 bytes each.
+#include <atomic>
+
 #include "fp32.hpp"
 #include "gemm_common.hpp"
 
@@ -775,6 +777,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_fixup_kernel(con
 // runs over the expert's row range, k-rows past its end come from the zero page.
 //   GQ / GP = 1: the rows of dY / X are taken through sorted_scattered_idxs (index / fan_out); 0: grouped order
 // ------------------------------------------------------------------------------------------------
+constexpr int DW_BAND = 4;
 template <typename T, int GQ, int GP>
 __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const DwArgs a) {
     constexpr int GATHER = GQ | GP;
@@ -783,10 +786,15 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int OT = (a.N_out + 255) / 256, IT = (a.K_in + 255) / 256;
+    // Tile walk: inside an expert the tiles are taken in bands of DW_BAND tile rows, down the band first, so that the 32
+    // consecutive tiles an XCD gets from xcd_remap form a DW_BAND x (32 / DW_BAND) block that shares DW_BAND dY panels and
+    // 32 / DW_BAND X panels in that XCD's L2 (a row-by-row walk shares 1 + 32).
     const int L = xcd_remap(blockIdx.x, gridDim.x);
     const int e = L / (OT * IT);
     const int rem = L % (OT * IT);
-    const int o0 = (rem / IT) * 256, i0 = (rem % IT) * 256;
+    const int band = rem / (DW_BAND * IT), in_band = rem % (DW_BAND * IT);
+    const int band_rows = (OT - band * DW_BAND < DW_BAND) ? OT - band * DW_BAND : DW_BAND;
+    const int o0 = (band * DW_BAND + in_band % band_rows) * 256, i0 = (in_band / band_rows) * 256;
     const int64_t row_lo = e ? a.offs[e - 1] : 0, row_hi = a.offs[e];
     const int rows = (int)(row_hi - row_lo);
     const int KT = (rows + BK - 1) / BK;
@@ -1000,15 +1008,15 @@ template <typename T> int dispatch_fwd(const FwdArgs &a, int wt, int epi, hipStr
 
 // Compute units of the current device (tiles that run at the same time), looked up once per device.
 inline int device_cus() {
-    static int cached[64] = {0};
+    static std::atomic<int> cached[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-    if (cached[dev] == 0) {
-        int n = 0;
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
         if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
-        cached[dev] = n;
+        cached[dev].store(n, std::memory_order_relaxed); // every thread that races here stores the same value
     }
-    return cached[dev];
+    return n;
 }
 
 // Launches of fewer rounds than this may split the tiles of their last round over the idle CUs.

@@ -5,6 +5,7 @@
 
 namespace xma_rocm {
 
+
 constexpr int HIST_THREADS = 512;
 constexpr int HIST_LDS_WORDS = 8192;  // 32 KB of counters per workgroup
 constexpr int HIST_MAX_BLOCKS = 256;  // partial histograms of the two-pass path
@@ -327,12 +328,7 @@ int route_launch(const IdT *ids, int64_t n, int E, uint32_t *counts, int64_t *in
     int nbits = 0;
     while ((1 << nbits) < E) ++nbits;
     const size_t lds3 = route_scatter_lds(E);
-    hipError_t err = hipFuncSetAttribute((const void *)route_scatter_kernel<IdT>,
-                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds3);
-    if (err != hipSuccess) {
-        xma_set_error("route: hipFuncSetAttribute(%zu bytes of LDS): %s", lds3, hipGetErrorString(err));
-        return XMA_ROCM_ELAUNCH;
-    }
+    if (xma_set_max_lds_once((const void *)route_scatter_kernel<IdT>, (int)route_scatter_lds(ROUTE_MAX_E))) return XMA_ROCM_ELAUNCH;
     int rc;
     const int stride = E | 1;
     int copies = 1;
