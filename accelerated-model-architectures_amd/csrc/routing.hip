@@ -1,10 +1,17 @@
 // Expert histogram (continuous_count) and the one-op routing (counts, offsets, stable expert-major permutation) for
 // gfx950.  HBM-bound integer work: wide coalesced loads, LDS-privatised counters, wave64 ballots for stable ranks,
 // LDS-staged output so that the scatter leaves the workgroup as contiguous runs.
+#include <mutex>
+
 #include "common.hpp"
 
 namespace xma_rocm {
 
+// Scratch of xma_rocm_route_static: the per-unit histograms live in this file-scope device array instead of a caller's
+// workspace, so that entry point allocates nothing.  Every GPU the library runs on holds its own copy at its own address
+// until the process ends; in host code the name is only a handle for hipGetSymbolAddress, never a device address.
+constexpr size_t ROUTE_STATIC_WORDS = (size_t)1 << 18; // 1 MiB: units x experts <= 262144
+static __device__ __align__(256) uint32_t scratch[ROUTE_STATIC_WORDS];
 
 constexpr int HIST_THREADS = 512;
 constexpr int HIST_LDS_WORDS = 8192;  // 32 KB of counters per workgroup
@@ -400,6 +407,59 @@ extern "C" size_t xma_rocm_route_workspace_bytes(int64_t n, int32_t num_experts)
     int64_t units = (n + ROUTE_CHUNK - 1) / ROUTE_CHUNK;
     if (units < 1) units = 1;
     return (size_t)units * (size_t)num_experts * sizeof(uint32_t);
+}
+
+// Device address of `scratch` on the current device, looked up once per device (with that device current).
+static int route_static_scratch(uint32_t **out) {
+    constexpr int MAX_DEVICES = 64;
+    static std::mutex lock;
+    static uint32_t *ptr[MAX_DEVICES] = {nullptr};
+    int dev = 0;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+        xma_set_error("route_static: hipGetDevice: %s (device %d)", hipGetErrorString(err), dev);
+        return XMA_ROCM_ELAUNCH;
+    }
+    std::lock_guard<std::mutex> guard(lock);
+    if (!ptr[dev]) {
+        uint32_t *p = nullptr;
+        err = hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || !p) {
+            xma_set_error("route_static: hipGetSymbolAddress(scratch): %s", hipGetErrorString(err));
+            return XMA_ROCM_ELAUNCH;
+        }
+        ptr[dev] = p;
+    }
+    *out = ptr[dev];
+    return XMA_ROCM_OK;
+}
+
+extern "C" size_t xma_rocm_route_static_max_units_times_experts(void) { return ROUTE_STATIC_WORDS; }
+
+extern "C" int xma_rocm_route_static(const void *ids, int ids_are_int64, int64_t n, int32_t E, uint32_t *counts,
+                                     int64_t *offsets_inclusive, int64_t *offsets_exclusive, void *sorted_expert_idxs,
+                                     int64_t *sorted_scattered_idxs, void *stream) {
+    XMA_REQUIRE(n >= 0 && E >= 1 && E <= ROUTE_MAX_E, XMA_ROCM_EINVAL, "route_static: n=%lld E=%d (E <= %d)",
+                (long long)n, E, ROUTE_MAX_E);
+    XMA_REQUIRE(n < (int64_t)1 << 31, XMA_ROCM_EUNSUPPORTED, "route_static: n=%lld does not fit 31 bits", (long long)n);
+    XMA_REQUIRE(counts && offsets_inclusive && (n == 0 || (ids && sorted_scattered_idxs)), XMA_ROCM_EINVAL,
+                "route_static: null pointer");
+    const size_t need = xma_rocm_route_workspace_bytes(n, E);
+    XMA_REQUIRE(need <= ROUTE_STATIC_WORDS * sizeof(uint32_t), XMA_ROCM_EWORKSPACE,
+                "route_static: ceil(n / %d) * E = %zu exceeds the static scratch of %zu words; use xma_rocm_route with a "
+                "workspace",
+                ROUTE_CHUNK, need / sizeof(uint32_t), ROUTE_STATIC_WORDS);
+    uint32_t *ws = nullptr;
+    int rc = route_static_scratch(&ws);
+    if (rc) return rc;
+    // every word of the scratch that the scatter reads is written by the unit histogram pass of the same call: nothing
+    // of an earlier call is carried over, nothing has to be cleared
+    hipStream_t st = (hipStream_t)stream;
+    if (ids_are_int64)
+        return route_launch<int64_t>((const int64_t *)ids, n, E, counts, offsets_inclusive, offsets_exclusive,
+                                     (int64_t *)sorted_expert_idxs, sorted_scattered_idxs, ws, st);
+    return route_launch<int32_t>((const int32_t *)ids, n, E, counts, offsets_inclusive, offsets_exclusive,
+                                 (int32_t *)sorted_expert_idxs, sorted_scattered_idxs, ws, st);
 }
 
 extern "C" int xma_rocm_route(const void *ids, int ids_are_int64, int64_t n, int32_t E, uint32_t *counts,

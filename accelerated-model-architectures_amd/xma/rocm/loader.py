@@ -33,6 +33,8 @@ SIGNATURES = {
     "xma_rocm_continuous_count": (_int, [_p, _int, _i64, _p, _i32, _p, _sz, _p]),
     "xma_rocm_route_workspace_bytes": (_sz, [_i64, _i32]),
     "xma_rocm_route": (_int, [_p, _int, _i64, _i32, _p, _p, _p, _p, _p, _p, _sz, _p]),
+    "xma_rocm_route_static_max_units_times_experts": (_sz, []),
+    "xma_rocm_route_static": (_int, [_p, _int, _i64, _i32, _p, _p, _p, _p, _p, _p]),
     "xma_rocm_scatter2scatter_workspace_bytes": (_sz, [_i64, _i32, _i32, _i32]),
     "xma_rocm_scatter2scatter": (
         _int,

@@ -85,6 +85,20 @@ XMA_API int xma_rocm_route(const void *ids, int ids_are_int64, int64_t n, int32_
                    int64_t *sorted_scattered_idxs, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
+ * xma_rocm_route without a workspace argument and without any allocation.  It has no counterpart in the reference; it
+ * is for callers that cannot allocate device memory around the call (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  Same arguments, results and kernels as xma_rocm_route; the per-unit
+ * histograms live in a device array that is part of the library image (1 MiB per GPU, held until the process ends).
+ * Limit: ceil(n / 4096) * num_experts <= xma_rocm_route_static_max_units_times_experts() (= 262144; e.g. 4 Mi ids
+ * over 256 experts); larger problems return XMA_ROCM_EWORKSPACE and must use xma_rocm_route.  All calls on one GPU
+ * share that array: calls that overlap on one GPU (two streams, two threads) race and must be serialised by the caller.
+ */
+XMA_API size_t xma_rocm_route_static_max_units_times_experts(void);
+XMA_API int xma_rocm_route_static(const void *ids, int ids_are_int64, int64_t n, int32_t num_experts, uint32_t *counts,
+                          int64_t *offsets_inclusive, int64_t *offsets_exclusive, void *sorted_expert_idxs,
+                          int64_t *sorted_scattered_idxs, void *stream);
+
+/*
  * Grouped GEMM with fused row gather / scatter: for every expert e and every
  * grouped position n in [offsets[e-1], offsets[e]):
  *     acc[n, :] = X[src(n), :K] @ B_e            B_e = W[e]^T  if !w_is_kn   (W[e] is (N, K), K contiguous)

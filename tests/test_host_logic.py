@@ -46,6 +46,12 @@ def test_argument_errors_are_reported_before_any_launch():
     assert lib.xma_rocm_continuous_count(None, 0, 10, None, 0, None, 0, None) == -1
     assert b"continuous_count" in lib.xma_rocm_last_error()
     assert lib.xma_rocm_route(None, 0, 10, 100000, None, None, None, None, None, None, 0, None) == -1
+    # the entry point with static scratch refuses what does not fit its array, before touching the device
+    assert lib.xma_rocm_route_static_max_units_times_experts() == 1 << 18
+    big = ctypes.c_void_p(256)
+    assert lib.xma_rocm_route_static(big, 0, 4096 * 129, 2048, big, big, None, None, big, None) == -3
+    assert b"static scratch" in lib.xma_rocm_last_error()
+    assert lib.xma_rocm_route_static(None, 0, 10, 100000, None, None, None, None, None, None) == -1
     assert lib.xma_rocm_combine(None, 8, None, None, 8, 4, 2, 12, 0, None) == -1  # H % 8 != 0
     assert lib.xma_rocm_combine(None, 8, None, None, 8, 4, 2, 16, 7, None) == -2  # dtype
     rc = lib.xma_rocm_scatter2scatter(None, 64, None, 64 * 64, 64, 0, None, None, None, 64, None, 0, None, 16, 60, 64, 2, 1, 1, 1,
