@@ -5,6 +5,7 @@ the Python host loads with ctypes.  No torch headers, no JIT cache."""
 from __future__ import annotations
 
 import os
+import re
 import subprocess
 import sys
 from concurrent.futures import ThreadPoolExecutor
@@ -15,7 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 OUT_DIR = os.path.join(HERE, "xma", "rocm")
 LIB = os.path.join(OUT_DIR, "libxma_rocm.so")
-SOURCES = ["api.hip", "routing.hip", "elementwise.hip", "grouped_gemm.hip", "grouped_gemm_staged.hip", "fp32.hip", "router.hip"]
+SOURCES = ["api.hip", "routing.hip", "elementwise.hip", "grouped_gemm.hip", "grouped_gemm_staged.hip", "fp32.hip", "router.hip", "swiglu.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
@@ -27,31 +28,110 @@ FLAGS = [
     "-fvisibility=hidden",
     # keep the compiler from forming packed fp32 VALU ops
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # per-kernel register, scratch and LDS figures on stderr (parsed below)
+    "-Rpass-analysis=kernel-resource-usage",
     "-I", CSRC,
     "-I", INCLUDE,
 ]
 
+# The grouped GEMM kernels keep 256 accumulators in AGPRs next to an almost full VGPR file and hand-placed waits around
+# asynchronous inline-assembly loads: a register that the compiler spills or reloads inside the MFMA loop, behind those
+# waits, would corrupt data silently (a few spills in prologue and epilogue, where nothing asynchronous is live, are
+# harmless).  The build therefore reads the generated ISA of those kernels and fails if a scratch access sits between
+# the first and the last MFMA of one of them, and says so if the compiler is not the version the kernels were written
+# and measured with.
+LOOP_NO_SCRATCH = {"grouped_gemm.hip": re.compile(r"grouped_gemm")}
+TESTED_HIPCC = "7.2"
+USAGE_REPORT = os.path.join(HERE, "build", "kernel_resource_usage.txt")
+
+
+def _scratch_inside_mfma_loop(asm_path: str, which: re.Pattern) -> list[str]:
+    """kernels matching `which` whose ISA has a scratch access between their first and last MFMA"""
+    bad, name, first, last, scratch = [], None, None, None, []
+
+    def close():
+        if name and first is not None and any(first < n < last for n in scratch):
+            bad.append(name)
+
+    with open(asm_path) as f:
+        for n, line in enumerate(f):
+            m = re.match(r"^(_Z\w+):\s*(;.*)?$", line)
+            if m:
+                close()
+                name = m.group(1) if which.search(m.group(1)) else None
+                first, last, scratch = None, None, []
+            elif name:
+                if "v_mfma" in line:
+                    first = n if first is None else first
+                    last = n
+                elif "scratch_" in line:
+                    scratch.append(n)
+    close()
+    return bad
+
+
+def _resource_usage(stderr: str) -> dict[str, dict[str, str]]:
+    """{kernel: {field: value}} from the -Rpass-analysis=kernel-resource-usage remarks"""
+    out: dict[str, dict[str, str]] = {}
+    cur = None
+    for line in stderr.splitlines():
+        m = re.search(r"remark:\s+(Function Name|[A-Za-z ]+(?: \[[^\]]*\])?):\s*(\S+)", line)
+        if not m:
+            continue
+        key, val = m.group(1).strip(), m.group(2)
+        if key == "Function Name":
+            cur = out.setdefault(val, {})
+        elif cur is not None:
+            cur[key] = val
+    return out
+
+
+def _check_compiler(verbose: bool) -> None:
+    r = subprocess.run([HIPCC, "--version"], capture_output=True, text=True)
+    m = re.search(r"HIP version:\s*(\S+)", r.stdout)
+    version = m.group(1) if m else "unknown"
+    if not version.startswith(TESTED_HIPCC):
+        print(f"build.py: warning: hipcc {version}, the kernels were written and measured with {TESTED_HIPCC}.x; "
+              f"re-run the GPU parity tests before trusting this build", file=sys.stderr)
+    elif verbose:
+        print(f"hipcc {version}", flush=True)
+
 
 def _compile(src: str, verbose: bool) -> str:
     obj = os.path.join(HERE, "build", src.replace(".hip", ".o"))
-    cmd = [HIPCC, *FLAGS, "-c", os.path.join(CSRC, src), "-o", obj]
+    extra = ["-save-temps=obj"] if src in LOOP_NO_SCRATCH else []  # keeps the device ISA next to the object
+    cmd = [HIPCC, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
     if verbose:
         print(" ".join(cmd), flush=True)
     r = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
-    err = "\n".join(l for l in r.stderr.splitlines() if noise not in l)
+    usage = _resource_usage(r.stderr)
+    err = "\n".join(l for l in r.stderr.splitlines() if noise not in l and "kernel-resource-usage" not in l)
+    err = re.sub(r"(?m)^\s*\d+ \|.*\n\s*\| \^\s*$\n?", "", err)  # source excerpts under the remarks
     if r.returncode != 0:
         raise RuntimeError(f"hipcc failed on {src}:\n{err}")
-    if err.strip() and verbose:
+    if re.search(r"warning|error", err) and verbose:
         print(err, file=sys.stderr)
-    return obj
+    if src in LOOP_NO_SCRATCH:
+        asm = os.path.join(HERE, "build", src.replace(".hip", "-hip-amdgcn-amd-amdhsa-gfx950.s"))
+        bad = _scratch_inside_mfma_loop(asm, LOOP_NO_SCRATCH[src])
+        if bad:
+            raise RuntimeError(f"{src}: scratch accesses inside the MFMA loop of:\n  " + "\n  ".join(bad))
+    return obj, usage
 
 
 def build(verbose: bool = False) -> str:
     os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
     os.makedirs(OUT_DIR, exist_ok=True)
+    _check_compiler(verbose)
     with ThreadPoolExecutor(max_workers=4) as pool:
-        objs = list(pool.map(lambda s: _compile(s, verbose), SOURCES))
+        results = list(pool.map(lambda s: _compile(s, verbose), SOURCES))
+    objs = [o for o, _ in results]
+    with open(USAGE_REPORT, "w") as f:
+        for _, usage in results:
+            for k, v in usage.items():
+                f.write(f"{k}: VGPRs {v.get('VGPRs')} AGPRs {v.get('AGPRs')} scratch {v.get('ScratchSize [bytes/lane]')} "
+                        f"LDS {v.get('LDS Size [bytes/block]')} occupancy {v.get('Occupancy [waves/SIMD]')}\n")
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     if verbose:
         print(" ".join(cmd), flush=True)

@@ -30,6 +30,36 @@ int xma_set_max_lds_once(const void *kernel, int bytes);
         }                              \
     } while (0)
 
+// ---------------------------------------------------------------- division by a launch constant
+// exact n / d for 0 <= n < 2^31 in three 32-bit instructions: with s = ceil(log2 d) and magic = ceil(2^(31+s) / d)
+// (which fits 32 bits), n / d = mulhi(2 n, magic) >> s
+struct FastDiv {
+    uint32_t magic;
+    int shift;
+};
+inline FastDiv make_fastdiv(uint32_t d) {
+    int s = 0;
+    while ((1u << s) < d) ++s;
+    FastDiv f;
+    f.shift = s;
+    f.magic = (uint32_t)((((uint64_t)1 << (31 + s)) + d - 1) / d);
+    return f;
+}
+__device__ __forceinline__ uint32_t fastdiv(uint32_t n, FastDiv f) { return __umulhi(n << 1, f.magic) >> f.shift; }
+
+// Index of a lane's piece of work -> (row, piece inside the row) for rows of `per_row` pieces: the multiply-high form
+// while the index fits 31 bits, the 64-bit division (a hundred instructions) only beyond that.
+__device__ __forceinline__ void split_row(int64_t g, int per_row, FastDiv d, int64_t &row, int &piece) {
+    if (g < ((int64_t)1 << 31)) {
+        const uint32_t r = fastdiv((uint32_t)g, d);
+        row = r;
+        piece = (int)((uint32_t)g - r * (uint32_t)per_row);
+    } else {
+        row = g / per_row;
+        piece = (int)(g % per_row);
+    }
+}
+
 // ---------------------------------------------------------------- element traits
 template <typename T> struct Elem;
 

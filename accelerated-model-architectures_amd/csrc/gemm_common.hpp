@@ -6,22 +6,6 @@
 constexpr int BM = 256, BN = 256; // output tile of every grouped GEMM kernel
 constexpr int GEMM_THREADS = 256;
 
-// exact n / d for 0 <= n < 2^31 in three 32-bit instructions: with s = ceil(log2 d) and magic = ceil(2^(31+s) / d)
-// (which fits 32 bits), n / d = mulhi(2 n, magic) >> s
-struct FastDiv {
-    uint32_t magic;
-    int shift;
-};
-inline FastDiv make_fastdiv(uint32_t d) {
-    int s = 0;
-    while ((1u << s) < d) ++s;
-    FastDiv f;
-    f.shift = s;
-    f.magic = (uint32_t)((((uint64_t)1 << (31 + s)) + d - 1) / d);
-    return f;
-}
-__device__ __forceinline__ uint32_t fastdiv(uint32_t n, FastDiv f) { return __umulhi(n << 1, f.magic) >> f.shift; }
-
 struct FwdArgs {
     const uint16_t *X;
     int64_t ldx;
@@ -36,6 +20,7 @@ struct FwdArgs {
     const uint16_t *scale;
     int64_t M;
     int N, K, E, fan_out, x_grouped, y_grouped;
+    FastDiv fan_div; // division of a scattered index by fan_out (indices are below 2^31)
     float *partial;  // workspace for the K slices of the tiles of the last round, or NULL (no tile is split)
     int split_cus;   // compute units of the device = tiles per round
     int grid_main;   // workgroups that take whole tiles (an upper bound of the tile count); split_cus more follow

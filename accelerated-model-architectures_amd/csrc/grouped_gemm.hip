@@ -76,39 +76,46 @@ template <int N, typename F> __device__ __forceinline__ void static_for(F &&f) {
 
 // ---- LDS layouts (byte offsets inside one 32 KB operand tile)
 //
-// Row-major tile [256 rows][8 chunks of 16 B]: chunk c of row r sits at slot c ^ (r & 7).  An LDS-DMA instruction
-// covers 8 rows (1 KB); wave w loads rows 64 w + 8 i + (lane >> 3), i = 0..7, and lane fills slot lane & 7, i.e. it
-// fetches logical chunk (lane & 7) ^ (lane >> 3) - the same for every i, so a lane's global address of piece i is a
-// fixed per-lane pointer plus the K offset of the step.
-__device__ __forceinline__ int rowmajor_lane_chunk(int lane) { return (lane & 7) ^ (lane >> 3); }
-// MFMA fragment of rows R0 + 32 i + (lane & 31), k16 sub-step kk: since R0 and 32 i are multiples of 8 the slot is
-// ((2 kk + (lane >> 5)) ^ (lane & 7)): one per-lane byte offset per kk, and i is an immediate (4096 i).
+// The LDS serves 16 lanes of a ds_read_b128 (32 lanes of a 64-bit read) at a time from 64 banks of 4 bytes, so the 16-byte
+// pieces those lanes ask for must fall on 16 different positions modulo 256 bytes.  Both layouts below are arranged for
+// that (measured with the fragment patterns alone, 4 waves per CU: 344 bytes/ns/CU against 281 for swizzles that only
+// spread 8 consecutive lanes over 128 bytes).
+//
+// Row-major tile [256 rows][8 chunks of 16 B]: chunk c of row r sits at slot c ^ ((r >> 1) & 7); rows 2 m and 2 m + 1
+// share the permutation and are 128 bytes apart.  An LDS-DMA instruction covers 8 rows (1 KB); wave w loads rows
+// 64 w + 8 i + (lane >> 3), i = 0..7, and lane fills slot lane & 7, i.e. it fetches logical chunk
+// (lane & 7) ^ (4 (i & 1) + (lane >> 4)): one of two per-lane constants, so a lane's global address of piece i is a fixed
+// per-lane pointer plus the K offset of the step.
+__device__ __forceinline__ int rowmajor_lane_chunk(int i, int lane) { return (lane & 7) ^ (((i & 1) << 2) + (lane >> 4)); }
+// MFMA fragment of rows R0 + 32 i + (lane & 31), k16 sub-step kk: R0 and 32 i are multiples of 16, so the slot is
+// ((2 kk + (lane >> 5)) ^ ((lane >> 1) & 7)): one per-lane byte offset per kk, and i is an immediate (4096 i).
 __device__ __forceinline__ uint32_t rowmajor_frag_offset(int R0, int kk, int lane) {
-    return (uint32_t)((R0 + (lane & 31)) * 128 + (((2 * kk + (lane >> 5)) ^ (lane & 7)) << 4));
+    return (uint32_t)((R0 + (lane & 31)) * 128 + (((2 * kk + (lane >> 5)) ^ ((lane >> 1) & 7)) << 4));
 }
 //
 // Transposed tile [64 k-rows][32 chunks of 16 B], exactly as in memory: chunk c of k-row kr sits at slot
-// c ^ ((kr & 3) << 1).  An LDS-DMA instruction covers 2 k-rows; wave w loads k-rows 16 w + 2 j + (lane >> 5), j = 0..7,
-// and lane fills slot lane & 31, i.e. it fetches logical chunk (lane & 31) ^ (((2 j + (lane >> 5)) & 3) << 1).
+// c ^ ((kr & 3) << 2).  An LDS-DMA instruction covers 2 k-rows; wave w loads k-rows 16 w + 2 j + (lane >> 5), j = 0..7,
+// and lane fills slot lane & 31, i.e. it fetches logical chunk (lane & 31) ^ (((2 j + (lane >> 5)) & 3) << 2).
 __device__ __forceinline__ int transposed_lane_chunk(int j, int lane) {
-    return (lane & 31) ^ (((2 * j + (lane >> 5)) & 3) << 1);
+    return (lane & 31) ^ (((2 * j + (lane >> 5)) & 3) << 2);
 }
 // MFMA fragment through ds_read_b64_tr_b16, which works on groups of 16 lanes: lane p of a group supplies the
 // address of 4 columns at one k-row and receives 4 consecutive k of one column.  With
 // p -> (k-row kb + p / 4, columns mb + 4 (p % 4)) lane p ends up with column mb + p, k = kb .. kb + 3; two reads
-// (kb and kb + 4) give the 8 k of an MFMA operand.  For the 32-row block i of the wave's 128 rows the chunk index is
-// (R0 / 8 + 4 i + c_lane) ^ s with s in {0, 2, 4, 6}: blocks 0 and 1 need one per-lane offset each, blocks 2 and 3
-// are those plus 128 bytes; kk adds 8192 bytes, the second read 2048.
-__device__ __forceinline__ uint32_t transposed_frag_offset(int R0, int odd, int lane) {
+// (kb and kb + 4) give the 8 k of an MFMA operand.  A pass of 32 lanes (groups 0 and 1: 32 columns at 4 k-rows) reads
+// eight 32-byte pieces; the column pair picks bit 1 of the chunk index, the k-row bits 2 and 3, so they are 8
+// different positions modulo 256 bytes.  The 32-row block i of the wave's 128 rows adds 4 i to the chunk index, which
+// the XOR does not commute with: one per-lane offset per block; kk adds 8192 bytes, the second read 2048.
+__device__ __forceinline__ uint32_t transposed_frag_offset(int R0, int blk, int lane) {
     const int p = lane & 15, G = lane >> 4;
-    const int m = R0 + odd * 32 + ((G & 1) << 4) + ((p & 3) << 2);
+    const int m = R0 + blk * 32 + ((G & 1) << 4) + ((p & 3) << 2);
     const int kr = ((G >> 1) << 3) + (p >> 2);
-    return (uint32_t)(kr * 512 + ((((m >> 3) ^ ((kr & 3) << 1))) << 4) + ((m & 7) << 1));
+    return (uint32_t)(kr * 512 + ((((m >> 3) ^ ((kr & 3) << 2))) << 4) + ((m & 7) << 1));
 }
 
 // per-lane LDS byte addresses of one operand's fragments in the CURRENT stage
 template <int TR> struct FragBase {
-    uint32_t b[TR ? 2 : 4]; // row-major: one per kk; transposed: blocks 0/2 and blocks 1/3
+    uint32_t b[4]; // row-major: one per kk; transposed: one per 32-row block
 };
 
 template <int TR> __device__ __forceinline__ void make_frag_base(FragBase<TR> &f, uint32_t tile_lds_addr, int R0, int lane) {
@@ -116,13 +123,13 @@ template <int TR> __device__ __forceinline__ void make_frag_base(FragBase<TR> &f
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) f.b[kk] = tile_lds_addr + rowmajor_frag_offset(R0, kk, lane);
     } else {
-        f.b[0] = tile_lds_addr + transposed_frag_offset(R0, 0, lane);
-        f.b[1] = tile_lds_addr + transposed_frag_offset(R0, 1, lane);
+#pragma unroll
+        for (int blk = 0; blk < 4; ++blk) f.b[blk] = tile_lds_addr + transposed_frag_offset(R0, blk, lane);
     }
 }
 template <int TR> __device__ __forceinline__ void flip_stage(FragBase<TR> &f) {
 #pragma unroll
-    for (int q = 0; q < (TR ? 2 : 4); ++q) f.b[q] ^= (uint32_t)(STAGE_CHUNKS * 16);
+    for (int q = 0; q < 4; ++q) f.b[q] ^= (uint32_t)(STAGE_CHUNKS * 16);
 }
 
 // All fragment reads are inline assembly with an immediate offset: (1) after an LDS-DMA load the compiler guards every
@@ -136,10 +143,8 @@ template <int TR, int I, int KK> __device__ __forceinline__ u32x4 read_frag(cons
         return r;
     } else {
         u32x2 lo, hi;
-        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(lo) : "v"(f.b[I & 1]), "n"(KK * 8192 + (I >> 1) * 128));
-        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2"
-                     : "=v"(hi)
-                     : "v"(f.b[I & 1]), "n"(KK * 8192 + (I >> 1) * 128 + 2048));
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(lo) : "v"(f.b[I]), "n"(KK * 8192));
+        asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2" : "=v"(hi) : "v"(f.b[I]), "n"(KK * 8192 + 2048));
         u32x4 r = {lo[0], lo[1], hi[0], hi[1]};
         return r;
     }
@@ -590,7 +595,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
     const int kt0 = (ROLE == ROLE_SLICES) ? ((ts.part * KT / ts.parts) & ~1) : 0;
     const int kt1 = (ROLE == ROLE_SLICES && ts.part + 1 < ts.parts) ? (((ts.part + 1) * KT / ts.parts) & ~1) : KT;
     const uint16_t *q_ptr[8], *p_ptr[8];
-    const int c_lane = rowmajor_lane_chunk(lane);
     {
         const uint16_t *We = a.W + (int64_t)e * a.w_es;
         if (WT == 0) {
@@ -598,7 +602,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
             for (int i = 0; i < 8; ++i) {
                 int r = n0 + wave * 64 + i * 8 + (lane >> 3);
                 if (r >= a.N) r = a.N - 1;
-                p_ptr[i] = We + (int64_t)r * a.ldw + c_lane * 8;
+                p_ptr[i] = We + (int64_t)r * a.ldw + rowmajor_lane_chunk(i, lane) * 8;
             }
         } else {
             const int max_chunk = ((a.N - n0) >> 3) - 1; // last valid 16-byte chunk of the tile's column range
@@ -633,7 +637,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
             if (k_tail && kt == KT - 1) { // uniform branch, taken by at most one step of a tile
                 asm volatile("" ::: "memory"); // keeps this rare path a branch instead of selects in every piece
                 if (piece < 8 || WT == 0) {
-                    if (kt * BK + rowmajor_lane_chunk(lane) * 8 >= a.K) src = zero;
+                    if (kt * BK + rowmajor_lane_chunk(piece & 7, lane) * 8 >= a.K) src = zero;
                 } else {
                     if (kt * BK + wave * 16 + 2 * (piece - 8) + (lane >> 5) >= a.K) src = zero;
                 }
@@ -658,8 +662,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
         int r = wave * 64 + i * 8 + (lane >> 3);
         if (r >= rows_valid) r = rows_valid - 1; // duplicates, masked at the store
         const int64_t n = row0 + r;
-        const int64_t src = a.x_grouped ? n : a.idx[n] / a.fan_out;
-        q_ptr[i] = a.X + src * a.ldx + c_lane * 8;
+        const int64_t src = a.x_grouped ? n : (int64_t)fastdiv((uint32_t)a.idx[n], a.fan_div);
+        q_ptr[i] = a.X + src * a.ldx + rowmajor_lane_chunk(i, lane) * 8;
     }
     static_for<8>([&](auto P) { issue_piece(kt0, P, IC<0>{}); });
     static_for<DMA_N0>([&](auto P) { issue_piece(kt0 + 1, P, IC<0>{}); });
@@ -790,8 +794,24 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
     // consecutive tiles an XCD gets from xcd_remap form a DW_BAND x (32 / DW_BAND) block that shares DW_BAND dY panels and
     // 32 / DW_BAND X panels in that XCD's L2 (a row-by-row walk shares 1 + 32).
     const int L = xcd_remap(blockIdx.x, gridDim.x);
-    const int e = L / (OT * IT);
     const int rem = L % (OT * IT);
+    // Experts are taken in the order of decreasing row count (equal counts: lower index first), the longest K loops
+    // first: a tile's duration is proportional to its expert's rows, and with skewed routing a large expert that came up
+    // last would keep a few compute units busy long after all others have finished.  Every wave ranks the experts in
+    // registers (lane = expert); with more experts than lanes the order stays the index order.
+    int e = L / (OT * IT);
+    if (a.E <= WAVE) {
+        const int64_t hi = a.offs[lane < a.E ? lane : a.E - 1];
+        int64_t lo = __shfl_up(hi, 1);
+        if (lane == 0) lo = 0;
+        const int cnt = (lane < a.E) ? (int)(hi - lo) : -1;
+        int rank = 0;
+        for (int i = 0; i < a.E; ++i) {
+            const int ci = __builtin_amdgcn_readlane(cnt, i);
+            rank += (ci > cnt || (ci == cnt && i < lane)) ? 1 : 0;
+        }
+        e = __builtin_ctzll(__ballot(rank == e && lane < a.E)); // exactly one lane
+    }
     const int band = rem / (DW_BAND * IT), in_band = rem % (DW_BAND * IT);
     const int band_rows = (OT - band * DW_BAND < DW_BAND) ? OT - band * DW_BAND : DW_BAND;
     const int o0 = (band * DW_BAND + in_band % band_rows) * 256, i0 = (in_band / band_rows) * 256;
@@ -1085,6 +1105,7 @@ extern "C" int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *
     a.K = K;
     a.E = E;
     a.fan_out = fan_out;
+    a.fan_div = make_fastdiv((uint32_t)fan_out);
     a.x_grouped = x_grouped;
     a.y_grouped = y_grouped;
     a.partial = nullptr;

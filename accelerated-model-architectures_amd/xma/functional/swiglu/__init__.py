@@ -1,8 +1,9 @@
 """swiglu / swiglu_packed with the reference's signatures
 (xma/functional/swiglu/__init__.py:39-87).  The torch branch restates
-xma/functional/swiglu/torch_implementation.py:9-30; the rocm branch of the
-packed form runs the stand-alone HIP kernels.  ``swiglu_packed`` is also the
-activation the MoE layer recognises and fuses into its grouped GEMMs."""
+xma/functional/swiglu/torch_implementation.py:9-30; the rocm branch runs the
+stand-alone HIP kernels (any 2-D size, bf16 / fp16 / fp32, forward and
+backward).  ``swiglu_packed`` is also the activation the MoE layer recognises
+and fuses into its grouped GEMMs."""
 
 from __future__ import annotations
 
@@ -50,6 +51,39 @@ class _SwigluPackedROCm(torch.autograd.Function):
         return dx
 
 
+def _row_major_2d(t: torch.Tensor) -> torch.Tensor:
+    """2-D view with contiguous rows (any row pitch is fine for the kernels; anything else is copied)"""
+    t = t.reshape(-1, t.size(-1)) if t.dim() != 2 else t
+    return t if t.stride(1) == 1 or t.size(1) == 1 else t.contiguous()
+
+
+class _SwigluROCm(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, g: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
+        from ...rocm.ops import swiglu_forward_rocm
+
+        g, u = _row_major_2d(g), _row_major_2d(u)
+        y = torch.empty(g.shape, dtype=g.dtype, device=g.device)
+        swiglu_forward_rocm(g=g, u=u, y=y)
+        ctx.save_for_backward(g, u)
+        return y
+
+    @staticmethod
+    def backward(ctx, dy: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+        from ...rocm.ops import swiglu_backward_rocm
+
+        g, u = ctx.saved_tensors
+        dg = torch.empty(g.shape, dtype=g.dtype, device=g.device)
+        du = torch.empty(u.shape, dtype=u.dtype, device=u.device)
+        swiglu_backward_rocm(g=g, u=u, dy=_row_major_2d(dy), dg=dg, du=du)
+        return dg, du
+
+
+def _check_rocm_dtype(x: torch.Tensor, what: str) -> None:
+    if x.dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise NotImplementedError(f"{what} on KernelBackend.rocm covers bf16/fp16/fp32 (got {x.dtype})")
+
+
 def swiglu(gate: torch.Tensor, up: torch.Tensor, *, kernel_backend: KernelBackend | None = None) -> torch.Tensor:
     """computes swiglu activation as `up * gate * sigmoid(gate)`"""
     assert gate.size() == up.size(), "tensors gate and up should have same shape"
@@ -57,9 +91,11 @@ def swiglu(gate: torch.Tensor, up: torch.Tensor, *, kernel_backend: KernelBacken
 
     kernel_backend = _resolve(kernel_backend, gate)
     if kernel_backend == KernelBackend.rocm:
-        # the separate-operand form has no dedicated kernel: interleave and use the packed one
-        packed = torch.stack([gate, up], dim=-1).flatten(-2)
-        return swiglu_packed(packed, kernel_backend=kernel_backend)
+        _check_rocm_dtype(gate, "swiglu")
+        original_shape = gate.size()
+        if gate.numel() == 0:
+            return torch.empty_like(gate)
+        return _SwigluROCm.apply(gate.reshape(-1, original_shape[-1]), up.reshape(-1, original_shape[-1])).view(original_shape)
     if kernel_backend == KernelBackend.torch:
         return _swiglu_torch(gate, up)
     raise ValueError(f"unexpected kernel_backend ({kernel_backend})")
@@ -73,11 +109,7 @@ def swiglu_packed(x: torch.Tensor, *, kernel_backend: KernelBackend | None = Non
 
     kernel_backend = _resolve(kernel_backend, x)
     if kernel_backend == KernelBackend.rocm:
-        if x.dtype not in (torch.bfloat16, torch.float16, torch.float32) or H % 8 != 0:
-            raise NotImplementedError(
-                f"swiglu_packed on KernelBackend.rocm covers bf16/fp16/fp32 with an output width that is a multiple of "
-                f"8 (got {x.dtype}, {H})"
-            )
+        _check_rocm_dtype(x, "swiglu_packed")
         y = _SwigluPackedROCm.apply(x.flatten(0, -2))
     elif kernel_backend == KernelBackend.torch:
         y = _swiglu_packed_torch(x.flatten(0, -2))

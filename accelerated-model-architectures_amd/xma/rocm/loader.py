@@ -32,6 +32,7 @@ SIGNATURES = {
     "xma_rocm_continuous_count_workspace_bytes": (_sz, [_i64, _i32]),
     "xma_rocm_continuous_count": (_int, [_p, _int, _i64, _p, _i32, _p, _sz, _p]),
     "xma_rocm_route_workspace_bytes": (_sz, [_i64, _i32]),
+    "xma_rocm_route_set_rank_method": (_int, [_int]),
     "xma_rocm_route": (_int, [_p, _int, _i64, _i32, _p, _p, _p, _p, _p, _p, _sz, _p]),
     "xma_rocm_route_static_max_units_times_experts": (_sz, []),
     "xma_rocm_route_static": (_int, [_p, _int, _i64, _i32, _p, _p, _p, _p, _p, _p]),
@@ -50,6 +51,8 @@ SIGNATURES = {
     "xma_rocm_combine_bwd": (_int, [_p, _i64, _p, _i64, _p, _i64, _i32, _i32, _int, _p]),
     "xma_rocm_swiglu_packed_forward": (_int, [_p, _i64, _p, _i64, _i64, _i32, _int, _p]),
     "xma_rocm_swiglu_packed_backward": (_int, [_p, _i64, _p, _i64, _p, _i64, _i64, _i32, _int, _p]),
+    "xma_rocm_swiglu_forward": (_int, [_p, _i64, _p, _i64, _p, _i64, _i64, _i32, _int, _p]),
+    "xma_rocm_swiglu_backward": (_int, [_p, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _i64, _i32, _int, _p]),
     "xma_rocm_router_topk": (_int, [_p, _i64, _i64, _i32, _i32, _int, _p, _p, _int, _p]),
     "xma_rocm_router_topk_bwd": (_int, [_p, _i64, _i64, _i32, _i32, _int, _p, _int, _p, _p, _i64, _p]),
 }

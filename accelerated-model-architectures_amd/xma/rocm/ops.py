@@ -308,6 +308,34 @@ def swiglu_packed_backward_rocm(x: torch.Tensor, dy: torch.Tensor, dx: torch.Ten
     )
 
 
+# --------------------------------------------------------------------------- stand-alone SwiGLU, separate operands
+@torch.library.custom_op("xma_rocm::swiglu_forward", mutates_args={"y"})
+def swiglu_forward_rocm(g: torch.Tensor, u: torch.Tensor, y: torch.Tensor) -> None:
+    """y = u * g * sigmoid(g) over 2-D tensors of any size (reference op: _Swiglu, swiglu/__init__.py:15, 39-63)."""
+    rows, cols = y.shape
+    assert g.shape == u.shape == y.shape and g.dtype == u.dtype == y.dtype
+    lib = get_library()
+    check(
+        lib.xma_rocm_swiglu_forward(_ptr(g), _rows(g, "g"), _ptr(u), _rows(u, "u"), _ptr(y), _rows(y, "y"), rows, cols,
+                                    _code(g), _stream(g)),
+        "xma_rocm_swiglu_forward",
+    )
+
+
+@torch.library.custom_op("xma_rocm::swiglu_backward", mutates_args={"dg", "du"})
+def swiglu_backward_rocm(g: torch.Tensor, u: torch.Tensor, dy: torch.Tensor, dg: torch.Tensor, du: torch.Tensor) -> None:
+    """(dg, du) of swiglu_forward_rocm (closed form of swiglu/triton_implementation/backward.py:14-23)."""
+    rows, cols = dy.shape
+    assert g.shape == u.shape == dy.shape == dg.shape == du.shape
+    assert g.dtype == u.dtype == dy.dtype == dg.dtype == du.dtype
+    lib = get_library()
+    check(
+        lib.xma_rocm_swiglu_backward(_ptr(g), _rows(g, "g"), _ptr(u), _rows(u, "u"), _ptr(dy), _rows(dy, "dy"), _ptr(dg),
+                                     _rows(dg, "dg"), _ptr(du), _rows(du, "du"), rows, cols, _code(g), _stream(g)),
+        "xma_rocm_swiglu_backward",
+    )
+
+
 # --------------------------------------------------------------------------- router behind the gate GEMM
 @torch.library.custom_op("xma_rocm::router_topk", mutates_args={"weights", "ids"})
 def router_topk_rocm(logits: torch.Tensor, weights: torch.Tensor, ids: torch.Tensor) -> None:

@@ -80,6 +80,12 @@ XMA_API int xma_rocm_continuous_count(const void *ids, int ids_are_int64, int64_
  * ids must lie in [0, E); E <= 2048.
  */
 XMA_API size_t xma_rocm_route_workspace_bytes(int64_t n, int32_t num_experts);
+/*
+ * How the scatter kernel of xma_rocm_route finds the stable rank of an id among equal ids of its wave (process-wide,
+ * takes effect with the next call): 0 (default) = value returned by an LDS atomic add, which gfx950 applies in lane
+ * order; 1 = log2(E) wave ballots per 64 ids, which relies on no ordering property of the hardware.  Results are bit-identical; the switch exists so that the claim can be tested on any machine.
+ */
+XMA_API int xma_rocm_route_set_rank_method(int method);
 XMA_API int xma_rocm_route(const void *ids, int ids_are_int64, int64_t n, int32_t num_experts, uint32_t *counts,
                    int64_t *offsets_inclusive, int64_t *offsets_exclusive, void *sorted_expert_idxs,
                    int64_t *sorted_scattered_idxs, void *workspace, size_t workspace_bytes, void *stream);
@@ -174,11 +180,24 @@ XMA_API int xma_rocm_combine_bwd(const void *expert_out, int64_t ld_in, const vo
  *     y[r, c] = u * g * sigmoid(g),  g = x[r, 2c], u = x[r, 2c + 1]
  * and its closed-form backward.  Replaces xma/functional/swiglu/torch_implementation.py:21-30
  * and xma/functional/swiglu/triton_implementation/backward.py:14-23 for the packed layout.
+ * Any cols_out >= 1 and any row pitch; rows whose starts are 16-byte aligned move as 16-byte accesses.
  */
 XMA_API int xma_rocm_swiglu_packed_forward(const void *x, int64_t ldx, void *y, int64_t ldy, int64_t rows, int32_t cols_out,
                                    int dtype, void *stream);
 XMA_API int xma_rocm_swiglu_packed_backward(const void *x, int64_t ldx, const void *dy, int64_t lddy, void *dx,
                                     int64_t lddx, int64_t rows, int32_t cols_out, int dtype, void *stream);
+
+/*
+ * Stand-alone SwiGLU on separate operands, y = up * gate * sigmoid(gate) over (rows, cols) with fp32 math, and its
+ * backward d_gate = dy * up * (s + g s (1 - s)), d_up = dy * g * s with s = sigmoid(gate).  Replaces _Swiglu.run,
+ * xma/functional/swiglu/__init__.py:39-63 (torch form: torch_implementation.py:9-18; backward:
+ * triton_implementation/backward.py:14-23).  Any 2-D size and row pitch, bf16 / fp16 / fp32.
+ */
+XMA_API int xma_rocm_swiglu_forward(const void *gate, int64_t ld_gate, const void *up, int64_t ld_up, void *y, int64_t ldy,
+                            int64_t rows, int32_t cols, int dtype, void *stream);
+XMA_API int xma_rocm_swiglu_backward(const void *gate, int64_t ld_gate, const void *up, int64_t ld_up, const void *dy,
+                             int64_t lddy, void *d_gate, int64_t ld_dgate, void *d_up, int64_t ld_dup, int64_t rows,
+                             int32_t cols, int dtype, void *stream);
 
 /*
  * Router behind the gate GEMM: for each of T rows of E expert logits, the k largest values in descending order

@@ -28,7 +28,7 @@ CONFIGS = {  # T, H, I, E, k, bias of the router logits (skew)
 }
 
 
-def _inputs(name, shared_weights=False):
+def _inputs(name, shared_weights=False, empty_expert=None):
     from xma import set_seed
     from xma.functional import swiglu_packed
     from xma.layers import MoE
@@ -49,6 +49,8 @@ def _inputs(name, shared_weights=False):
     logits = torch.randn(T, E, generator=g, device="cuda")
     if bias:
         logits = logits + bias * torch.randn(E, generator=g, device="cuda")
+    if empty_expert is not None:
+        logits[:, empty_expert] = -1e9  # never selected
     rw, sel = oracle.routing_weights(logits, k, torch.bfloat16)
     grad = torch.randn(T, H, generator=g, device="cuda").to(torch.bfloat16)
     return moe, x, rw, sel, grad
@@ -101,6 +103,45 @@ def test_full_size_sampled_tokens_against_oracle(name):
         e = nerr(got[tok.cuda()], ref)
         print(f"   {label}: nerr={e:.2e}", flush=True)
         assert e <= TOL, f"{name} {label}: {e}"
+
+
+@pytest.mark.parametrize("name", ["c3", "c4", "c5"])
+def test_full_size_weight_gradients_per_expert(name):
+    """dW of single experts at full size.  An expert's weight gradients depend only on its own tokens, so the fp32 oracle
+    is run on exactly those tokens as a one-expert layer (k = 1, router weight = the weight of the slot that chose the
+    expert) and compared with that expert's slices of the device's dw_fc and dw_proj, each normalised by its own
+    maximum: the smallest non-empty expert, the largest and one in the middle.  A wrong expert -> slice mapping or a bad
+    ragged K tail shows here even if it cancels in the sum over experts.  One expert is left without tokens: its
+    slices must be exact zeros."""
+    from xma.layers.moe import rocm_implementation as R
+
+    print(f"full size {name}: per-expert weight gradients", flush=True)
+    T, H, I, E, k, _ = CONFIGS[name]
+    empty = E // 2
+    moe, x, rw, sel, grad = _inputs(name, empty_expert=empty)
+    _run(moe, x, rw, sel, grad)
+    dw_fc, dw_proj = moe.c_fc.weight.grad, moe.c_proj.weight.grad
+    assert torch.isfinite(dw_fc).all() and torch.isfinite(dw_proj).all()
+    counts, incl, excl, _, ss = R.route(sel, E)
+    counts = counts.cpu().view(torch.int32).tolist()
+    assert counts[empty] == 0
+    assert float(dw_fc[empty].abs().max()) == 0.0 and float(dw_proj[empty].abs().max()) == 0.0
+    order = sorted((c, e) for e, c in enumerate(counts) if c > 0)
+    picks = {order[0][1], order[len(order) // 2][1], order[-1][1]}
+    for e in sorted(picks):
+        idx = ss[int(excl[e]) : int(incl[e])]
+        tok, flat_w = idx // k, rw.flatten()[idx]
+        n = idx.numel()
+        want = oracle.experts_forward_backward(
+            x[tok].cpu(), flat_w.view(n, 1).cpu(), torch.zeros(n, 1, dtype=torch.int64),
+            moe.c_fc.weight.detach()[e : e + 1].cpu(), moe.c_proj.weight.detach()[e : e + 1].cpu(), oracle.swiglu_packed,
+            grad[tok].cpu(), compute_dtype=torch.float32,
+        )
+        e1, e2 = nerr(dw_fc[e], want["dw_fc"][0]), nerr(dw_proj[e], want["dw_proj"][0])
+        print(f"   expert {e} ({n} rows): dw_fc nerr={e1:.2e} dw_proj nerr={e2:.2e}", flush=True)
+        assert e1 <= TOL and e2 <= TOL, (name, e, e1, e2)
+    moe.c_fc.weight.grad = None
+    moe.c_proj.weight.grad = None
 
 
 def test_full_size_shared_weights_equal_dense_mlp():

@@ -154,6 +154,72 @@ def test_swiglu_packed_standalone(dtype):
         assert nerr(xd.grad, want) <= _tol(dtype)
 
 
+def _2d_sizes():
+    """the reference's 2-D size rule (tests/utils.py:31-42: squares 2^i + j, and ragged sizes around 3000), thinned so
+    that the CPU oracle stays within seconds"""
+    import random
+
+    rng = random.Random(0)
+    sizes = [(2**i + j, 2**i + j) for i in range(11) for j in (0, 1, 3, 7, 9)]
+    ragged = [(3000 + rng.randint(-1000, 1000), 3000 + rng.randint(-1000, 1000)) for _ in range(50)]
+    return sizes + ragged[:8]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_swiglu_two_operands(dtype):
+    """swiglu(gate, up) on separate operands, forward and backward, over the reference's 2-D size grid
+    (tests/functional/swiglu_test.py:62-95: integer-valued inputs in [-8, 8), fp32 atol 7e-5 / 4.6e-5) - odd widths,
+    widths below one 16-byte access, rows that are not 16-byte aligned - against the oracle's closed forms."""
+    from xma import KernelBackend
+    from xma.functional import swiglu
+
+    g = torch.Generator().manual_seed(11)
+    for rows, cols in _2d_sizes():
+        print(f"swiglu case {rows}x{cols} {dtype}", flush=True)
+        gate = torch.randint(-8, 8, (rows, cols), generator=g).to(dtype)
+        up = torch.randint(-8, 8, (rows, cols), generator=g).to(dtype)
+        dy = torch.randn(rows, cols, generator=g).to(dtype)
+        gd, ud = gate.cuda().requires_grad_(), up.cuda().requires_grad_()
+        y = swiglu(gd, ud, kernel_backend=KernelBackend.rocm)
+        y.backward(dy.cuda())
+        want = oracle.swiglu(gate.float(), up.float())
+        dg, du = oracle.swiglu_backward(gate.float(), up.float(), dy.float())
+        assert y.dtype == dtype and y.shape == (rows, cols)
+        assert nerr(y, want) <= _tol(dtype), (rows, cols)
+        assert nerr(gd.grad, dg) <= _tol(dtype) and nerr(ud.grad, du) <= _tol(dtype), (rows, cols)
+        if dtype == torch.float32:
+            assert (y.cpu() - want).abs().max() <= 7e-5
+            assert (gd.grad.cpu() - dg).abs().max() <= 4.6e-5 * dy.abs().max() * 4
+
+
+def test_swiglu_views_and_shapes():
+    """3-D inputs, operands that are column slices of one wider tensor (row pitch larger than the width, starts not
+    16-byte aligned), empty input; and the packed form at widths that are not multiples of 8."""
+    from xma import KernelBackend
+    from xma.functional import swiglu, swiglu_packed
+
+    g = torch.Generator().manual_seed(12)
+    for dtype in (torch.bfloat16, torch.float32):
+        x = (torch.randn(3, 37, 2 * 203, generator=g) * 2).to(dtype)
+        xd = x.cuda()
+        for lo in (0, 1, 8):  # chunk-style halves of one tensor; lo shifts the alignment of the row starts
+            gate, up = x[..., lo:203], x[..., 203 + lo :]
+            y = swiglu(xd[..., lo:203], xd[..., 203 + lo :], kernel_backend=KernelBackend.rocm)
+            assert y.shape == gate.shape
+            assert nerr(y, oracle.swiglu(gate.float(), up.float())) <= _tol(dtype)
+        for cols in (1, 3, 12, 203, 1001):
+            xp = (torch.randn(5, 29, 2 * cols, generator=g) * 2).to(dtype)
+            dy = torch.randn(5, 29, cols, generator=g).to(dtype)
+            xpd = xp.cuda().requires_grad_()
+            y = swiglu_packed(xpd, kernel_backend=KernelBackend.rocm)
+            y.backward(dy.cuda())
+            assert nerr(y, oracle.swiglu_packed(xp.float())) <= _tol(dtype), cols
+            dg, du = oracle.swiglu_backward(xp[..., 0::2].float(), xp[..., 1::2].float(), dy.float())
+            assert nerr(xpd.grad, torch.stack([dg, du], dim=-1).flatten(-2)) <= _tol(dtype), cols
+        empty = torch.empty(0, 16, dtype=dtype, device="cuda")
+        assert swiglu(empty, empty, kernel_backend=KernelBackend.rocm).shape == (0, 16)
+
+
 def test_scatter2scatter_with_and_without_workspace():
     """The same launch through the C ABI with the scratch for splitting the last round of tiles along K and without
     it (every tile by one workgroup): both within tolerance of the oracle; the workspace query and its error code."""

@@ -125,3 +125,29 @@ def test_route_moe_shapes():
         logits = torch.randn(T, E, generator=g) + bias * torch.randn(E, generator=g)
         sel = logits.topk(k, dim=-1).indices
         _check_route(sel.flatten(), E)
+
+
+def test_route_rank_methods_agree():
+    """The scatter kernel has two ways to rank an id among the equal ids of its wave: the value returned by an LDS atomic
+    add (relies on gfx950 applying the lanes of one instruction in lane order) and wave ballots (relies on nothing).
+    Both must give the oracle's stable permutation, bit for bit, on uniform, skewed, sorted and single-expert ids."""
+    from xma.rocm import get_library
+
+    lib = get_library()
+    g = torch.Generator().manual_seed(9)
+    cases = [
+        (torch.randint(0, 64, (1 << 20,), generator=g, dtype=torch.int32), 64),
+        (zipf_ids(300001, 64, 1.1, 3), 64),
+        (torch.randint(0, 128, (70000,), generator=g, dtype=torch.int64).sort().values, 128),
+        (torch.full((20000,), 2, dtype=torch.int32), 3),
+        (torch.randint(0, 1000, (50000,), generator=g, dtype=torch.int64), 1000),
+    ]
+    try:
+        for method in (1, 0):
+            assert lib.xma_rocm_route_set_rank_method(method) == 0
+            for ids, E in cases:
+                print(f"rank method {method}: n={ids.numel()} E={E}", flush=True)
+                _check_route(ids, E)
+        assert lib.xma_rocm_route_set_rank_method(2) == -1
+    finally:
+        lib.xma_rocm_route_set_rank_method(0)

@@ -32,7 +32,7 @@ def test_library_exports_every_declared_symbol():
     assert lib.xma_rocm_abi_version() == 1
     # host-only entry points (no GPU work)
     assert lib.xma_rocm_route_workspace_bytes(4 * 1024 * 1024, 64) == (4 * 1024 * 1024 // 4096) * 64 * 4
-    assert lib.xma_rocm_continuous_count_workspace_bytes(4 * 1024 * 1024, 64) == 256 * 64 * 4
+    assert lib.xma_rocm_continuous_count_workspace_bytes(4 * 1024 * 1024, 64) == 1024 * 64 * 4
     assert lib.xma_rocm_continuous_count_workspace_bytes(1000, 64) == 0
     assert lib.xma_rocm_route_workspace_bytes(0, 8) == 8 * 4
     assert lib.xma_rocm_route_workspace_bytes(-1, 8) == 0
