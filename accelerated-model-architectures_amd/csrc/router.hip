@@ -93,8 +93,8 @@ template <int G> __device__ __forceinline__ float group_softmax(float my_val, in
 template <int DT> struct Cand {
     uint32_t packed; // key16 << 16 | (0xffff - index)
     static __device__ __forceinline__ Cand none() { return {0u}; }
-    static __device__ __forceinline__ Cand make(const void *row, int e) {
-        const uint32_t b = ((const uint16_t *)row)[e];
+    static __device__ __forceinline__ Cand make(const void *row, int e) { return from_bits(((const uint16_t *)row)[e], e); }
+    static __device__ __forceinline__ Cand from_bits(uint32_t b, int e) {
         const uint32_t inf = (DT == XMA_ROCM_BF16) ? 0x7f80u : 0x7c00u;
         uint32_t key;
         if ((b & 0x7fffu) > inf)
@@ -218,6 +218,148 @@ __global__ __launch_bounds__(RT_THREADS) void router_topk_bwd_kernel(const void 
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// Gate projection fused with the router: logits = x @ Wg^T (fp32 accumulation, rounded to the activation dtype as the
+// stock linear layer does), then top-k, fp32 softmax and expert ids from the rounded logits, in one kernel
+// (xma/layers/moe/__init__.py:182-195, 256-262).  x (T, H) is streamed from HBM exactly once; Wg (E, H) stays in cache.
+//
+// A workgroup of 4 waves takes 32 tokens and splits H into four K ranges, one per wave, so that even a layer of a few
+// thousand tokens puts four waves on every SIMD and keeps enough loads in flight.  A wave multiplies its 32 x (H / 4)
+// slice of x with Wg by v_mfma_f32_32x32x16 (tokens = register dimension, experts = lanes, NB blocks of 32 experts); both
+// operands come straight from global memory, 64 contiguous bytes per lane and K step - a step's 64 k are dealt to the two
+// half-waves as 32 + 32, which is the same permutation of k for both operands and therefore leaves the product unchanged.
+// The four partial results meet in LDS; wave w then owns 8 of the 32 tokens: their logits sit across the 32 lanes of a
+// half-wave, NB per lane, exactly the layout the selection network of router_topk_kernel works on (G = 32).
+// ------------------------------------------------------------------------------------------------
+constexpr int RG_THREADS = 256, RG_TOKENS = 32, RG_MAX_E = 128, RG_MAX_K = 32;
+
+template <typename T, int DT, int NB>
+__global__ __launch_bounds__(RG_THREADS) void router_gate_topk_kernel(const uint16_t *__restrict__ x, int64_t ldx,
+                                                                      const uint16_t *__restrict__ wg, int64_t ldw,
+                                                                      int64_t n_tokens, int H, int E, int k,
+                                                                      uint16_t *__restrict__ logits, int64_t ldl,
+                                                                      void *__restrict__ weights, void *__restrict__ ids,
+                                                                      int ids_i64) {
+    __shared__ float s_part[4][16 * NB][64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r = lane & 31, half = lane >> 5;
+    const int64_t t0 = (int64_t)blockIdx.x * RG_TOKENS;
+    const int64_t my_t = (t0 + r < n_tokens) ? t0 + r : n_tokens - 1; // clamped: rows past the end are never stored
+    const int steps = (H + 63) / 64;
+    const int s_begin = wave * steps / 4, s_end = (wave + 1) * steps / 4;
+    const uint16_t *xrow = x + my_t * ldx + half * 32;
+    const uint16_t *wrow[NB];
+    bool w_ok[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+        const int e = b * 32 + r;
+        w_ok[b] = e < E;
+        wrow[b] = wg + (int64_t)(w_ok[b] ? e : E - 1) * ldw + half * 32;
+    }
+    struct Stage {
+        u32x4 xa[4];
+        u32x4 wb[NB][4];
+    };
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+    auto fetch = [&](Stage &st, int step) {
+        const int k0 = step * 64;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const bool in = k0 + half * 32 + 8 * q < H; // H is a multiple of 8: a 16-byte chunk is inside or outside
+            st.xa[q] = in ? *(const u32x4 *)(xrow + k0 + 8 * q) : zero4;
+#pragma unroll
+            for (int b = 0; b < NB; ++b) st.wb[b][q] = (in && w_ok[b]) ? *(const u32x4 *)(wrow[b] + k0 + 8 * q) : zero4;
+        }
+    };
+    f32x16 acc[NB];
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[b][v] = 0.f;
+    auto multiply = [&](const Stage &st) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int b = 0; b < NB; ++b) acc[b] = Elem<T>::mfma(st.xa[q], st.wb[b][q], acc[b]);
+    };
+    // two stages of operands in registers: the loads of step s + 1 are in flight while step s multiplies
+    Stage s0, s1;
+    if (s_begin < s_end) fetch(s0, s_begin);
+    for (int step = s_begin; step < s_end; step += 2) {
+        if (step + 1 < s_end) fetch(s1, step + 1);
+        multiply(s0);
+        if (step + 1 < s_end) {
+            if (step + 2 < s_end) fetch(s0, step + 2);
+            multiply(s1);
+        }
+    }
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s_part[wave][b * 16 + v][lane] = acc[b][v];
+    __syncthreads();
+
+    // wave w finishes accumulator slots v = 4 w .. 4 w + 3: in slot v the lanes of half h hold token
+    // 8 (v / 4) + 4 h + v % 4 of the tile, lane r of the half the experts 32 b + r
+    const int g = r;
+    for (int vv = 0; vv < 4; ++vv) {
+        const int v = 4 * wave + vv;
+        const int64_t t = t0 + 8 * (v >> 2) + 4 * half + (v & 3);
+        const bool live = t < n_tokens;
+        Cand<DT> c[NB];
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const float sum = (s_part[0][b * 16 + v][lane] + s_part[1][b * 16 + v][lane]) +
+                              (s_part[2][b * 16 + v][lane] + s_part[3][b * 16 + v][lane]);
+            const uint32_t bits = Elem<T>::pack(sum, 0.f) & 0xffffu;
+            const int e = b * 32 + r;
+            if (live && e < E) logits[t * ldl + e] = (uint16_t)bits;
+            c[b] = (live && e < E) ? Cand<DT>::from_bits(bits, e) : Cand<DT>::none();
+        }
+        Cand<DT> mine = Cand<DT>::none();
+        for (int round = 0; round < k; ++round) {
+            Cand<DT> best = c[0];
+#pragma unroll
+            for (int b = 1; b < NB; ++b)
+                if (c[b].beats(best)) best = c[b];
+            best = best.template group_best<32>();
+            const int be = best.index();
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+                if (b * 32 + r == be && !best.is_none()) c[b] = Cand<DT>::none(); // taken
+            if (g == round) mine = best;
+        }
+        const float w = group_softmax<32>(mine.value(), g, k, lane - g);
+        if (live && g < k) {
+            Scalar<DT>::store(weights, t * k + g, w);
+            if (ids_i64)
+                ((int64_t *)ids)[t * k + g] = mine.index();
+            else
+                ((int32_t *)ids)[t * k + g] = mine.index();
+        }
+    }
+}
+
+template <typename T, int DT>
+int router_gate_launch(const void *x, int64_t ldx, const void *wg, int64_t ldw, int64_t n_tokens, int H, int E, int k,
+                       void *logits, int64_t ldl, void *weights, void *ids, int ids_i64, hipStream_t st) {
+    const unsigned grid = (unsigned)((n_tokens + RG_TOKENS - 1) / RG_TOKENS);
+#define RG_LAUNCH(NB)                                                                                                   \
+    router_gate_topk_kernel<T, DT, NB><<<grid, RG_THREADS, 0, st>>>((const uint16_t *)x, ldx, (const uint16_t *)wg, ldw, \
+                                                                    n_tokens, H, E, k, (uint16_t *)logits, ldl, weights, \
+                                                                    ids, ids_i64)
+    if (E <= 32)
+        RG_LAUNCH(1);
+    else if (E <= 64)
+        RG_LAUNCH(2);
+    else if (E <= 96)
+        RG_LAUNCH(3);
+    else
+        RG_LAUNCH(4);
+#undef RG_LAUNCH
+    return xma_check_launch("router_gate_topk_kernel");
+}
+
 struct RouterShape {
     int G, vpl;
     int64_t blocks;
@@ -289,6 +431,35 @@ extern "C" int xma_rocm_router_topk(const void *logits, int64_t ld, int64_t T, i
     ROUTER_DISPATCH(dtype, s, (router_topk_kernel<DT, G, VPL><<<(int)s.blocks, RT_THREADS, 0, st>>>(
                                   logits, ld, T, E, k, weights, ids, ids_is_i64)));
     return xma_check_launch("router_topk_kernel");
+}
+
+extern "C" int xma_rocm_router_gate_topk_supported(int32_t H, int32_t E, int32_t k, int dtype) {
+    return (dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16) && H >= 8 && H % 8 == 0 && E >= 1 && E <= RG_MAX_E && k >= 1 &&
+           k <= E && k <= RG_MAX_K;
+}
+
+extern "C" int xma_rocm_router_gate_topk(const void *x, int64_t ldx, const void *gate_weight, int64_t ldw, int64_t T,
+                                         int32_t H, int32_t E, int32_t k, int dtype, void *logits, int64_t ldl,
+                                         void *weights, void *ids, int ids_is_i64, void *stream) {
+    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED,
+                "router_gate_topk: dtype %d (bf16 and fp16 only; fp32 goes through a linear layer and xma_rocm_router_topk)",
+                dtype);
+    XMA_REQUIRE(T >= 0 && H >= 8 && E >= 1 && k >= 1 && k <= E, XMA_ROCM_EINVAL,
+                "router_gate_topk: T=%lld H=%d E=%d k=%d (1 <= k <= E)", (long long)T, H, E, k);
+    XMA_REQUIRE(E <= RG_MAX_E && k <= RG_MAX_K && H % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0, XMA_ROCM_EUNSUPPORTED,
+                "router_gate_topk: E=%d k=%d H=%d ldx=%lld ldw=%lld (E <= %d, k <= %d, H and ld %% 8 == 0)", E, k, H,
+                (long long)ldx, (long long)ldw, RG_MAX_E, RG_MAX_K);
+    XMA_REQUIRE(ldx >= H && ldw >= H && ldl >= E, XMA_ROCM_EINVAL, "router_gate_topk: leading dimension shorter than a row");
+    if (T == 0) return XMA_ROCM_OK;
+    XMA_REQUIRE(x && gate_weight && logits && weights && ids && ((uintptr_t)x & 15) == 0 && ((uintptr_t)gate_weight & 15) == 0,
+                XMA_ROCM_EINVAL, "router_gate_topk: null or misaligned pointer");
+    XMA_REQUIRE((T + RG_TOKENS - 1) / RG_TOKENS < ((int64_t)1 << 31), XMA_ROCM_EUNSUPPORTED, "router_gate_topk: too many rows");
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == XMA_ROCM_BF16)
+        return router_gate_launch<__bf16, XMA_ROCM_BF16>(x, ldx, gate_weight, ldw, T, H, E, k, logits, ldl, weights, ids,
+                                                         ids_is_i64, st);
+    return router_gate_launch<_Float16, XMA_ROCM_F16>(x, ldx, gate_weight, ldw, T, H, E, k, logits, ldl, weights, ids,
+                                                      ids_is_i64, st);
 }
 
 extern "C" int xma_rocm_router_topk_bwd(const void *logits, int64_t ld, int64_t T, int32_t E, int32_t k, int dtype,

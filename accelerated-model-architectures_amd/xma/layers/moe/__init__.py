@@ -101,15 +101,19 @@ class MoE(nn.Module):
         self, x: torch.Tensor, *, kernel_backend: KernelBackend | None = None
     ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
         # (T, H) -> logits (T, E), weights (T, k) = fp32 softmax over the k selected logits, experts (T, k)
-        router_logits = self.gate(x)
         if kernel_backend is None:
             kernel_backend = Accelerator.get_kernel_backend()
-        if kernel_backend == KernelBackend.rocm and router_logits.is_cuda:
+        if kernel_backend == KernelBackend.rocm and x.is_cuda:
             from . import rocm_implementation as R
 
-            # top-k, softmax and the cast in one kernel; equal logits go to the lower expert index
+            # equal logits go to the lower expert index
+            if self.gate.bias is None and R.router_gate_topk_supported(x, self.gate.weight, self.top_k):
+                # gate GEMM, top-k, softmax, cast and int32 expert ids in one kernel: x is read once
+                return R.router_gate_topk(x, self.gate.weight, self.top_k)
+            router_logits = self.gate(x)
             router_weights, selected_experts = R.router_topk(router_logits, self.top_k)
             return router_logits, router_weights, selected_experts
+        router_logits = self.gate(x)
         router_weights, selected_experts = self._get_topk(router_logits)
         router_weights = F.softmax(router_weights.float(), dim=-1).type_as(x)
         return router_logits, router_weights, selected_experts

@@ -45,10 +45,10 @@ class _RouterTopK(torch.autograd.Function):
     (xma/layers/moe/__init__.py:186-193, 256-262)"""
 
     @staticmethod
-    def forward(ctx, router_logits: torch.Tensor, top_k: int):
+    def forward(ctx, router_logits: torch.Tensor, top_k: int, ids_dtype: torch.dtype):
         T = router_logits.size(0)
         weights = torch.empty(T, top_k, dtype=router_logits.dtype, device=router_logits.device)
-        ids = torch.empty(T, top_k, dtype=torch.int64, device=router_logits.device)
+        ids = torch.empty(T, top_k, dtype=ids_dtype, device=router_logits.device)
         ops.router_topk_rocm(router_logits, weights, ids)
         ctx.save_for_backward(router_logits, ids)
         ctx.mark_non_differentiable(ids)
@@ -59,12 +59,52 @@ class _RouterTopK(torch.autograd.Function):
         router_logits, ids = ctx.saved_tensors
         d_logits = torch.empty_like(router_logits, memory_format=torch.contiguous_format)
         ops.router_topk_bwd_rocm(router_logits, ids, d_weights.contiguous(), d_logits)
-        return d_logits, None
+        return d_logits, None, None
 
 
-def router_topk(router_logits: torch.Tensor, top_k: int):
-    """(router weights (T, k) in the logits' dtype, selected experts int64 (T, k)); differentiable in the logits."""
-    return _RouterTopK.apply(router_logits, top_k)
+class _RouterGateTopK(torch.autograd.Function):
+    """gate projection + top-k + fp32 softmax + cast + int32 expert ids in one kernel; backward: the router's
+    d_logits kernel, then the two skinny GEMMs of the linear layer (d_x = d_logits @ Wg, d_Wg = d_logits^T @ x) on the
+    stock GEMM.  Counterpart of gate(x) and xma/layers/moe/__init__.py:186-193, 256-262."""
+
+    @staticmethod
+    def forward(ctx, x: torch.Tensor, gate_weight: torch.Tensor, top_k: int):
+        T, E = x.size(0), gate_weight.size(0)
+        logits = torch.empty(T, E, dtype=x.dtype, device=x.device)
+        weights = torch.empty(T, top_k, dtype=x.dtype, device=x.device)
+        ids = torch.empty(T, top_k, dtype=torch.int32, device=x.device)
+        ops.router_gate_topk_rocm(x, gate_weight, logits, weights, ids)
+        ctx.save_for_backward(x, gate_weight, logits, ids)
+        ctx.mark_non_differentiable(ids)
+        return logits, weights, ids
+
+    @staticmethod
+    def backward(ctx, d_logits_out, d_weights, _d_ids):
+        x, gate_weight, logits, ids = ctx.saved_tensors
+        d_logits = torch.empty_like(logits)
+        ops.router_topk_bwd_rocm(logits, ids, d_weights.contiguous(), d_logits)
+        if d_logits_out is not None:  # the caller also used the returned router logits (an auxiliary loss)
+            d_logits = d_logits + d_logits_out
+        d_x = d_logits @ gate_weight if ctx.needs_input_grad[0] else None
+        d_w = d_logits.t() @ x if ctx.needs_input_grad[1] else None
+        return d_x, d_w, None
+
+
+def router_gate_topk(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int):
+    """(router logits (T, E), router weights (T, k), selected experts int32 (T, k)) from the activations and the gate's
+    weight (E, H); differentiable in both."""
+    return _RouterGateTopK.apply(x, gate_weight, top_k)
+
+
+def router_gate_topk_supported(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int) -> bool:
+    return x.is_cuda and x.dim() == 2 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and gate_weight.is_contiguous() and \
+        ops.router_gate_topk_supported(x.size(1), gate_weight.size(0), top_k, x.dtype)
+
+
+def router_topk(router_logits: torch.Tensor, top_k: int, ids_dtype: torch.dtype = torch.int64):
+    """(router weights (T, k) in the logits' dtype, selected experts (T, k), int64 as torch.topk gives them or int32 for
+    the routing kernel); differentiable in the logits."""
+    return _RouterTopK.apply(router_logits, top_k, ids_dtype)
 
 
 # ----------------------------------------------------------------------------------------- op mirrors

@@ -54,7 +54,10 @@ SIGNATURES = {
     "xma_rocm_swiglu_forward": (_int, [_p, _i64, _p, _i64, _p, _i64, _i64, _i32, _int, _p]),
     "xma_rocm_swiglu_backward": (_int, [_p, _i64, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _i64, _i32, _int, _p]),
     "xma_rocm_router_topk": (_int, [_p, _i64, _i64, _i32, _i32, _int, _p, _p, _int, _p]),
+    "xma_rocm_router_gate_topk_supported": (_int, [_i32, _i32, _i32, _int]),
+    "xma_rocm_router_gate_topk": (_int, [_p, _i64, _p, _i64, _i64, _i32, _i32, _i32, _int, _p, _i64, _p, _p, _int, _p]),
     "xma_rocm_router_topk_bwd": (_int, [_p, _i64, _i64, _i32, _i32, _int, _p, _int, _p, _p, _i64, _p]),
+    "xma_rocm_diag_mfma_stream": (_int, [_p, _i32, _p, _i32, _p]),
 }
 
 

@@ -122,6 +122,19 @@ def route_rocm(
 
 
 # --------------------------------------------------------------------------- a5 a7 a8 a10
+_S2S_WORKSPACE_BYTES: dict[tuple[int, int, int, int, int], int] = {}
+
+
+def scatter2scatter_workspace_bytes(M: int, N: int, K: int, E: int, device_index: int) -> int:
+    """scratch of one grouped GEMM launch (0 for launches of many rounds of tiles); the library's answer depends on the
+    shape and the device only, so it is asked once per shape"""
+    key = (M, N, K, E, device_index)
+    if key not in _S2S_WORKSPACE_BYTES:
+        with torch.cuda.device(device_index):
+            _S2S_WORKSPACE_BYTES[key] = get_library().xma_rocm_scatter2scatter_workspace_bytes(M, N, K, E)
+    return _S2S_WORKSPACE_BYTES[key]
+
+
 def _scatter2scatter(X, W, idx, offs, out, aux, scale, fan_out, x_grouped, y_grouped, epilogue, M, N, K):
     w_is_kn, w_es, ldw = _weight_layout(W)
     assert W.dtype == X.dtype
@@ -132,7 +145,7 @@ def _scatter2scatter(X, W, idx, offs, out, aux, scale, fan_out, x_grouped, y_gro
     lib = get_library()
     # scratch for the K slices of the tiles of a last, partial round (0 bytes for launches of many rounds); it comes from
     # torch's caching allocator like every other buffer of the op
-    ws_bytes = lib.xma_rocm_scatter2scatter_workspace_bytes(M, N, K, W.size(0))
+    ws_bytes = scatter2scatter_workspace_bytes(M, N, K, W.size(0), X.device.index or 0)
     workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=X.device) if ws_bytes else None
     check(
         lib.xma_rocm_scatter2scatter(
@@ -350,6 +363,37 @@ def router_topk_rocm(logits: torch.Tensor, weights: torch.Tensor, ids: torch.Ten
         lib.xma_rocm_router_topk(_ptr(logits), _rows(logits, "logits"), T, E, k, _code(logits), _ptr(weights), _ptr(ids),
                                  int(ids.dtype == torch.int64), _stream(logits)),
         "xma_rocm_router_topk",
+    )
+
+
+ROUTER_GATE_MAX_E, ROUTER_GATE_MAX_K = 128, 32
+
+
+def router_gate_topk_supported(H: int, E: int, k: int, dtype: torch.dtype) -> bool:
+    """whether the fused gate projection + router kernel covers the shape (otherwise: linear layer + router_topk_rocm).
+    Plain Python, so that a traced caller (torch.compile) can evaluate it; it restates
+    xma_rocm_router_gate_topk_supported, and a test holds the two together."""
+    return (dtype in (torch.bfloat16, torch.float16) and H >= 8 and H % 8 == 0 and 1 <= E <= ROUTER_GATE_MAX_E
+            and 1 <= k <= min(E, ROUTER_GATE_MAX_K))
+
+
+@torch.library.custom_op("xma_rocm::router_gate_topk", mutates_args={"logits", "weights", "ids"})
+def router_gate_topk_rocm(x: torch.Tensor, gate_weight: torch.Tensor, logits: torch.Tensor, weights: torch.Tensor,
+                          ids: torch.Tensor) -> None:
+    """logits = x @ gate_weight^T (rounded to x's dtype), then weights / ids as router_topk_rocm, in one kernel
+    (xma/layers/moe/__init__.py:182-195, 256-262)."""
+    T, H = x.shape
+    E = gate_weight.size(0)
+    k = weights.size(1)
+    assert gate_weight.shape == (E, H) and logits.shape == (T, E) and weights.shape == (T, k) and ids.shape == (T, k)
+    assert x.dtype == gate_weight.dtype == logits.dtype == weights.dtype and ids.dtype in (torch.int32, torch.int64)
+    assert weights.is_contiguous() and ids.is_contiguous()
+    lib = get_library()
+    check(
+        lib.xma_rocm_router_gate_topk(_ptr(x), _rows(x, "x"), _ptr(gate_weight), _rows(gate_weight, "gate_weight"), T, H, E, k,
+                                      _code(x), _ptr(logits), _rows(logits, "logits"), _ptr(weights), _ptr(ids),
+                                      int(ids.dtype == torch.int64), _stream(x)),
+        "xma_rocm_router_gate_topk",
     )
 
 

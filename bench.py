@@ -1,11 +1,12 @@
 """MoE hot-path benchmark on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c5|c2]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c5|c2|copy|mfma_peak]
 
 Default workload: the Mixtral-shaped layer (T=8192, H=4096, I=14336, E=8, top-2, packed SwiGLU, bf16).
-A step is one forward + backward of the expert computation (routing histogram/sort, grouped
-up-projection + SwiGLU, grouped down-projection, combine, and all of their gradients) on synthetic
-inputs that are resident in HBM before the timed region.  Prints ONE JSON line:
+A step is one forward + backward of the layer behind the gate: router (top-k + softmax + expert ids from the
+given router logits), routing histogram/sort, grouped up-projection + SwiGLU, grouped down-projection, combine, and
+all of their gradients down to the logits, on synthetic inputs (drawn on the CPU with torch.manual_seed(0), then
+copied) that are resident in HBM before the timed region.  Prints ONE JSON line:
 
   value        tokens/s over the K timed steps (c2: routed ids/s)
   roofline     the dominant kernel against its roofline; `achieved` = algorithmic FLOPs (or bytes)
@@ -43,11 +44,12 @@ WORKLOADS = {
 
 # HBM bytes per launch of each workload's dominant kernel, from two counter runs (FETCH_SIZE scaled by 2.0, WRITE_SIZE by
 # 1.0: the factors a 1 GiB device copy, `--workload copy`, gives for the same counters).  bench.py cannot read hardware
-# counters itself; the figures are re-measured with rocprofv3 whenever the kernel changes.
+# counters itself: the figures are copied from the profile named beside them and are NOT measured in this run.
 MEASURED_TRAFFIC_BYTES = {
     "c3": 9.31e9,  # up-projection + SwiGLU GEMM: 7.89 GB fetched + 1.42 GB written (3.42 GB algorithmic)
-    "c2": 70.9e6,  # route_scatter_kernel: 17.1 MB fetched + 53.8 MB written
+    "c2": 92.2e6,  # route: unit histogram 17.1 MB + scan 4.2 MB + scatter 70.9 MB (17.1 MB fetched + 53.8 MB written)
 }
+TRAFFIC_SOURCE = "profiles/hbm_traffic_c3_c2_pmc.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE; a constant, not measured in this run)"
 
 
 def _time_gpu(fn, iters: int, warmup: int = 2) -> float:
@@ -65,27 +67,32 @@ def _time_gpu(fn, iters: int, warmup: int = 2) -> float:
 
 
 def _make_moe_inputs(cfg, device, seed=0):
+    """module and inputs of a workload, drawn on the CPU from one seeded generator (so the CPU baseline and the device see
+    the same bits) and copied to the device; weights expert by expert to bound the host memory"""
     from xma.functional import swiglu_packed
     from xma.layers import MoE
 
-    g = torch.Generator(device=device).manual_seed(seed)
+    g = torch.Generator().manual_seed(seed)
     T, H, I, E, k = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["k"]
     with torch.device("meta"):
         moe = MoE(E, k, H, I, swiglu_packed, True, add_bias=False, std=0.02)
     moe = moe.to_empty(device=device).to(torch.bfloat16)
     with torch.no_grad():
-        for p in (moe.c_fc.weight, moe.c_proj.weight, moe.gate.weight):
-            p.copy_((torch.randn(p.shape, generator=g, device=device, dtype=torch.float32) * 0.02).to(p.dtype))
+        for p in (moe.c_fc.weight, moe.c_proj.weight):
+            for e in range(E):
+                p[e].copy_((torch.randn(p.shape[1:], generator=g) * 0.02).to(p.dtype))
+        moe.gate.weight.copy_((torch.randn(moe.gate.weight.shape, generator=g) * 0.02).to(torch.bfloat16))
         moe.c_fc.N_array.fill_(2 * I), moe.c_fc.K_array.fill_(H)
         moe.c_proj.N_array.fill_(H), moe.c_proj.K_array.fill_(I)
-    x = torch.randn(T, H, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
-    logits = torch.randn(T, E, generator=g, device=device, dtype=torch.float32)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16).to(device)
+    logits = torch.randn(T, E, generator=g)
     if cfg["bias"]:
-        logits = logits + cfg["bias"] * torch.randn(E, generator=g, device=device, dtype=torch.float32)
+        logits = logits + cfg["bias"] * torch.randn(E, generator=g)
+    logits = logits.to(device)
     vals, sel = logits.topk(k, dim=-1)
     rw = torch.softmax(vals.float(), dim=-1).to(torch.bfloat16)
-    grad = torch.randn(T, H, generator=g, device=device, dtype=torch.float32).to(torch.bfloat16)
-    return moe, x, rw, sel, grad
+    grad = torch.randn(T, H, generator=g).to(torch.bfloat16).to(device)
+    return moe, x, logits, rw, sel, grad
 
 
 def _kernel_table(moe, x, rw, sel, grad, cfg, iters):
@@ -159,7 +166,8 @@ def _kernel_table(moe, x, rw, sel, grad, cfg, iters):
                             f"({nset * comb_bytes >> 20} MiB, more than the Infinity Cache): cold figures"}
     del eos, ys, grads, gdys
     mem("route", lambda: R.route(sel, E), Tk * 8 + Tk * 8 + Tk * 8 + E * 20)
-    # the router behind the gate GEMM (outside the timed step, which starts from the router's outputs)
+    # the router: top-k + softmax + ids from given logits (part of the timed step), and fused with the gate projection
+    # (what MoE.forward runs), beside the reference's chain of stock ops
     lg = torch.randn(T, E, device=dev, dtype=torch.float32).to(x.dtype)
     r_w = torch.empty(T, k, device=dev, dtype=x.dtype)
     r_ids = torch.empty(T, k, device=dev, dtype=torch.int64)
@@ -168,6 +176,14 @@ def _kernel_table(moe, x, rw, sel, grad, cfg, iters):
     mem("router_topk_bwd", lambda: ops.router_topk_bwd_rocm(lg, r_ids, r_w, d_lg), 2 * T * E * esz + T * k * (esz + 8))
     mem("router_torch(topk+softmax+cast)", lambda: torch.softmax(lg.topk(k, dim=-1).values.float(), -1).to(x.dtype),
         T * E * esz + T * k * (esz + 8))
+    wg = moe.gate.weight.detach()
+    if ops.router_gate_topk_supported(H, E, k, x.dtype):
+        r_ids32 = torch.empty(T, k, device=dev, dtype=torch.int32)
+        r_lg = torch.empty(T, E, device=dev, dtype=x.dtype)
+        gate_bytes = T * H * esz + E * H * esz + T * E * esz + T * k * (esz + 4)
+        mem("gate+router_fused(gemm+top-k+softmax+ids)", lambda: ops.router_gate_topk_rocm(x, wg, r_lg, r_w, r_ids32), gate_bytes)
+        mem("gate+router_torch(linear+topk+softmax+cast)",
+            lambda: torch.softmax(torch.nn.functional.linear(x, wg).topk(k, dim=-1).values.float(), -1).to(x.dtype), gate_bytes)
     return table, notes
 
 
@@ -175,18 +191,21 @@ def run_moe(args, cfg, name):
     from oracle import moe as oracle_moe
     from xma import KernelBackend
 
+    from xma.layers.moe import rocm_implementation as R
+
     dev = torch.device("cuda:0")
-    moe, x, rw, sel, grad = _make_moe_inputs(cfg, dev)
+    moe, x, logits, rw, sel, grad = _make_moe_inputs(cfg, dev)
     T, H, I, E, k = cfg["T"], cfg["H"], cfg["I"], cfg["E"], cfg["k"]
     xg = x.clone().requires_grad_()
-    rwg = rw.clone().requires_grad_()
+    lg = logits.to(torch.bfloat16).requires_grad_()  # the router works in the activations' dtype, as behind the gate
 
     def step():
         for p in moe.parameters():
             p.grad = None
         xg.grad = None
-        rwg.grad = None
-        y = moe._compute_experts(xg, rwg, sel, kernel_backend=KernelBackend.rocm)
+        lg.grad = None
+        w, ids = R.router_topk(lg, k, ids_dtype=torch.int32)
+        y = moe._compute_experts(xg, w, ids, kernel_backend=KernelBackend.rocm)
         y.backward(grad)
 
     for _ in range(args.warmup):
@@ -197,6 +216,24 @@ def run_moe(args, cfg, name):
         step()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+
+    # the whole layer as MoE.forward runs it (gate projection fused with the router), for the record
+    def layer_step():
+        for p in moe.parameters():
+            p.grad = None
+        xg.grad = None
+        y, _ = moe(xg, kernel_backend=KernelBackend.rocm)
+        y.backward(grad)
+
+    for _ in range(2):
+        layer_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(max(args.steps // 2, 1)):
+        layer_step()
+    torch.cuda.synchronize()
+    layer_ms = (time.perf_counter() - t0) * 1e3 / max(args.steps // 2, 1)
+    rw, sel = R.router_topk(lg.detach(), k)  # the routing the timed steps used (bf16 logits)
     counts = torch.bincount(sel.flatten(), minlength=E)
 
     table, notes = _kernel_table(moe, x, rw, sel, grad, cfg, args.kernel_iters)
@@ -214,9 +251,7 @@ def run_moe(args, cfg, name):
         "unit": "TFLOP/s",
         "frac": round(gemms[dom]["tflops"] / PEAK_BF16_TFLOPS, 4),
         "traffic": MEASURED_TRAFFIC_BYTES.get(name) if dom.startswith("up_swiglu") else None,
-        # measured on this hardware: independent bf16 MFMAs alone, random operands, no memory traffic (power-limited clock);
-        # with all-zero operands the same stream reaches 2475
-        "mfma_only_random_operands_tflops": 1700.0,
+        "traffic_source": TRAFFIC_SOURCE if name in MEASURED_TRAFFIC_BYTES else None,
         "all_gemms_tflops": round(total_flops / total_ms / 1e9, 1),
         "all_gemms_frac": round(total_flops / total_ms / 1e9 / PEAK_BF16_TFLOPS, 4),
     }
@@ -262,6 +297,8 @@ def run_moe(args, cfg, name):
             "tokens": T,
             "rows_per_expert_min_mean_max": [int(counts.min()), float(counts.float().mean()), int(counts.max())],
             "step_tflops": round(18.0 * T * k * H * I / ms_per_step / 1e9, 1),
+            "step": "router top-k/softmax/ids from the given logits + routing + experts fwd+bwd down to d_logits",
+            "whole_layer_ms": round(layer_ms, 4),  # MoE.forward + backward with the gate projection fused into the router
         },
         "roofline": roofline,
         "cpu_baseline": cpu,
@@ -360,7 +397,8 @@ def run_routing(args):
             "peak": PEAK_HBM_GBS,
             "unit": "GB/s",
             "frac": round(route_bytes / route_graph_ms / 1e6 / PEAK_HBM_GBS, 4),
-            "traffic": None if args.zipf else MEASURED_TRAFFIC_BYTES["c2"] + 17.1e6 + 4.2e6,  # scatter + unit hist + scan
+            "traffic": None if args.zipf else MEASURED_TRAFFIC_BYTES["c2"],
+            "traffic_source": None if args.zipf else TRAFFIC_SOURCE,
         },
         "cpu_baseline": {"value": round(n / dt, 1), "unit": "ids/s", "cores": 1, "kind": "port",
                          "sample": f"numpy stable argsort + bincount + cumsum of the same {n} ids, mean of {reps}"},
@@ -391,12 +429,41 @@ def run_copy(args):
                       "config": {"workload": f"copy: torch copy_ of {nbytes} bytes (reads {nbytes}, writes {nbytes} per launch)"}}))
 
 
+def run_mfma_peak(args):
+    """What the matrix pipes sustain with nothing else going on: independent bf16 MFMAs from registers on every compute
+    unit, once with random operands and once with all-zero operands (which toggle nothing and run at the full clock).
+    The GEMM kernels' fractions of the 2.5 PFLOP/s figure are read beside the first number."""
+    from xma.rocm import get_library
+    from xma.rocm.loader import check
+
+    lib = get_library()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    g = torch.Generator().manual_seed(0)
+    rnd = (torch.rand(16 * 256 * 8, generator=g) * 4 - 2).to(torch.bfloat16).cuda()  # 8 bf16 per lane and fragment
+    out = torch.empty(cus * 256, dtype=torch.float32, device="cuda")
+    iters = 20000
+    flops = 2.0 * 32 * 32 * 16 * 64 * 4 * cus * iters
+    res = {}
+    for label, ops_ in (("random_operands", rnd), ("zero_operands", torch.zeros_like(rnd))):
+        def call():
+            check(lib.xma_rocm_diag_mfma_stream(ops_.data_ptr(), iters, out.data_ptr(), cus,
+                                                torch.cuda.current_stream().cuda_stream), "xma_rocm_diag_mfma_stream")
+        ms = _time_gpu(call, max(args.steps, 3), warmup=max(args.warmup, 1))
+        res[label] = {"ms": round(ms, 3), "tflops": round(flops / ms / 1e9, 1), "frac_of_2500": round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+    print(json.dumps({"metric": "mfma_only_bf16_tflops", "value": res["random_operands"]["tflops"], "unit": "TFLOP/s", "n_gpus": 1,
+                      "steps": args.steps, "warmup": args.warmup, "ms_per_step": res["random_operands"]["ms"],
+                      "higher_is_better": True, "dtype": "bf16",
+                      "config": {"workload": f"mfma_peak: {iters} x 64 independent v_mfma_f32_32x32x16_bf16 per wave, 4 waves on "
+                                             f"each of {cus} compute units, operands in registers, no memory traffic"},
+                      "results": res}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "copy"])
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "copy", "mfma_peak"])
     ap.add_argument("--zipf", action="store_true", help="c2 only: Zipf(s=1.1) ids instead of uniform")
     ap.add_argument("--kernel-iters", type=int, default=5)
     ap.add_argument("--cpu-fraction", type=int, default=1, help="CPU baseline runs on T / this many tokens")
@@ -411,6 +478,8 @@ def main():
     get_library()
     if args.workload == "copy":
         run_copy(args)
+    elif args.workload == "mfma_peak":
+        run_mfma_peak(args)
     elif args.workload == "c2":
         run_routing(args)
     else:

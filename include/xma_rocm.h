@@ -209,6 +209,19 @@ XMA_API int xma_rocm_swiglu_backward(const void *gate, int64_t ld_gate, const vo
 XMA_API int xma_rocm_router_topk(const void *logits, int64_t ld, int64_t T, int32_t E, int32_t k, int dtype, void *weights,
                          void *ids, int ids_is_i64, void *stream);
 /*
+ * Gate projection and router in one kernel: logits (T, E) = x (T, H) @ gate_weight (E, H)^T with fp32 accumulation,
+ * rounded to `dtype` (what the stock linear layer returns), then everything xma_rocm_router_topk does, on those rounded
+ * logits: weights (T, k), ids (T, k) (int32 for xma_rocm_route, or int64).  x is read from HBM once; the (T, E) logits
+ * are written for the module's return value and the backward, never read back.
+ * Replaces gate(x) + _get_topk + softmax + type_as, xma/layers/moe/__init__.py:182-195 and :256-262.
+ * bf16 / fp16, H % 8 == 0, E <= 128, k <= min(E, 32): xma_rocm_router_gate_topk_supported says whether a shape is
+ * covered (otherwise: a linear layer followed by xma_rocm_router_topk).
+ */
+XMA_API int xma_rocm_router_gate_topk_supported(int32_t H, int32_t E, int32_t k, int dtype);
+XMA_API int xma_rocm_router_gate_topk(const void *x, int64_t ldx, const void *gate_weight, int64_t ldw, int64_t T, int32_t H,
+                              int32_t E, int32_t k, int dtype, void *logits, int64_t ldl, void *weights, void *ids,
+                              int ids_is_i64, void *stream);
+/*
  * Backward of xma_rocm_router_topk: with w = softmax of the selected logits (fp32, recomputed),
  *     d_logits[t, ids[t, j]] = w_j * (d_weights[t, j] - sum_i w_i * d_weights[t, i]),  0 elsewhere.
  * Writes all T x E elements of d_logits (row stride ldd), so the caller need not clear it.  Replaces the autograd
@@ -216,6 +229,15 @@ XMA_API int xma_rocm_router_topk(const void *logits, int64_t ld, int64_t T, int3
  */
 XMA_API int xma_rocm_router_topk_bwd(const void *logits, int64_t ld, int64_t T, int32_t E, int32_t k, int dtype, const void *ids,
                              int ids_is_i64, const void *d_weights, void *d_logits, int64_t ldd, void *stream);
+
+/*
+ * Measurement aid with no counterpart in the reference: `workgroups` workgroups of 4 waves each issue iters x 64
+ * independent v_mfma_f32_32x32x16_bf16 on operands read once from `operands` (16 x 256 x 16 bytes: 8 A and 8 B fragments
+ * per lane), nothing else in the loop.  2 * 32 * 32 * 16 * 64 * 4 * workgroups * iters FLOP per call; out receives
+ * workgroups x 256 floats.  bench.py --workload mfma_peak times it with random and with all-zero operands: the rate the
+ * matrix pipes sustain under the power limit, beside which the GEMM kernels' figures are read.
+ */
+XMA_API int xma_rocm_diag_mfma_stream(const void *operands, int32_t iters, float *out, int32_t workgroups, void *stream);
 
 #ifdef __cplusplus
 }

@@ -141,3 +141,71 @@ def test_router_in_the_layer_forward_and_gate_gradient():
     want.backward(grad.float().cpu())
     assert nerr(y, want.detach()) <= 1e-2
     assert nerr(moe.gate.weight.grad, wg.grad) <= 2e-2  # bf16 router weights and a bf16 gate GEMM in the chain
+
+
+GATE_CASES = [  # T, H, E, k
+    (7, 64, 8, 2),
+    (1000, 4096, 8, 2),
+    (513, 2048, 64, 6),
+    (300, 2048, 128, 8),
+    (33, 72, 1, 1),
+    (257, 136, 3, 2),
+    (100, 200, 100, 32),
+    (65, 8, 33, 5),
+    (8192, 4096, 8, 2),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("T,H,E,k", GATE_CASES)
+def test_router_gate_topk_fused(dtype, T, H, E, k):
+    """Gate projection fused with the router (xma/layers/moe/__init__.py:182-195, 256-262).  Logits against the fp32
+    product (one rounding to the 16-bit dtype plus the summation order); expert ids bit-exact and router weights within a
+    unit in the last place against the oracle's top-k and softmax applied to the logits the device produced; int32 ids;
+    d_x and d_Wg against the fp32 chain's gradient (2e-2: 16-bit router weights and 16-bit d_logits in the chain)."""
+    from tests.utils import nerr
+    from xma.layers.moe import rocm_implementation as R
+
+    print(f"router gate {dtype} T={T} H={H} E={E} k={k}", flush=True)
+    g = torch.Generator().manual_seed(T + H + E + k)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    wg = (torch.randn(E, H, generator=g) * (H**-0.5)).to(dtype)
+    dw = torch.randn(T, k, generator=g).to(dtype)
+    xd, wd = x.cuda().requires_grad_(), wg.cuda().requires_grad_()
+    assert R.router_gate_topk_supported(xd, wd, k)
+    logits, w, ids = R.router_gate_topk(xd, wd, k)
+    assert ids.dtype == torch.int32 and not ids.requires_grad and logits.shape == (T, E) and logits.dtype == dtype
+    dev_logits = logits.detach().cpu()
+    xf, wf = x.float().requires_grad_(), wg.float().requires_grad_()
+    lg = xf @ wf.t()
+    ulp = ULP[dtype] * 2  # values up to 2^k have ulps of 2^(k - mantissa bits)
+    assert (lg.detach() - dev_logits.float()).abs().max().item() <= ulp * max(1.0, lg.detach().abs().max().item())
+    want_w, want_ids = oracle.routing_topk(dev_logits, k, dtype)
+    assert torch.equal(ids.cpu().long(), want_ids)
+    assert (w.detach().cpu().float() - want_w.float()).abs().max().item() <= ULP[dtype]
+    # gradients: the device's logit values, the fp32 chain's derivative
+    lg = lg + (dev_logits.float() - lg).detach()
+    rw = torch.softmax(lg.gather(-1, want_ids), -1)
+    rw.backward(dw.float())
+    w.backward(dw.cuda())
+    assert nerr(xd.grad, xf.grad) <= 2e-2 and nerr(wd.grad, wf.grad) <= 2e-2
+
+
+def test_router_gate_topk_strided_rows_and_fallback():
+    """x as a column slice of a wider tensor (row pitch > H); shapes the fused kernel does not cover are reported as such
+    and the layer falls back to the linear layer + router_topk"""
+    from xma.layers.moe import rocm_implementation as R
+    from xma.rocm import ops
+
+    g = torch.Generator().manual_seed(2)
+    wide = torch.randn(300, 512 + 64, generator=g).to(torch.bfloat16).cuda()
+    x = wide[:, 64:]
+    wg = (torch.randn(16, 512, generator=g) * 0.05).to(torch.bfloat16).cuda()
+    assert R.router_gate_topk_supported(x, wg, 4)
+    logits, w, ids = R.router_gate_topk(x, wg, 4)
+    l2, w2, ids2 = R.router_gate_topk(x.contiguous(), wg, 4)
+    assert torch.equal(logits, l2) and torch.equal(w, w2) and torch.equal(ids, ids2)
+    assert not ops.router_gate_topk_supported(512, 129, 2, torch.bfloat16)
+    assert not ops.router_gate_topk_supported(512, 64, 33, torch.bfloat16)
+    assert not ops.router_gate_topk_supported(516, 64, 2, torch.bfloat16)
+    assert not ops.router_gate_topk_supported(512, 64, 2, torch.float32)

@@ -71,6 +71,22 @@ def test_argument_errors_are_reported_before_any_launch():
     assert lib.xma_rocm_continuous_count(None, 0, 0, ctypes.c_void_p(16), 4, None, 0, None) == 0
 
 
+def test_fused_router_shape_rule_matches_the_library():
+    """the Python restatement of the fused gate + router kernel's coverage (evaluated under torch.compile, where a ctypes
+    call cannot be traced) against the library's own answer"""
+    from xma.rocm import get_library
+    from xma.rocm.ops import router_gate_topk_supported
+
+    lib = get_library()
+    codes = {torch.bfloat16: 0, torch.float16: 1, torch.float32: 2}
+    for dtype, code in codes.items():
+        for H in (0, 4, 8, 12, 64, 4096):
+            for E in (0, 1, 8, 32, 33, 128, 129, 2048):
+                for k in (0, 1, 2, 8, 32, 33, 128):
+                    assert router_gate_topk_supported(H, E, k, dtype) == bool(
+                        lib.xma_rocm_router_gate_topk_supported(H, E, k, code)), (dtype, H, E, k)
+
+
 def test_backend_selection_and_errors():
     from xma import Accelerator, KernelBackend
     from xma.functional import continuous_count, swiglu_packed
