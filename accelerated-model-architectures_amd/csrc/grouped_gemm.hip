@@ -382,10 +382,18 @@ __device__ __forceinline__ bool locate_tile(const FwdArgs &a, unsigned char *sme
     return true;
 }
 
-// ---- epilogue of one 256 x 256 tile (LDS is free: no wave reads operand tiles any more)
+// Scattered index and row scale of a lane's row in each of the four 32-row blocks of its wave (row wq + 32 i + lane % 32
+// of the tile, clamped to the last valid row), when the caller has fetched them ahead of the epilogue.
+struct EpiRows {
+    int idx[4];
+    float sc[4];
+};
+
+// ---- epilogue of one 256 x 256 tile; smem: staging area that no wave reads operand tiles from any more
 template <typename T, int EPI>
 __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4][4], unsigned char *smem, int64_t row0,
-                                              int rows_valid, int n0, int tid, int only_i = -1) {
+                                              int rows_valid, int n0, int tid, int only_i = -1,
+                                              const EpiRows *pre = nullptr) {
     // only_i >= 0: just the 32-row block only_i of every wave (the fix-up kernel spreads a tile over four workgroups)
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -415,9 +423,12 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
             int r = wq + i * 32 + lrow;
             if (r >= rows_valid) r = rows_valid - 1; // duplicates are computed and never stored
             const int64_t n = row0 + r;
-            dst_i[i] = need_idx ? (int)a.idx[n] : (int)n;
+            dst_i[i] = need_idx ? (pre ? pre->idx[i] : (int)a.idx[n]) : (int)n;
         }
-        if (a.scale) {
+        if (a.scale && pre) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) sc_i[i] = pre->sc[i];
+        } else if (a.scale) {
             uint16_t raw[4];
 #pragma unroll
             for (int i = 0; i < 4; ++i) raw[i] = a.scale[dst_i[i]];
@@ -507,7 +518,7 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
             int r = wq + i * 32 + lrow;
             if (r >= rows_valid) r = rows_valid - 1;
             sc_i[i] = 1.f;
-            if (a.scale) sc_i[i] = Elem<T>::lo((uint32_t)a.scale[a.idx[row0 + r]]);
+            if (a.scale) sc_i[i] = pre ? pre->sc[i] : Elem<T>::lo((uint32_t)a.scale[a.idx[row0 + r]]);
         }
         u32x4 zin[16];
         auto load_block = [&](int i) {
@@ -777,6 +788,380 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_fixup_kernel(con
 }
 
 // ------------------------------------------------------------------------------------------------
+// Persistent forward / dX kernel: one workgroup per compute unit walks the tiles b, b + gridDim.x, ... of the launch and
+// overlaps the set-up of a tile with the epilogue of the tile before it.
+//
+// Between two main loops a workgroup has to find its next tile, fetch the scattered row indices, and wait for the first
+// K step to arrive from HBM: three dependent round trips with idle matrix pipes, as long as the epilogue itself.  Here
+// everything a tile needs is fetched one tile ahead: while tile i is in its main loop the schedule entry, the gathered
+// row indices and the epilogue's indices of tile i + 1 are loaded into registers, and the 16 LDS-DMA pieces of the first
+// K step of tile i + 1 go out right behind the last barrier of tile i's main loop, before its epilogue starts.  They land
+// in stage 0 while the epilogue stages its rows in the LDS above it (stage 1 and the 32 KB that the two stages leave
+// free), so the next main loop starts as soon as the epilogue's stores have been handed over.
+//
+// The LDS-DMA loads are issued from inline assembly here (M0 is written next to the load): the compiler guards every
+// LDS access it cannot prove disjoint from an LDS-DMA load it knows of with s_waitcnt vmcnt(0), which would make the
+// epilogue wait for the loads it is supposed to hide.  What the compiler does not know it cannot wait for too little
+// either: vmcnt retires in order, so a wait sized for the compiler's own loads only ever covers more than it has to; the
+// waits that protect the operand tiles are all explicit.
+//
+// The expert-major schedule (tiles before each expert, row offsets) is computed once per workgroup into LDS instead of
+// once per tile.  E <= PST_MAX_E; launches with more experts use grouped_gemm_kernel.
+// ------------------------------------------------------------------------------------------------
+constexpr int PST_MAX_E = 1023;
+constexpr int PST_SMEM_BYTES = 160 * 1024 - 64;
+constexpr int PST_STAGING_OFF = STAGE_CHUNKS * 16; // the epilogue's staging area starts above stage 0
+// Rows fetched one tile ahead wait in LDS, one dword per lane and item (1 KB per item), so that no register is held
+// across the main loop: 8 gathered rows of the next tile, 2 x 4 rows of the epilogue (next tile's arrive while this
+// tile's are still needed), 4 row scales of this tile.
+constexpr int PST_ROWS_OFF = PST_STAGING_OFF + 4 * EPI_BWD_WAVE_BYTES;
+constexpr int PST_QR = 0, PST_ER = 8, PST_SC = 16, PST_ROW_ITEMS = 20;
+constexpr int PST_TABLE_OFF = PST_SMEM_BYTES - 2 * (PST_MAX_E + 1) * (int)sizeof(int);
+static_assert(EPI_BWD_WAVE_BYTES >= EPI_WAVE_BYTES && PST_ROWS_OFF + PST_ROW_ITEMS * 1024 <= PST_TABLE_OFF,
+              "epilogue staging and the prefetched rows must fit between stage 0 and the schedule tables");
+
+__device__ __forceinline__ void lds_dma16_raw(const void *src, uint32_t lds_wave_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(lds_wave_base), "v"(src)
+                 : "memory", "m0");
+}
+// one dword per lane: lane l's value lands at lds_wave_base + 4 l
+__device__ __forceinline__ void lds_dma4_raw(const void *src, uint32_t lds_wave_base) {
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, off" ::"s"(lds_wave_base), "v"(src)
+                 : "memory", "m0");
+}
+
+// Optional phase stamps of the persistent kernel (builds with -DXMA_PST_TIMING only): workgroup b writes the 100 MHz
+// real-time counter at six points of each of its first PST_TIMING_TILES tiles; xma_rocm_debug_pst_times copies them out.
+#ifdef XMA_PST_TIMING
+constexpr int PST_TIMING_TILES = 48;
+__device__ uint64_t g_pst_times[256][PST_TIMING_TILES][8];
+#define PST_STAMP(k)                                                                                   \
+    do {                                                                                               \
+        if (threadIdx.x == 0 && blockIdx.x < 256 && tile_no < PST_TIMING_TILES)                        \
+            g_pst_times[blockIdx.x][tile_no][k] = __builtin_amdgcn_s_memrealtime();                    \
+    } while (0)
+#else
+#define PST_STAMP(k) \
+    do {             \
+    } while (0)
+#endif
+
+struct PstTile {
+    int valid, t, e, n0, rows_valid, row0; // t: position in the workgroup's walk (linear tile id before the XCD remap)
+};
+
+template <typename T, int WT, int EPI>
+__global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kernel(const FwdArgs a) {
+    extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+    int *s_pre = (int *)(smem + PST_TABLE_OFF); // [E + 1] tiles of the experts before e
+    int *s_hi = s_pre + (PST_MAX_E + 1);        // [E] inclusive row offsets
+    const int NT = (a.N + BN - 1) / BN;
+    const int KT = (a.K + BK - 1) / BK;
+    const int KT_full = a.K / BK;                // end of the steps without a chunk past K
+    const bool k_tail = (a.K & (BK - 1)) != 0;
+    const uint16_t *zero = (const uint16_t *)g_zero_page;
+    const uint32_t lds0 = lds_addr_of(smem);
+
+    // ---- schedule tables, once per workgroup
+    {
+        const int tid0 = threadIdx.x, lane0 = tid0 & 63;
+        if (tid0 < WAVE) {
+            int carry = 0;
+            for (int b = 0; b < a.E; b += WAVE) {
+                const int x = b + lane0;
+                int v = 0;
+                if (x < a.E) {
+                    const int64_t hi = a.offs[x];
+                    const int64_t cnt = hi - (x ? a.offs[x - 1] : 0);
+                    v = (int)((cnt + BM - 1) / BM) * NT;
+                    s_hi[x] = (int)hi;
+                }
+                int s = v;
+#pragma unroll
+                for (int d = 1; d < WAVE; d <<= 1) {
+                    const int t = __shfl_up(s, d);
+                    if (lane0 >= d) s += t;
+                }
+                if (x < a.E) s_pre[x] = carry + s - v;
+                carry += __shfl(s, WAVE - 1);
+            }
+            if (lane0 == 0) s_pre[a.E] = carry;
+        }
+        __syncthreads();
+    }
+    int full = __builtin_amdgcn_readfirstlane(s_pre[a.E]); // tiles this launch computes whole
+    if (a.partial) { // the tiles of a last, partial round are left to the K-slice and fix-up launches (see locate_tile)
+        const int total = full;
+        full = total / a.split_cus * a.split_cus;
+        const int rest = total - full;
+        int parts = rest ? a.split_cus / rest : 1;
+        if (parts > KT / SPLIT_MIN_STEPS) parts = KT / SPLIT_MIN_STEPS;
+        if (parts < 2) full = total;
+    }
+
+    // first tile at or behind position t of this workgroup's walk (every wave computes the same, from LDS only)
+    auto lookup = [&](int t, int lane) -> PstTile {
+        PstTile r;
+        r.valid = 0;
+        for (; t < a.grid_main; t += gridDim.x) {
+            const int L = xcd_remap(t, a.grid_main);
+            if (L >= full) continue;
+            int e;
+            if (a.E <= WAVE) {
+                const int x = lane < a.E ? lane : a.E;
+                const int lo = s_pre[x], hi = s_pre[x < a.E ? x + 1 : a.E];
+                e = __builtin_ctzll(__ballot(lo <= L && L < hi));
+            } else { // two levels of 64-way search
+                const int seg = (a.E + WAVE - 1) / WAVE;
+                const int x1 = lane * seg < a.E ? lane * seg : a.E;
+                const int b0 = (63 - __builtin_clzll(__ballot(s_pre[x1] <= L))) * seg;
+                const int x = b0 + lane < a.E ? b0 + lane : a.E;
+                const int lo = s_pre[x], hi = s_pre[x < a.E ? x + 1 : a.E];
+                e = b0 + __builtin_ctzll(__ballot(lane < seg && lo <= L && L < hi));
+            }
+            e = __builtin_amdgcn_readfirstlane(e);
+            const int local = L - __builtin_amdgcn_readfirstlane(s_pre[e]);
+            const int row_hi = __builtin_amdgcn_readfirstlane(s_hi[e]);
+            const int row_lo = e ? __builtin_amdgcn_readfirstlane(s_hi[e - 1]) : 0;
+            const int tiles_m = (row_hi - row_lo + BM - 1) / BM;
+            const int m_tile = local % tiles_m, n_tile = local / tiles_m;
+            r.valid = 1;
+            r.t = t;
+            r.e = e;
+            r.row0 = row_lo + m_tile * BM;
+            r.rows_valid = (row_hi - r.row0 < BM) ? row_hi - r.row0 : BM;
+            r.n0 = n_tile * BN;
+            break;
+        }
+        return r;
+    };
+    // Rows of a lane: the 8 rows of its LDS-DMA pieces (q) and the 4 rows of its epilogue (e), clamped to the tile's last
+    // valid row (duplicates are computed and never stored).  Where a row's scattered index is needed, its low dword is
+    // fetched by a 4-byte LDS-DMA load into the lane's slot of an item of the row area and read back behind the main loop.
+    const uint32_t *idx32 = (const uint32_t *)a.idx;
+    const bool need_q_idx = !a.x_grouped, need_e_idx = !a.y_grouped || a.scale != nullptr;
+    auto q_row = [&](const PstTile &t, int i, int lane, int wave) {
+        const int r = wave * 64 + i * 8 + (lane >> 3);
+        return t.row0 + (r < t.rows_valid ? r : t.rows_valid - 1);
+    };
+    auto e_row = [&](const PstTile &t, int i, int lane, int wave) {
+        const int r = (wave & 1) * 128 + i * 32 + (lane & 31);
+        return t.row0 + (r < t.rows_valid ? r : t.rows_valid - 1);
+    };
+    auto row_item_lds = [&](int item, int wave) { return lds0 + (uint32_t)(PST_ROWS_OFF + item * 1024 + wave * 256); };
+    auto row_item = [&](int item, int tid) { return ((const uint32_t *)(smem + PST_ROWS_OFF + item * 1024))[tid]; };
+    auto prefetch_rows = [&](const PstTile &t, int lane, int wave, bool q, int e_buf) {
+        if (q && need_q_idx) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) lds_dma4_raw(idx32 + 2 * (int64_t)q_row(t, i, lane, wave), row_item_lds(PST_QR + i, wave));
+        }
+        if (need_e_idx) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                lds_dma4_raw(idx32 + 2 * (int64_t)e_row(t, i, lane, wave), row_item_lds(PST_ER + 4 * e_buf + i, wave));
+        }
+    };
+
+    // Addresses of the 16 LDS-DMA pieces of a tile: a uniform base per operand (SGPRs: the tile's corner of the weight
+    // matrix; the activations' first row for a gathered operand, the tile's first row for a grouped one) and one 32-bit
+    // byte offset per piece and lane.  A K step adds a uniform amount to the bases, so a piece in the loop is the M0
+    // update and the load, without any vector address arithmetic.  The host has checked that the offsets fit 32 bits.
+    uint32_t q_off[8], p_off[8];
+    const char *q_base = nullptr, *p_base = nullptr;
+    const int64_t p_step_b = (WT == 0) ? 2 * BK : (int64_t)2 * BK * a.ldw; // bytes per K step along the weights
+    auto make_pointers = [&](const PstTile &t, int lane, int wave, const uint32_t (&raw)[8]) {
+        const uint16_t *We = a.W + (int64_t)t.e * a.w_es;
+        if (WT == 0) {
+            p_base = (const char *)(We + (int64_t)t.n0 * a.ldw);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                int r = wave * 64 + i * 8 + (lane >> 3);
+                if (t.n0 + r >= a.N) r = a.N - 1 - t.n0;
+                p_off[i] = (uint32_t)r * (uint32_t)(2 * a.ldw) + rowmajor_lane_chunk(i, lane) * 16;
+            }
+        } else {
+            p_base = (const char *)(We + t.n0);
+            const int max_chunk = ((a.N - t.n0) >> 3) - 1;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                int cj = transposed_lane_chunk(j, lane);
+                if (cj > max_chunk) cj = max_chunk;
+                p_off[j] = (uint32_t)(wave * 16 + 2 * j + (lane >> 5)) * (uint32_t)(2 * a.ldw) + cj * 16;
+            }
+        }
+        q_base = (const char *)(need_q_idx ? a.X : a.X + (int64_t)t.row0 * a.ldx);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t src = need_q_idx ? fastdiv(raw[i], a.fan_div) : raw[i] - (uint32_t)t.row0;
+            q_off[i] = src * (uint32_t)(2 * a.ldx) + rowmajor_lane_chunk(i, lane) * 16;
+        }
+    };
+    // piece 0..15 of K step kt of the tile the bases and offsets describe -> stage kt & 1; FULL: the step exists and has
+    // no chunk past K
+    int wave_u = 0; // this wave's index, set per tile (uniform)
+    int lane_v = 0;
+    auto issue_piece = [&](int kt, auto PIECE, auto FULL) {
+        constexpr int piece = PIECE.value;
+        if constexpr (!FULL.value) {
+            if (kt >= KT) return; // uniform
+        }
+        // LDS destination = the piece's place in stage 0 (loop invariant) + the stage; both uniform
+        const uint32_t dst0 = lds0 + (uint32_t)(((piece >> 3) * OP_CHUNKS + (piece & 7) * 64 + wave_u * 512) * 16);
+        const uint32_t stage = (uint32_t)((kt & 1) * STAGE_CHUNKS * 16);
+        const uint32_t dst = dst0 + stage;
+        const char *base = (piece < 8) ? q_base + (int64_t)kt * (2 * BK) : p_base + (int64_t)kt * p_step_b; // uniform
+        const uint32_t off = (piece < 8) ? q_off[piece] : p_off[piece - 8];
+        if constexpr (FULL.value) {
+            asm volatile("s_add_i32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" ::"s"(dst0), "s"(stage), "v"(off),
+                         "s"(base)
+                         : "memory", "m0", "scc");
+        } else {
+            const char *src = base + off;
+            if (k_tail && kt == KT - 1) {
+                asm volatile("" ::: "memory");
+                if (piece < 8 || WT == 0) {
+                    if (kt * BK + rowmajor_lane_chunk(piece & 7, lane_v) * 8 >= a.K) src = (const char *)zero;
+                } else {
+                    if (kt * BK + wave_u * 16 + 2 * (piece - 8) + (lane_v >> 5) >= a.K) src = (const char *)zero;
+                }
+            }
+            lds_dma16_raw(src, dst);
+        }
+    };
+
+    // ---- first tile: its gathered rows are fetched on the spot, the rows of its epilogue go the way of all later ones
+    PstTile cur;
+    int e_buf = 0; // which of the two epilogue-row buffers holds the current tile's
+    {
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        cur = lookup((int)blockIdx.x, lane);
+        if (!cur.valid) return;
+        uint32_t q_raw[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int n = q_row(cur, i, lane, wave);
+            q_raw[i] = need_q_idx ? idx32[2 * (int64_t)n] : (uint32_t)n;
+        }
+        make_pointers(cur, lane, wave, q_raw);
+        wave_u = wave, lane_v = lane;
+        static_for<16>([&](auto P) { issue_piece(0, P, IC<0>{}); });
+        prefetch_rows(cur, lane, wave, false, e_buf);
+    }
+
+    [[maybe_unused]] int tile_no = 0;
+    for (;; ++tile_no) {
+        PST_STAMP(0);
+        // Everything derived from the thread index is derived again for every tile behind an opaque copy of it: hoisted
+        // out of the tile loop those values would live across the main loop and be spilled.
+        int tid = threadIdx.x;
+        asm volatile("" : "+v"(tid));
+        const int lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+        wave_u = wave, lane_v = lane;
+        // the first K step and the rows of this tile's epilogue have landed in every wave, the stores of the last
+        // epilogue have been handed over and its staging area is dead
+        asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
+        PST_STAMP(1);
+        static_for<DMA_N0>([&](auto P) { issue_piece(1, P, IC<0>{}); });
+
+        // one tile ahead: the next tile's schedule entry and rows, and this tile's row scales (their addresses are the
+        // epilogue's row indices, fetched a tile ago); all of it lands in LDS during the main loop
+        const PstTile nxt = lookup(cur.t + (int)gridDim.x, lane);
+        if (nxt.valid) prefetch_rows(nxt, lane, wave, true, e_buf ^ 1);
+        if (a.scale) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                // the aligned dword that holds the 16-bit scale (the host checks that the vector starts on 4 bytes)
+                const uint32_t s_idx = row_item(PST_ER + 4 * e_buf + i, tid);
+                lds_dma4_raw((const uint32_t *)a.scale + (s_idx >> 1), row_item_lds(PST_SC + i, wave));
+            }
+        }
+
+        PST_STAMP(2);
+        f32x16 acc[4][4];
+        zero_acc(acc);
+        const int wq = (wave & 1) * 128, wp = (wave >> 1) * 128;
+        FragBase<0> qb;
+        FragBase<WT> pb;
+        make_frag_base<0>(qb, lds0, wq, lane);
+        make_frag_base<WT>(pb, lds0 + OP_CHUNKS * 16, wp, lane);
+        const int q_blocks = (cur.rows_valid > wq) ? (cur.rows_valid - wq + 31) >> 5 : 0;
+        auto main_loop = [&](auto NI_) {
+            constexpr int NI = NI_.value;
+            Frags f0, f1;
+            if constexpr (NI > 0) {
+                static_for<4>([&](auto I) { f0.p[I.value] = read_frag<WT, I.value, 0>(pb); });
+                static_for<NI>([&](auto I) { f0.q[I.value] = read_frag<0, I.value, 0>(qb); });
+            }
+            auto k_step = [&](int kt, auto FULL) {
+                int kt_a = kt + 1, kt_b = kt + 2;
+                asm volatile("" : "+s"(kt_a), "+s"(kt_b));
+                mma_step<T, WT, 0, 1, NI>(f0, f1, pb, qb, acc, [&](auto G) {
+                    if constexpr (G.value < DMA_N1) issue_piece(kt_a, IC<DMA_N0 + G.value>{}, FULL);
+                });
+                mma_step<T, WT, 0, 2, NI>(f1, f0, pb, qb, acc, [&](auto G) {
+                    if constexpr (G.value < DMA_N2) issue_piece(kt_a, IC<DMA_N0 + DMA_N1 + G.value>{}, FULL);
+                });
+                mma_step<T, WT, 0, 3, NI>(f0, f1, pb, qb, acc, NoHook());
+                XMA_WAIT_LOADS_AND_BARRIER();
+                flip_stage(pb);
+                flip_stage(qb);
+                mma_step<T, WT, 0, 0, NI>(f1, f0, pb, qb, acc, [&](auto G) {
+                    if constexpr (G.value < DMA_N0) issue_piece(kt_b, G, FULL);
+                    if constexpr (G.value + 8 < DMA_N0) issue_piece(kt_b, IC<G.value + 8>{}, FULL);
+                });
+            };
+            int kt = 0;
+            if constexpr (NI == 4)
+                for (; kt + 2 < KT_full; ++kt) k_step(kt, IC<1>{});
+            for (; kt < KT; ++kt) k_step(kt, IC<0>{});
+        };
+        if (q_blocks > 2)
+            main_loop(IC<4>{});
+        else if (q_blocks == 2)
+            main_loop(IC<2>{});
+        else if (q_blocks == 1)
+            main_loop(IC<1>{});
+        else
+            main_loop(IC<0>{});
+        // every load has landed (the index loads above as well), no wave touches the operand tiles any more
+        XMA_WAIT_LOADS_AND_BARRIER();
+        PST_STAMP(3);
+
+        int tid_e = threadIdx.x;
+        asm volatile("" : "+v"(tid_e));
+        const int lane_e = tid_e & 63, wave_e = __builtin_amdgcn_readfirstlane(tid_e >> 6);
+        if (nxt.valid) { // first K step of the next tile: in flight during the epilogue
+            uint32_t q_raw[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                q_raw[i] = need_q_idx ? row_item(PST_QR + i, tid_e) : (uint32_t)q_row(nxt, i, lane_e, wave_e);
+            make_pointers(nxt, lane_e, wave_e, q_raw);
+            wave_u = wave_e, lane_v = lane_e;
+            static_for<16>([&](auto P) { issue_piece(0, P, IC<0>{}); });
+        }
+        PST_STAMP(4);
+        EpiRows er;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const uint32_t s_idx = need_e_idx ? row_item(PST_ER + 4 * e_buf + i, tid_e) : 0u;
+            er.idx[i] = (int)s_idx;
+            er.sc[i] = 1.f;
+            if (a.scale) {
+                const uint32_t w = row_item(PST_SC + i, tid_e);
+                er.sc[i] = (s_idx & 1) ? Elem<T>::hi(w) : Elem<T>::lo(w);
+            }
+        }
+        tile_epilogue<T, EPI>(a, acc, smem + PST_STAGING_OFF, cur.row0, cur.rows_valid, cur.n0, tid_e, -1, &er);
+        PST_STAMP(5);
+        if (!nxt.valid) break;
+        cur = nxt;
+        e_buf ^= 1;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
 // dW kernel: DW[e][o][i] = sum_n DY[n][o] X[n][i]; both operands are token-major = transposed sources; the K loop
 // runs over the expert's row range, k-rows past its end come from the zero page.
 //   GQ / GP = 1: the rows of dY / X are taken through sorted_scattered_idxs (index / fan_out); 0: grouped order
@@ -984,15 +1369,25 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
 
 inline int device_cus();
 template <typename T, int WT, int EPI> int launch_fwd(const FwdArgs &a, hipStream_t st) {
-    int rc = gemm_set_smem(grouped_gemm_kernel<T, WT, EPI, ROLE_TILES>, GEMM_SMEM_BYTES);
-    if (rc) return rc;
-    int launch_grid = a.grid_main;
-    if (fwd_persistent(EPI, ROLE_TILES)) {
-        const int cus = device_cus();
-        if (cus > 0 && cus < launch_grid) launch_grid = cus;
+    int rc;
+    const int cus = device_cus();
+    // The persistent kernel fetches a row scale as the aligned dword around it and addresses the operands of a tile with
+    // 32-bit byte offsets from a uniform base: 256 rows of W or of a grouped X, any row of a gathered X.
+    const int64_t x_rows = a.x_grouped ? 256 : (a.M + a.fan_out - 1) / a.fan_out;
+    const bool offsets_fit = x_rows * a.ldx * 2 < ((int64_t)1 << 32) && (int64_t)256 * a.ldw * 2 < ((int64_t)1 << 32);
+    if (a.E <= PST_MAX_E && cus > 0 && ((uintptr_t)a.scale & 3) == 0 && offsets_fit) {
+        // whole tiles: one persistent workgroup per compute unit
+        if ((rc = gemm_set_smem(grouped_gemm_persistent_kernel<T, WT, EPI>, PST_SMEM_BYTES))) return rc;
+        const int launch_grid = cus < a.grid_main ? cus : a.grid_main;
+        grouped_gemm_persistent_kernel<T, WT, EPI><<<launch_grid, GEMM_THREADS, PST_SMEM_BYTES, st>>>(a);
+        if ((rc = xma_check_launch("grouped_gemm_persistent_kernel"))) return rc;
+    } else {
+        if ((rc = gemm_set_smem(grouped_gemm_kernel<T, WT, EPI, ROLE_TILES>, GEMM_SMEM_BYTES))) return rc;
+        int launch_grid = a.grid_main;
+        if (fwd_persistent(EPI, ROLE_TILES) && cus > 0 && cus < launch_grid) launch_grid = cus;
+        grouped_gemm_kernel<T, WT, EPI, ROLE_TILES><<<launch_grid, GEMM_THREADS, GEMM_SMEM_BYTES, st>>>(a);
+        if ((rc = xma_check_launch("grouped_gemm_kernel"))) return rc;
     }
-    grouped_gemm_kernel<T, WT, EPI, ROLE_TILES><<<launch_grid, GEMM_THREADS, GEMM_SMEM_BYTES, st>>>(a);
-    if ((rc = xma_check_launch("grouped_gemm_kernel"))) return rc;
     if (!a.partial) return XMA_ROCM_OK;
     // the tiles of the last round as K slices (no epilogue: one instantiation serves all), then their sum + epilogue
     if ((rc = gemm_set_smem(grouped_gemm_kernel<T, WT, XMA_ROCM_EPI_STORE, ROLE_SLICES>, GEMM_SMEM_BYTES))) return rc;
@@ -1130,6 +1525,17 @@ extern "C" int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *
     if (dtype == XMA_ROCM_BF16) return dispatch_fwd<__bf16>(a, w_is_kn ? 1 : 0, epilogue, st);
     return dispatch_fwd<_Float16>(a, w_is_kn ? 1 : 0, epilogue, st);
 }
+
+#ifdef XMA_PST_TIMING
+extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_times(void *host_out) {
+    return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_pst_times), sizeof(g_pst_times));
+}
+extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_reset(void) {
+    void *p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_pst_times)) != hipSuccess) return -1;
+    return (int)hipMemset(p, 0, sizeof(g_pst_times));
+}
+#endif
 
 extern "C" size_t xma_rocm_scatter2scatter_workspace_bytes(int64_t M, int32_t N, int32_t K, int32_t E) {
     (void)K;

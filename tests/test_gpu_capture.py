@@ -24,9 +24,14 @@ def _make(T=300, E=8, k=2, H=256, I=512, dtype=torch.bfloat16, seed=0):
     return moe, x
 
 
-def test_compiled_module_matches_eager():
+@pytest.mark.parametrize("backend", ["aot_eager", "inductor"])
+def test_compiled_module_matches_eager(backend):
+    """torch.compile(fullgraph=True) of the module, with the tracing-only backend and with the default one the
+    reference's test uses (tests/layers/moe_test.py:104-105 passes no backend, i.e. inductor): the custom ops mutate
+    caller-allocated outputs, so functionalisation has to carry them through unchanged."""
     from xma import KernelBackend
 
+    torch._dynamo.reset()
     moe, x = _make()
     print("compile: eager run", flush=True)
     xe = x.clone().requires_grad_()
@@ -37,16 +42,25 @@ def test_compiled_module_matches_eager():
     for p in moe.parameters():
         p.grad = None
     print("compile: compiled run (fullgraph)", flush=True)
-    cmoe = torch.compile(moe, fullgraph=True, backend="aot_eager")
+    cmoe = torch.compile(moe, fullgraph=True, backend=backend)
     xc = x.clone().requires_grad_()
-    yc, _ = cmoe(xc, kernel_backend=KernelBackend.rocm)
-    yc.sum().backward()
+    try:
+        yc, _ = cmoe(xc, kernel_backend=KernelBackend.rocm)
+        yc.sum().backward()
+    except torch._dynamo.exc.BackendCompilerFailed as err:  # the code generator's own toolchain, not the ops under test
+        if backend == "inductor":
+            pytest.skip(f"inductor cannot generate code on this machine: {str(err)[:300]}")
+        raise
     torch.cuda.synchronize()
     got = {"y": yc, "dx": xc.grad, "dw_fc": moe.c_fc.weight.grad, "dw_proj": moe.c_proj.weight.grad,
            "dgate": moe.gate.weight.grad}
     for name in want:
-        # same kernels on the same inputs: bit-identical
-        assert torch.equal(got[name], want[name]), name
+        # same kernels on the same inputs: bit-identical.  The code generator may fold the sum of the two contributions
+        # to dx (experts and gate) and the gate's stock GEMMs into other kernels than eager mode runs: one rounding apart.
+        if backend == "inductor" and name in ("dx", "dgate"):
+            assert nerr(got[name], want[name]) <= 2.0**-7, name  # a unit in the last place of bf16
+        else:
+            assert torch.equal(got[name], want[name]), name
 
 
 def test_graph_capture_and_replay():
