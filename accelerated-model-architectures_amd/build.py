@@ -97,10 +97,10 @@ def _check_compiler(verbose: bool) -> None:
         print(f"hipcc {version}", flush=True)
 
 
-def _compile(src: str, verbose: bool) -> str:
-    obj = os.path.join(HERE, "build", src.replace(".hip", ".o"))
+def _compile(src: str, verbose: bool, defines: tuple[str, ...] = (), tag: str = "") -> str:
+    obj = os.path.join(HERE, "build", src.replace(".hip", tag + ".o"))
     extra = ["-save-temps=obj"] if src in LOOP_NO_SCRATCH else []  # keeps the device ISA next to the object
-    cmd = [HIPCC, *FLAGS, *extra, "-c", os.path.join(CSRC, src), "-o", obj]
+    cmd = [HIPCC, *FLAGS, *extra, *defines, "-c", os.path.join(CSRC, src), "-o", obj]
     if verbose:
         print(" ".join(cmd), flush=True)
     r = subprocess.run(cmd, capture_output=True, text=True)
@@ -113,7 +113,7 @@ def _compile(src: str, verbose: bool) -> str:
     if re.search(r"warning|error", err) and verbose:
         print(err, file=sys.stderr)
     if src in LOOP_NO_SCRATCH:
-        asm = os.path.join(HERE, "build", src.replace(".hip", "-hip-amdgcn-amd-amdhsa-gfx950.s"))
+        asm = os.path.join(HERE, "build", src.replace(".hip", tag + "-hip-amdgcn-amd-amdhsa-gfx950.s"))
         bad = _scratch_inside_mfma_loop(asm, LOOP_NO_SCRATCH[src])
         if bad:
             raise RuntimeError(f"{src}: scratch accesses inside the MFMA loop of:\n  " + "\n  ".join(bad))
@@ -141,5 +141,21 @@ def build(verbose: bool = False) -> str:
     return LIB
 
 
+TIMING_LIB = os.path.join(OUT_DIR, "libxma_rocm_timing.so")
+
+
+def build_timing(verbose: bool = False) -> str:
+    """A second library for diagnostics/tile_phases.py: grouped_gemm.hip compiled with -DXMA_PST_TIMING (the persistent
+    GEMM kernel stamps the real-time counter at six points of every tile), linked with the objects of the normal build.
+    Not part of build(): nothing in the product loads it."""
+    build(verbose)
+    obj, _ = _compile("grouped_gemm.hip", verbose, ("-DXMA_PST_TIMING",), "_timing")
+    objs = [obj if s == "grouped_gemm.hip" else os.path.join(HERE, "build", s.replace(".hip", ".o")) for s in SOURCES]
+    r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", TIMING_LIB, *objs], capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"link failed:\n{r.stderr}")
+    return TIMING_LIB
+
+
 if __name__ == "__main__":
-    print(build(verbose=True))
+    print(build_timing(verbose=True) if "--timing" in sys.argv[1:] else build(verbose=True))

@@ -263,6 +263,37 @@ struct TileSched {
     int tail_index;        // index of a split tile among the tiles of the last round
 };
 
+// Order of an expert's tiles.  The 32 consecutive tiles that xcd_remap hands to an XCD share operand panels in that XCD's
+// L2: r row tiles x c column tiles need r activation panels and c weight panels for r c tiles, and the K loop runs as
+// fast as those panels arrive.  Walking all row tiles of a column before the next column suits an expert of up to a
+// dozen row tiles (measured best for 9: 9 + 3.6 panels, and the same activation panels in every round of the launch);
+// an expert of 48 row tiles would have 32 tiles share one weight panel and fetch 32 activation panels (measured: the
+// K loop of an expert of 64 row tiles takes 142 us instead of 100).  So the row tiles of a larger expert are cut into
+// bands of equal height, at most FWD_BAND, and the walk goes down a band's column, then along the band, then to the next
+// band.  Low bands measured better than square ones (4 x 8 before 6 x 5 before 8 x 4): a weight panel is one
+// contiguous block, an activation panel 256 gathered rows.  local: index of the tile among the expert's tiles_m x NT.
+constexpr int FWD_SINGLE_BAND_TILES = 12;
+#ifdef XMA_PST_TIMING
+__device__ int g_pst_band = 6; // A/B switch of the timing build
+#define FWD_BAND g_pst_band
+#else
+constexpr int FWD_BAND = 6;
+#endif
+__device__ __forceinline__ void tile_of_expert(int local, int tiles_m, int NT, int &m_tile, int &n_tile) {
+    if (tiles_m <= FWD_SINGLE_BAND_TILES) {
+        m_tile = local % tiles_m, n_tile = local / tiles_m;
+        return;
+    }
+    const int bands = (tiles_m + FWD_BAND - 1) / FWD_BAND;
+    const int h = (tiles_m + bands - 1) / bands; // height of every band but the last, which has what is left
+    int band = local / (h * NT);
+    if (band > bands - 1) band = bands - 1;
+    const int in_band = local - band * h * NT;
+    const int rows = (band == bands - 1) ? tiles_m - h * (bands - 1) : h;
+    m_tile = band * h + in_band % rows;
+    n_tile = in_band / rows;
+}
+
 constexpr int SPLIT_MIN_STEPS = 8; // a K slice is at least this many K steps
 
 // Expert-major schedule: work[e] = ceil(rows_e / BM) * n_tiles, prefix sum over the experts in LDS, then the tile of
@@ -371,7 +402,8 @@ __device__ __forceinline__ bool locate_tile(const FwdArgs &a, unsigned char *sme
         __syncthreads(); // s_pre is dead from here on
     }
     const int tiles_m = (int)((row_hi - row_lo + BM - 1) / BM);
-    const int m_tile = local % tiles_m, n_tile = local / tiles_m;
+    int m_tile, n_tile;
+    tile_of_expert(local, tiles_m, NT, m_tile, n_tile);
     ts.e = e;
     ts.row0 = row_lo + (int64_t)m_tile * BM;
     ts.rows_valid = (int)((row_hi - ts.row0 < BM) ? row_hi - ts.row0 : BM);
@@ -835,6 +867,7 @@ __device__ __forceinline__ void lds_dma4_raw(const void *src, uint32_t lds_wave_
 #ifdef XMA_PST_TIMING
 constexpr int PST_TIMING_TILES = 48;
 __device__ uint64_t g_pst_times[256][PST_TIMING_TILES][8];
+__device__ int g_pst_no_ovl; // A/B switch of the timing build: 1 = no tile overlaps its neighbours' set-up
 #define PST_STAMP(k)                                                                                   \
     do {                                                                                               \
         if (threadIdx.x == 0 && blockIdx.x < 256 && tile_no < PST_TIMING_TILES)                        \
@@ -901,8 +934,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
 
     // first tile at or behind position t of this workgroup's walk (every wave computes the same, from LDS only)
     auto lookup = [&](int t, int lane) -> PstTile {
-        PstTile r;
-        r.valid = 0;
+        PstTile r = {0, 0, 0, 0, 0, 0};
         for (; t < a.grid_main; t += gridDim.x) {
             const int L = xcd_remap(t, a.grid_main);
             if (L >= full) continue;
@@ -924,7 +956,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
             const int row_hi = __builtin_amdgcn_readfirstlane(s_hi[e]);
             const int row_lo = e ? __builtin_amdgcn_readfirstlane(s_hi[e - 1]) : 0;
             const int tiles_m = (row_hi - row_lo + BM - 1) / BM;
-            const int m_tile = local % tiles_m, n_tile = local / tiles_m;
+            int m_tile, n_tile;
+            tile_of_expert(local, tiles_m, NT, m_tile, n_tile);
             r.valid = 1;
             r.t = t;
             r.e = e;
@@ -962,6 +995,27 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
         }
     };
 
+    // The same fetches as 16 items of one LDS-DMA load each, for the first K step of a tile to issue one by one between
+    // its MFMAs: 0..7 the gathered rows of the next tile, 8..11 the rows of its epilogue, 12..15 the row scales of this
+    // tile.  An item that is not needed loads from the zero page instead, so that their number is always 16 and the wait
+    // in front of that step's barrier can leave exactly these loads in flight.
+    auto prefetch_item = [&](auto ITEM, const PstTile &t, int lane, int wave, int tid, int e_buf) {
+        constexpr int it = ITEM.value;
+        const void *src = zero;
+        uint32_t dst;
+        if constexpr (it < 8) {
+            dst = row_item_lds(PST_QR + it, wave);
+            if (t.valid && need_q_idx) src = idx32 + 2 * (int64_t)q_row(t, it, lane, wave);
+        } else if constexpr (it < 12) {
+            dst = row_item_lds(PST_ER + 4 * (e_buf ^ 1) + (it - 8), wave);
+            if (t.valid && need_e_idx) src = idx32 + 2 * (int64_t)e_row(t, it - 8, lane, wave);
+        } else {
+            dst = row_item_lds(PST_SC + (it - 12), wave);
+            if (a.scale) src = (const uint32_t *)a.scale + (row_item(PST_ER + 4 * e_buf + (it - 12), tid) >> 1);
+        }
+        lds_dma4_raw(src, dst);
+    };
+
     // Addresses of the 16 LDS-DMA pieces of a tile: a uniform base per operand (SGPRs: the tile's corner of the weight
     // matrix; the activations' first row for a gathered operand, the tile's first row for a grouped one) and one 32-bit
     // byte offset per piece and lane.  A K step adds a uniform amount to the bases, so a piece in the loop is the M0
@@ -969,32 +1023,30 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
     uint32_t q_off[8], p_off[8];
     const char *q_base = nullptr, *p_base = nullptr;
     const int64_t p_step_b = (WT == 0) ? 2 * BK : (int64_t)2 * BK * a.ldw; // bytes per K step along the weights
-    auto make_pointers = [&](const PstTile &t, int lane, int wave, const uint32_t (&raw)[8]) {
-        const uint16_t *We = a.W + (int64_t)t.e * a.w_es;
+    // offsets of pieces i (activations) and 8 + i (weights); i == 0 also sets the two bases; raw: the row of piece i (its
+    // scattered index for a gathered operand)
+    auto make_pointer = [&](const PstTile &t, auto I_, int lane, int wave, uint32_t raw) {
+        constexpr int i = I_.value;
+        if constexpr (i == 0) {
+            const uint16_t *We = a.W + (int64_t)t.e * a.w_es;
+            p_base = (WT == 0) ? (const char *)(We + (int64_t)t.n0 * a.ldw) : (const char *)(We + t.n0);
+            q_base = (const char *)(need_q_idx ? a.X : a.X + (int64_t)t.row0 * a.ldx);
+        }
         if (WT == 0) {
-            p_base = (const char *)(We + (int64_t)t.n0 * a.ldw);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                int r = wave * 64 + i * 8 + (lane >> 3);
-                if (t.n0 + r >= a.N) r = a.N - 1 - t.n0;
-                p_off[i] = (uint32_t)r * (uint32_t)(2 * a.ldw) + rowmajor_lane_chunk(i, lane) * 16;
-            }
+            int r = wave * 64 + i * 8 + (lane >> 3);
+            if (t.n0 + r >= a.N) r = a.N - 1 - t.n0;
+            p_off[i] = (uint32_t)r * (uint32_t)(2 * a.ldw) + rowmajor_lane_chunk(i, lane) * 16;
         } else {
-            p_base = (const char *)(We + t.n0);
             const int max_chunk = ((a.N - t.n0) >> 3) - 1;
-#pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                int cj = transposed_lane_chunk(j, lane);
-                if (cj > max_chunk) cj = max_chunk;
-                p_off[j] = (uint32_t)(wave * 16 + 2 * j + (lane >> 5)) * (uint32_t)(2 * a.ldw) + cj * 16;
-            }
+            int cj = transposed_lane_chunk(i, lane);
+            if (cj > max_chunk) cj = max_chunk;
+            p_off[i] = (uint32_t)(wave * 16 + 2 * i + (lane >> 5)) * (uint32_t)(2 * a.ldw) + cj * 16;
         }
-        q_base = (const char *)(need_q_idx ? a.X : a.X + (int64_t)t.row0 * a.ldx);
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t src = need_q_idx ? fastdiv(raw[i], a.fan_div) : raw[i] - (uint32_t)t.row0;
-            q_off[i] = src * (uint32_t)(2 * a.ldx) + rowmajor_lane_chunk(i, lane) * 16;
-        }
+        const uint32_t src = need_q_idx ? fastdiv(raw, a.fan_div) : raw - (uint32_t)t.row0;
+        q_off[i] = src * (uint32_t)(2 * a.ldx) + rowmajor_lane_chunk(i, lane) * 16;
+    };
+    auto make_pointers = [&](const PstTile &t, int lane, int wave, const uint32_t (&raw)[8]) {
+        static_for<8>([&](auto I) { make_pointer(t, I, lane, wave, raw[I.value]); });
     };
     // piece 0..15 of K step kt of the tile the bases and offsets describe -> stage kt & 1; FULL: the step exists and has
     // no chunk past K
@@ -1050,6 +1102,11 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
         prefetch_rows(cur, lane, wave, false, e_buf);
     }
 
+#ifdef XMA_PST_TIMING
+    const bool ovl_allowed = !g_pst_no_ovl;
+#else
+    constexpr bool ovl_allowed = true;
+#endif
     [[maybe_unused]] int tile_no = 0;
     for (;; ++tile_no) {
         PST_STAMP(0);
@@ -1065,28 +1122,37 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
         PST_STAMP(1);
         static_for<DMA_N0>([&](auto P) { issue_piece(1, P, IC<0>{}); });
 
-        // one tile ahead: the next tile's schedule entry and rows, and this tile's row scales (their addresses are the
-        // epilogue's row indices, fetched a tile ago); all of it lands in LDS during the main loop
-        const PstTile nxt = lookup(cur.t + (int)gridDim.x, lane);
-        if (nxt.valid) prefetch_rows(nxt, lane, wave, true, e_buf ^ 1);
-        if (a.scale) {
+        // One tile ahead: the next tile's schedule entry and rows, and this tile's row scales (their addresses are the
+        // epilogue's row indices, fetched a tile ago); all of it lands in LDS during the main loop.  A full tile with an
+        // even number of at least four K steps does this between the MFMAs of its first K step, and sets up and issues
+        // the first K step of the next tile between the MFMAs of its last one (`ovl`); any other tile does it here and
+        // behind the loop, with idle matrix pipes.
+        const int wq = (wave & 1) * 128, wp = (wave >> 1) * 128;
+        const int q_blocks = (cur.rows_valid > wq) ? (cur.rows_valid - wq + 31) >> 5 : 0;
+        // uniform over the workgroup: the waves of a tile's lower half (wq == 0) and upper half disagree on q_blocks, so
+        // the decision is taken on the tile's row count
+        const bool ovl = cur.rows_valid > 128 + 64 && (KT & 1) == 0 && KT >= 4 && ovl_allowed;
+        PstTile nxt = {0, 0, 0, 0, 0, 0};
+        if (!ovl) {
+            nxt = lookup(cur.t + (int)gridDim.x, lane);
+            if (nxt.valid) prefetch_rows(nxt, lane, wave, true, e_buf ^ 1);
+            if (a.scale) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                // the aligned dword that holds the 16-bit scale (the host checks that the vector starts on 4 bytes)
-                const uint32_t s_idx = row_item(PST_ER + 4 * e_buf + i, tid);
-                lds_dma4_raw((const uint32_t *)a.scale + (s_idx >> 1), row_item_lds(PST_SC + i, wave));
+                for (int i = 0; i < 4; ++i) {
+                    // the aligned dword that holds the 16-bit scale (the host checks that the vector starts on 4 bytes)
+                    const uint32_t s_idx = row_item(PST_ER + 4 * e_buf + i, tid);
+                    lds_dma4_raw((const uint32_t *)a.scale + (s_idx >> 1), row_item_lds(PST_SC + i, wave));
+                }
             }
         }
 
         PST_STAMP(2);
         f32x16 acc[4][4];
         zero_acc(acc);
-        const int wq = (wave & 1) * 128, wp = (wave >> 1) * 128;
         FragBase<0> qb;
         FragBase<WT> pb;
         make_frag_base<0>(qb, lds0, wq, lane);
         make_frag_base<WT>(pb, lds0 + OP_CHUNKS * 16, wp, lane);
-        const int q_blocks = (cur.rows_valid > wq) ? (cur.rows_valid - wq + 31) >> 5 : 0;
         auto main_loop = [&](auto NI_) {
             constexpr int NI = NI_.value;
             Frags f0, f1;
@@ -1094,28 +1160,68 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
                 static_for<4>([&](auto I) { f0.p[I.value] = read_frag<WT, I.value, 0>(pb); });
                 static_for<NI>([&](auto I) { f0.q[I.value] = read_frag<0, I.value, 0>(qb); });
             }
-            auto k_step = [&](int kt, auto FULL) {
+            // One K step.  FULL: steps kt + 1 and kt + 2 exist and are complete.  MODE 1, the first step of a tile that
+            // overlaps (`ovl`): the free slots of its second half take the next tile's schedule entry and the 16 row
+            // items; they are the youngest loads at the step's barrier, which leaves exactly them in flight.  MODE 2, the
+            // last step of such a tile (it lives in stage 1, stage 0 has been free since the barrier before): its slots
+            // take the operand addresses of the next tile and the 16 pieces of that tile's first K step, which stay in
+            // flight through the epilogue.  The loads of this tile have all been issued by then.
+            auto k_step = [&](int kt, auto FULL, auto MODE) {
+                constexpr int mode = MODE.value;
                 int kt_a = kt + 1, kt_b = kt + 2;
                 asm volatile("" : "+s"(kt_a), "+s"(kt_b));
                 mma_step<T, WT, 0, 1, NI>(f0, f1, pb, qb, acc, [&](auto G) {
-                    if constexpr (G.value < DMA_N1) issue_piece(kt_a, IC<DMA_N0 + G.value>{}, FULL);
+                    if constexpr (mode == 2) {
+                        // also when there is no next tile (all fields zero then: addresses that nothing is loaded from):
+                        // a branch here would only add a join of sixteen registers to the loop
+                        make_pointer(nxt, G, lane, wave,
+                                     need_q_idx ? row_item(PST_QR + G.value, tid) : (uint32_t)q_row(nxt, G.value, lane, wave));
+                    } else if constexpr (G.value < DMA_N1) {
+                        issue_piece(kt_a, IC<DMA_N0 + G.value>{}, FULL);
+                    }
                 });
                 mma_step<T, WT, 0, 2, NI>(f1, f0, pb, qb, acc, [&](auto G) {
-                    if constexpr (G.value < DMA_N2) issue_piece(kt_a, IC<DMA_N0 + DMA_N1 + G.value>{}, FULL);
+                    if constexpr (mode == 1) {
+                        if constexpr (G.value == 0) nxt = lookup(cur.t + (int)gridDim.x, lane);
+                    } else if constexpr (mode == 2) {
+                        if (nxt.valid) issue_piece(0, G, IC<1>{});
+                    } else if constexpr (G.value < DMA_N2) {
+                        issue_piece(kt_a, IC<DMA_N0 + DMA_N1 + G.value>{}, FULL);
+                    }
                 });
-                mma_step<T, WT, 0, 3, NI>(f0, f1, pb, qb, acc, NoHook());
-                XMA_WAIT_LOADS_AND_BARRIER();
+                mma_step<T, WT, 0, 3, NI>(f0, f1, pb, qb, acc, [&](auto G) {
+                    if constexpr (mode == 1) {
+                        prefetch_item(IC<2 * G.value>{}, nxt, lane, wave, tid, e_buf);
+                        prefetch_item(IC<2 * G.value + 1>{}, nxt, lane, wave, tid, e_buf);
+                    } else if constexpr (mode == 2) {
+                        if (nxt.valid) issue_piece(0, IC<8 + G.value>{}, IC<1>{});
+                    }
+                });
+                if constexpr (mode == 0)
+                    XMA_WAIT_LOADS_AND_BARRIER(); // step kt + 1 has landed; nobody reads this stage any more
+                else
+                    asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory"); // all but the 16 youngest
                 flip_stage(pb);
                 flip_stage(qb);
                 mma_step<T, WT, 0, 0, NI>(f1, f0, pb, qb, acc, [&](auto G) {
-                    if constexpr (G.value < DMA_N0) issue_piece(kt_b, G, FULL);
-                    if constexpr (G.value + 8 < DMA_N0) issue_piece(kt_b, IC<G.value + 8>{}, FULL);
+                    if constexpr (mode != 2) {
+                        if constexpr (G.value < DMA_N0) issue_piece(kt_b, G, FULL);
+                        if constexpr (G.value + 8 < DMA_N0) issue_piece(kt_b, IC<G.value + 8>{}, FULL);
+                    }
                 });
             };
-            int kt = 0;
-            if constexpr (NI == 4)
-                for (; kt + 2 < KT_full; ++kt) k_step(kt, IC<1>{});
-            for (; kt < KT; ++kt) k_step(kt, IC<0>{});
+            int kt = 0, kt_end = KT;
+            if constexpr (NI == 4) {
+                if (ovl) { // KT >= 4, so the first step is followed by two complete ones
+                    k_step(0, IC<1>{}, IC<1>{});
+                    kt = 1, kt_end = KT - 1;
+                }
+                for (; kt + 2 < KT_full && kt < kt_end; ++kt) k_step(kt, IC<1>{}, IC<0>{});
+            }
+            for (; kt < kt_end; ++kt) k_step(kt, IC<0>{}, IC<0>{});
+            if constexpr (NI == 4) {
+                if (ovl) k_step(KT - 1, IC<0>{}, IC<2>{});
+            }
         };
         if (q_blocks > 2)
             main_loop(IC<4>{});
@@ -1125,14 +1231,20 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
             main_loop(IC<1>{});
         else
             main_loop(IC<0>{});
-        // every load has landed (the index loads above as well), no wave touches the operand tiles any more
-        XMA_WAIT_LOADS_AND_BARRIER();
+        if (ovl) {
+            // The waves met at the last step's barrier with their reads of stage 1 done; only the read-ahead of the last
+            // sub-step is in flight, into registers nobody uses, and the next tile's first K step, into stage 0.
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        } else {
+            // every load has landed (the index loads above as well), no wave touches the operand tiles any more
+            XMA_WAIT_LOADS_AND_BARRIER();
+        }
         PST_STAMP(3);
 
         int tid_e = threadIdx.x;
         asm volatile("" : "+v"(tid_e));
         const int lane_e = tid_e & 63, wave_e = __builtin_amdgcn_readfirstlane(tid_e >> 6);
-        if (nxt.valid) { // first K step of the next tile: in flight during the epilogue
+        if (!ovl && nxt.valid) { // first K step of the next tile: in flight during the epilogue
             uint32_t q_raw[8];
 #pragma unroll
             for (int i = 0; i < 8; ++i)
@@ -1375,13 +1487,22 @@ template <typename T, int WT, int EPI> int launch_fwd(const FwdArgs &a, hipStrea
     // 32-bit byte offsets from a uniform base: 256 rows of W or of a grouped X, any row of a gathered X.
     const int64_t x_rows = a.x_grouped ? 256 : (a.M + a.fan_out - 1) / a.fan_out;
     const bool offsets_fit = x_rows * a.ldx * 2 < ((int64_t)1 << 32) && (int64_t)256 * a.ldw * 2 < ((int64_t)1 << 32);
-    if (a.E <= PST_MAX_E && cus > 0 && ((uintptr_t)a.scale & 3) == 0 && offsets_fit) {
-        // whole tiles: one persistent workgroup per compute unit
-        if ((rc = gemm_set_smem(grouped_gemm_persistent_kernel<T, WT, EPI>, PST_SMEM_BYTES))) return rc;
-        const int launch_grid = cus < a.grid_main ? cus : a.grid_main;
-        grouped_gemm_persistent_kernel<T, WT, EPI><<<launch_grid, GEMM_THREADS, PST_SMEM_BYTES, st>>>(a);
-        if ((rc = xma_check_launch("grouped_gemm_persistent_kernel"))) return rc;
-    } else {
+    // The persistent kernel exists for the operand layouts the layer launches: x @ W^T with any epilogue, dy @ W with a
+    // plain store or the SwiGLU backward.  (dy @ W with the SwiGLU forward epilogue, reachable through the C ABI only,
+    // would be the one instantiation whose register allocation spills inside the K loop.)
+    constexpr bool persistent_variant = !(WT == 1 && EPI == XMA_ROCM_EPI_SWIGLU);
+    bool persistent = false;
+    if constexpr (persistent_variant) {
+        if (a.E <= PST_MAX_E && cus > 0 && ((uintptr_t)a.scale & 3) == 0 && offsets_fit) {
+            // whole tiles: one persistent workgroup per compute unit
+            if ((rc = gemm_set_smem(grouped_gemm_persistent_kernel<T, WT, EPI>, PST_SMEM_BYTES))) return rc;
+            const int launch_grid = cus < a.grid_main ? cus : a.grid_main;
+            grouped_gemm_persistent_kernel<T, WT, EPI><<<launch_grid, GEMM_THREADS, PST_SMEM_BYTES, st>>>(a);
+            if ((rc = xma_check_launch("grouped_gemm_persistent_kernel"))) return rc;
+            persistent = true;
+        }
+    }
+    if (!persistent) {
         if ((rc = gemm_set_smem(grouped_gemm_kernel<T, WT, EPI, ROLE_TILES>, GEMM_SMEM_BYTES))) return rc;
         int launch_grid = a.grid_main;
         if (fwd_persistent(EPI, ROLE_TILES) && cus > 0 && cus < launch_grid) launch_grid = cus;
@@ -1529,6 +1650,12 @@ extern "C" int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *
 #ifdef XMA_PST_TIMING
 extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_times(void *host_out) {
     return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_pst_times), sizeof(g_pst_times));
+}
+extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_band(int v) {
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_pst_band), &v, sizeof(v));
+}
+extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_no_ovl(int v) {
+    return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_pst_no_ovl), &v, sizeof(v));
 }
 extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_reset(void) {
     void *p = nullptr;

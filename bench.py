@@ -46,8 +46,8 @@ WORKLOADS = {
 # 1.0: the factors a 1 GiB device copy, `--workload copy`, gives for the same counters).  bench.py cannot read hardware
 # counters itself: the figures are copied from the profile named beside them and are NOT measured in this run.
 MEASURED_TRAFFIC_BYTES = {
-    "c3": 9.31e9,  # up-projection + SwiGLU GEMM: 7.89 GB fetched + 1.42 GB written (3.42 GB algorithmic)
-    "c2": 92.2e6,  # route: unit histogram 17.1 MB + scan 4.2 MB + scatter 70.9 MB (17.1 MB fetched + 53.8 MB written)
+    "c3": 8.97e9,  # up-projection + SwiGLU GEMM: 7.56 GB fetched + 1.41 GB written (3.42 GB algorithmic)
+    "c2": 92.2e6,  # route: unit histogram 18.9 MB + scan 0.6 MB + scatter 72.7 MB (36.1 MB fetched + 56.2 MB written)
 }
 TRAFFIC_SOURCE = "profiles/hbm_traffic_c3_c2_pmc.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE; a constant, not measured in this run)"
 
@@ -162,8 +162,12 @@ def _kernel_table(moe, x, rw, sel, grad, cfg, iters):
     mem("combine_bwd", rotating(lambda i: ops.combine_bwd_rocm(eos[i], grads[i], d_rw)), Tk * H * esz + T * H * esz + T * k * esz)
     mem("group(dy*w)", rotating(lambda i: ops.group_rocm(grads[i], ss, gdys[i], flat_w, k)),
         T * H * esz + Tk * H * esz + Tk * (8 + esz))
-    notes = {"hbm_kernels": f"combine, combine_bwd and group(dy*w) timed on {nset} rotating buffer sets "
-                            f"({nset * comb_bytes >> 20} MiB, more than the Infinity Cache): cold figures"}
+    # what the machine does with the plainest kernels on the same buffers: a device-to-device copy and a fill of Tk x H
+    mem("reference: copy of (Tk,H) [torch copy_]", rotating(lambda i: gdys[i].copy_(eos[i])), 2 * Tk * H * esz)
+    mem("reference: fill of (Tk,H) [torch fill_]", rotating(lambda i: gdys[i].fill_(1.0)), Tk * H * esz)
+    notes = {"hbm_kernels": f"combine, combine_bwd, group(dy*w) and the two reference lines timed on {nset} rotating buffer "
+                            f"sets ({nset * comb_bytes >> 20} MiB, more than the Infinity Cache): cold figures; the reference "
+                            f"lines are stock torch kernels, the rate a plain copy / fill of the same size reaches here"}
     del eos, ys, grads, gdys
     mem("route", lambda: R.route(sel, E), Tk * 8 + Tk * 8 + Tk * 8 + E * 20)
     # the router: top-k + softmax + ids from given logits (part of the timed step), and fused with the gate projection
@@ -370,6 +374,24 @@ def run_routing(args):
     route_ms = _time_gpu(step, args.kernel_iters * 5, warmup=5)
     hist_bytes = n * 4 + E * 4
     route_bytes = n * 4 + n * 8 + n * 4 + E * 20
+    # what the machine does with the plainest kernels at this size: a fill of the 12 B/id that route writes, and a copy
+    # that moves as many bytes as route (half in, half out), each replayed from a graph like the calls above
+    outs = [torch.empty(n * 12, dtype=torch.uint8, device="cuda") for _ in range(nbuf)]
+    halves = [torch.empty(route_bytes // 2, dtype=torch.uint8, device="cuda") for _ in range(nbuf)]
+
+    def ref_graph_ms(fn, reps=20):
+        fn(0)
+        torch.cuda.synchronize()
+        g_ = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g_):
+            for i in range(nbuf):
+                fn(i)
+        return _time_gpu(g_.replay, reps, warmup=3) / nbuf
+
+    fill_ms = ref_graph_ms(lambda i: outs[i].view(torch.int32).fill_(1))
+    copy_ms = ref_graph_ms(lambda i: halves[i].copy_(halves[(i + 1) % nbuf]))
+    read_ms = ref_graph_ms(lambda i: halves[0][:64].copy_(bufs[i].view(torch.uint8)[:64]))  # launch floor of one kernel
+    del outs, halves
     t1 = time.perf_counter()
     reps = 3
     for _ in range(reps):
@@ -412,6 +434,12 @@ def run_routing(args):
                             "frac_hbm_peak": round(route_bytes / route_graph_ms / 1e6 / PEAK_HBM_GBS, 4)},
             "continuous_count_graph": {"ms": round(hist_graph_ms, 5), "gbs": round(hist_bytes / hist_graph_ms / 1e6, 1),
                                        "frac_hbm_peak": round(hist_bytes / hist_graph_ms / 1e6 / PEAK_HBM_GBS, 4)},
+            "reference: fill of 12 B/id [torch fill_, graph]": {"ms": round(fill_ms, 5), "gbs": round(n * 12 / fill_ms / 1e6, 1),
+                                                                "frac_hbm_peak": round(n * 12 / fill_ms / 1e6 / PEAK_HBM_GBS, 4)},
+            "reference: copy moving route's bytes [torch copy_, graph]": {
+                "ms": round(copy_ms, 5), "gbs": round(route_bytes / copy_ms / 1e6, 1),
+                "frac_hbm_peak": round(route_bytes / copy_ms / 1e6 / PEAK_HBM_GBS, 4)},
+            "reference: one 64-byte copy kernel [graph]": {"ms": round(read_ms, 5)},
         },
     }
     print(json.dumps(out))

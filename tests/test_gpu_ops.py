@@ -72,6 +72,95 @@ def test_scatter2scatter(dtype, case, w_kn, x_grouped, y_grouped):
         assert nerr(out, want) <= _tol(dtype)
 
 
+def _routing_with_counts(counts, k, seed):
+    """a routing whose experts own exactly `counts` rows (sum divisible by k): the slots are dealt out at random"""
+    g = torch.Generator().manual_seed(seed)
+    E, M = len(counts), sum(counts)
+    assert M % k == 0
+    flat = torch.repeat_interleave(torch.arange(E), torch.tensor(counts))[torch.randperm(M, generator=g)]
+    sel = flat.view(M // k, k)
+    se, ss = flat.sort(stable=True)
+    offs = torch.bincount(se, minlength=E).cumsum(0)
+    assert torch.bincount(se, minlength=E).tolist() == list(counts)
+    return sel, se, ss, offs
+
+
+# rows per expert around the 32-row blocks and 256-row tiles of the kernels (an empty expert, single rows, one row more or
+# less than a block, a tile and two tiles), with K = 4 or 6 steps of 64 (complete and with a tail) and one odd step count:
+# tiles of more than 192 rows and an even number of at least four K steps fetch the next tile's operands inside their
+# last K step, all others behind it
+ROW_COUNT_CASES = [
+    # counts, k, K, N
+    ((1, 31, 33, 65, 129, 257, 0, 512), 2, 256, 264),
+    ((257, 1, 193, 192, 511, 513, 224, 3), 2, 232, 520),
+    ((300, 260, 1, 255), 1, 384, 72),
+    ((256, 200, 700, 4), 4, 328, 512),
+    ((193, 250, 256, 257), 1, 320, 264),  # five K steps: odd
+    ((3333, 259, 4000), 2, 256, 520),  # 14 and 16 row tiles: the tiles of such an expert are walked in bands of row tiles
+    ((3100, 7), 1, 64, 776),  # 13 row tiles in bands of 5, 5 and 3
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("case", ROW_COUNT_CASES)
+@pytest.mark.parametrize("w_kn", [False, True])
+def test_scatter2scatter_expert_row_counts(dtype, case, w_kn):
+    from xma.layers.moe import rocm_implementation as R
+
+    counts, k, K, N = case
+    print(f"case counts={counts} k={k} K={K} N={N} w_kn={w_kn} {dtype}", flush=True)
+    sel, se, ss, offs = _routing_with_counts(counts, k, 11)
+    E, M = len(counts), sum(counts)
+    T = M // k
+    g = torch.Generator().manual_seed(12)
+    scale = torch.rand(M, generator=g).to(dtype)
+    if w_kn:
+        W = (torch.randn(E, K, N, generator=g) * 0.1).to(dtype)
+        Wd = W.cuda()
+    else:
+        W = (torch.randn(E, N, K, generator=g) * 0.1).to(dtype).permute(0, 2, 1)
+        Wd = W.permute(0, 2, 1).contiguous().cuda().permute(0, 2, 1)
+    for x_grouped, y_grouped, rs in [(False, True, None), (True, False, scale), (True, True, None), (False, False, scale)]:
+        X = torch.randn(M if x_grouped else T, K, generator=g).to(dtype)
+        want = oracle.scatter2scatter(X, W, se, ss, k, x_grouped, y_grouped, rs)
+        out = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+        R.scatter2scatter(X.cuda(), Wd, se.cuda(), ss.cuda(), out, k, x_grouped, y_grouped, offs.cuda(),
+                          None if rs is None else rs.cuda())
+        torch.cuda.synchronize()
+        assert torch.isfinite(out).all()
+        assert nerr(out, want) <= _tol(dtype)
+        # every row against its own magnitude: a wrong row of a small expert does not hide behind the large ones
+        row_err = (out.cpu().float() - want.float()).abs().amax(dim=1) / want.float().abs().amax(dim=1).clamp_min(1e-6)
+        assert row_err.max() <= 4 * _tol(dtype), int(row_err.argmax())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("case", ROW_COUNT_CASES)
+def test_group_bwd_W_expert_row_counts(dtype, case):
+    from xma.rocm import ops
+
+    counts, k, K, N = case
+    print(f"case counts={counts} k={k} K={K} N={N} {dtype}", flush=True)
+    sel, se, ss, offs = _routing_with_counts(counts, k, 13)
+    E, M = len(counts), sum(counts)
+    T = M // k
+    g = torch.Generator().manual_seed(14)
+    x_tok = torch.randn(T, K, generator=g).to(dtype)
+    dy_grp = torch.randn(M, N, generator=g).to(dtype)
+    x_grp = torch.randn(M, K, generator=g).to(dtype)
+    for X, x_fan, want in [(x_grp, 0, oracle.group_bwd_W(dy_grp, x_grp, offs, E)),
+                           (x_tok, k, oracle.group_bwd_W(dy_grp, oracle.group(x_tok, ss, None, k), offs, E))]:
+        DW = torch.full((E, N, K), float("nan"), dtype=dtype, device="cuda").permute(0, 2, 1)
+        ops.group_bwd_W_rocm(dy_grp.cuda(), X.cuda(), ss.cuda(), offs.cuda(), DW, None, 0, x_fan)
+        torch.cuda.synchronize()
+        assert torch.isfinite(DW).all()
+        for e in range(E):  # every expert's slice against its own magnitude
+            if counts[e] == 0:
+                assert (DW[e] == 0).all()
+            else:
+                assert nerr(DW[e], want[e]) <= _tol(dtype), e
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("case", CASES)
 def test_group_bwd_W(dtype, case):
