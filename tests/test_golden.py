@@ -1,4 +1,8 @@
-"""The oracle and the host-side torch backend against the committed golden fixtures (tests/golden/*.npz)."""
+"""The oracle and the host-side torch backend against the committed golden fixtures (tests/golden/*.npz).
+
+The fixtures were written by this oracle (tests/golden/make_golden.py; the reference holds no vectors for this path), so
+they pin regressions of the oracle and of the torch backend, not parity: what pins the oracle itself is
+tests/test_oracle_routing.py and tests/test_oracle_moe.py."""
 
 import os
 
