@@ -35,18 +35,18 @@ FLAGS = [
 ]
 
 # The grouped GEMM kernels keep 256 accumulators in AGPRs next to an almost full VGPR file and hand-placed waits around
-# asynchronous inline-assembly loads: a register that the compiler spills or reloads inside the MFMA loop, behind those
-# waits, would corrupt data silently (a few spills in prologue and epilogue, where nothing asynchronous is live, are
-# harmless).  The build therefore reads the generated ISA of those kernels and fails if a scratch access sits between
-# the first and the last MFMA of one of them, and says so if the compiler is not the version the kernels were written
-# and measured with.
+# asynchronous inline-assembly loads: a register that the compiler spills inside the MFMA loop, behind those waits,
+# could be stored before its load has arrived and corrupt data silently.  The build therefore reads the generated ISA of
+# those kernels and fails if a scratch STORE sits between the first and the last MFMA of one of them (spills in front of
+# the first MFMA, where nothing asynchronous is live, are harmless, and so is reloading such a value later), and says so
+# if the compiler is not the version the kernels were written and measured with.
 LOOP_NO_SCRATCH = {"grouped_gemm.hip": re.compile(r"grouped_gemm")}
 TESTED_HIPCC = "7.2"
 USAGE_REPORT = os.path.join(HERE, "build", "kernel_resource_usage.txt")
 
 
 def _scratch_inside_mfma_loop(asm_path: str, which: re.Pattern) -> list[str]:
-    """kernels matching `which` whose ISA has a scratch access between their first and last MFMA"""
+    """kernels matching `which` whose ISA has a scratch store between their first and last MFMA"""
     bad, name, first, last, scratch = [], None, None, None, []
 
     def close():
@@ -64,7 +64,7 @@ def _scratch_inside_mfma_loop(asm_path: str, which: re.Pattern) -> list[str]:
                 if "v_mfma" in line:
                     first = n if first is None else first
                     last = n
-                elif "scratch_" in line:
+                elif "scratch_store" in line:
                     scratch.append(n)
     close()
     return bad
@@ -116,7 +116,7 @@ def _compile(src: str, verbose: bool, defines: tuple[str, ...] = (), tag: str = 
         asm = os.path.join(HERE, "build", src.replace(".hip", tag + "-hip-amdgcn-amd-amdhsa-gfx950.s"))
         bad = _scratch_inside_mfma_loop(asm, LOOP_NO_SCRATCH[src])
         if bad:
-            raise RuntimeError(f"{src}: scratch accesses inside the MFMA loop of:\n  " + "\n  ".join(bad))
+            raise RuntimeError(f"{src}: scratch stores inside the MFMA loop of:\n  " + "\n  ".join(bad))
     return obj, usage
 
 
