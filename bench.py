@@ -163,10 +163,10 @@ def _kernel_table(moe, x, rw, sel, grad, cfg, iters):
     mem("group(dy*w)", rotating(lambda i: ops.group_rocm(grads[i], ss, gdys[i], flat_w, k)),
         T * H * esz + Tk * H * esz + Tk * (8 + esz))
     # what the machine does with the plainest kernels on the same buffers: a device-to-device copy and a fill of Tk x H
-    mem("reference: copy of (Tk,H) [torch copy_]", rotating(lambda i: gdys[i].copy_(eos[i])), 2 * Tk * H * esz)
-    mem("reference: fill of (Tk,H) [torch fill_]", rotating(lambda i: gdys[i].fill_(1.0)), Tk * H * esz)
-    notes = {"hbm_kernels": f"combine, combine_bwd, group(dy*w) and the two reference lines timed on {nset} rotating buffer "
-                            f"sets ({nset * comb_bytes >> 20} MiB, more than the Infinity Cache): cold figures; the reference "
+    mem("plain copy of (Tk,H) [torch copy_]", rotating(lambda i: gdys[i].copy_(eos[i])), 2 * Tk * H * esz)
+    mem("plain fill of (Tk,H) [torch fill_]", rotating(lambda i: gdys[i].fill_(1.0)), Tk * H * esz)
+    notes = {"hbm_kernels": f"combine, combine_bwd, group(dy*w) and the two plain copy / fill lines timed on {nset} rotating buffer "
+                            f"sets ({nset * comb_bytes >> 20} MiB, more than the Infinity Cache): cold figures; the plain "
                             f"lines are stock torch kernels, the rate a plain copy / fill of the same size reaches here"}
     del eos, ys, grads, gdys
     mem("route", lambda: R.route(sel, E), Tk * 8 + Tk * 8 + Tk * 8 + E * 20)
@@ -434,12 +434,12 @@ def run_routing(args):
                             "frac_hbm_peak": round(route_bytes / route_graph_ms / 1e6 / PEAK_HBM_GBS, 4)},
             "continuous_count_graph": {"ms": round(hist_graph_ms, 5), "gbs": round(hist_bytes / hist_graph_ms / 1e6, 1),
                                        "frac_hbm_peak": round(hist_bytes / hist_graph_ms / 1e6 / PEAK_HBM_GBS, 4)},
-            "reference: fill of 12 B/id [torch fill_, graph]": {"ms": round(fill_ms, 5), "gbs": round(n * 12 / fill_ms / 1e6, 1),
+            "plain fill of 12 B/id [torch fill_, graph]": {"ms": round(fill_ms, 5), "gbs": round(n * 12 / fill_ms / 1e6, 1),
                                                                 "frac_hbm_peak": round(n * 12 / fill_ms / 1e6 / PEAK_HBM_GBS, 4)},
-            "reference: copy moving route's bytes [torch copy_, graph]": {
+            "plain copy moving route's bytes [torch copy_, graph]": {
                 "ms": round(copy_ms, 5), "gbs": round(route_bytes / copy_ms / 1e6, 1),
                 "frac_hbm_peak": round(route_bytes / copy_ms / 1e6 / PEAK_HBM_GBS, 4)},
-            "reference: one 64-byte copy kernel [graph]": {"ms": round(read_ms, 5)},
+            "one 64-byte copy kernel [graph]": {"ms": round(read_ms, 5)},
         },
     }
     print(json.dumps(out))
