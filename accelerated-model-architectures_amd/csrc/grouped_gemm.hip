@@ -178,7 +178,9 @@ __device__ __forceinline__ void load_frags(Frags &f, const FragBase<PTR> &pb, co
 // slower, although an isolated instruction-mix benchmark prefers them).  NI < 4: only the first NI of the wave's four
 // 32-wide Q blocks hold valid rows; the MFMAs and fragment reads of the others are left out.
 constexpr int MMA_GROUP = 2;
-template <typename T, int PTR, int QTR, int KK, int NI = 4, typename Hook>
+// READ_NEXT = 0: no fragment reads (the last sub-step of a tile whose hooks hold compiler-generated code: fragments read
+// ahead there would never be used, so the compiler would treat their registers as free while the reads are in flight).
+template <typename T, int PTR, int QTR, int KK, int NI = 4, int READ_NEXT = 1, typename Hook>
 __device__ __forceinline__ void mma_step(Frags &cur, Frags &nxt, const FragBase<PTR> &pb, const FragBase<QTR> &qb,
                                          f32x16 (&acc)[4][4], Hook hook) {
     wait_frags(cur); // issued at least 8 MFMAs ago
@@ -193,7 +195,7 @@ __device__ __forceinline__ void mma_step(Frags &cur, Frags &nxt, const FragBase<
         __builtin_amdgcn_sched_barrier(0);
         // fragment reads: 8 (4 P, 4 Q) over the first SLOTS / 2 slots
         constexpr int RPS = 16 / SLOTS; // reads per slot of the first half
-        if constexpr (t < SLOTS / 2) {
+        if constexpr (t < SLOTS / 2 && READ_NEXT != 0) {
             static_for<RPS>([&](auto R) {
                 constexpr int r = t * RPS + R.value, f = r >> 1;
                 if constexpr ((r & 1) == 0) {
@@ -1203,7 +1205,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
                     asm volatile("s_waitcnt vmcnt(16) lgkmcnt(0)\n\ts_barrier" ::: "memory"); // all but the 16 youngest
                 flip_stage(pb);
                 flip_stage(qb);
-                mma_step<T, WT, 0, 0, NI>(f1, f0, pb, qb, acc, [&](auto G) {
+                mma_step<T, WT, 0, 0, NI, (mode == 2 ? 0 : 1)>(f1, f0, pb, qb, acc, [&](auto G) {
                     if constexpr (mode != 2) {
                         if constexpr (G.value < DMA_N0) issue_piece(kt_b, G, FULL);
                         if constexpr (G.value + 8 < DMA_N0) issue_piece(kt_b, IC<G.value + 8>{}, FULL);
@@ -1232,8 +1234,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
         else
             main_loop(IC<0>{});
         if (ovl) {
-            // The waves met at the last step's barrier with their reads of stage 1 done; only the read-ahead of the last
-            // sub-step is in flight, into registers nobody uses, and the next tile's first K step, into stage 0.
+            // The waves met at the last step's barrier with their reads of stage 1 done (the last sub-step reads no
+            // fragments ahead); only the next tile's first K step is in flight, into stage 0.
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
         } else {
             // every load has landed (the index loads above as well), no wave touches the operand tiles any more
