@@ -189,7 +189,9 @@ __device__ __forceinline__ void mma_step(Frags &cur, Frags &nxt, const FragBase<
         constexpr int t = S.value;
         __builtin_amdgcn_sched_barrier(0);
         static_for<MMA_GROUP>([&](auto M) {
-            constexpr int m = t * MMA_GROUP + M.value, j = m >> 2, i = m & 3;
+            // the 4 x 4 blocks in boustrophedon order: consecutive MFMAs differ in one operand only (measured 0 - 1 % faster
+            // than row by row on the six GEMMs of the Mixtral-shaped layer; the sums are the same)
+            constexpr int m = t * MMA_GROUP + M.value, j = m >> 2, i = (j & 1) ? 3 - (m & 3) : (m & 3);
             if constexpr (i < NI) acc[j][i] = Elem<T>::mfma(cur.p[j], cur.q[i], acc[j][i]);
         });
         __builtin_amdgcn_sched_barrier(0);
