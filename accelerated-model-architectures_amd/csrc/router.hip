@@ -52,32 +52,43 @@ template <> struct Scalar<XMA_ROCM_F32> {
     static __device__ __forceinline__ void store(void *p, int64_t i, float v) { ((float *)p)[i] = v; }
 };
 
-// Exchange with the lane whose group-local index differs in bit log2(M) (or, for 4 and 8, with the mirrored lane of
-// the 8- or 16-lane block, which lies in the other half just the same): cross-lane moves inside a row of 16 lanes
-// are DPP operands of the VALU, 16 is an LDS-crossbar swizzle, only 32 needs a general permute.
-template <int M> __device__ __forceinline__ uint32_t lane_exchange(uint32_t v) {
+// A lane's own value and that of the lane whose index differs in bit log2(M) (for 4 and 8: of the mirrored lane of the
+// 8- or 16-lane block, which lies in the other half just the same), as an unordered pair - which of the two members is
+// the lane's own differs from lane to lane, so only commutative use is meant.  Inside a row of 16 lanes the partner is a
+// DPP operand of the consuming VALU instruction; rows are exchanged by v_permlane16_swap / v_permlane32_swap, which swap
+// the odd rows (the upper half) of one register with the even rows (the lower half) of another.  No LDS round trip.
+struct LanePair {
+    uint32_t a, b;
+};
+template <int M> __device__ __forceinline__ LanePair pair_exchange(uint32_t v) {
     const int x = (int)v;
-    if constexpr (M == 1) return (uint32_t)__builtin_amdgcn_update_dpp(x, x, 0xB1, 0xf, 0xf, false);  // quad_perm 1,0,3,2
-    if constexpr (M == 2) return (uint32_t)__builtin_amdgcn_update_dpp(x, x, 0x4E, 0xf, 0xf, false);  // quad_perm 2,3,0,1
-    if constexpr (M == 4) return (uint32_t)__builtin_amdgcn_update_dpp(x, x, 0x141, 0xf, 0xf, false); // row_half_mirror
-    if constexpr (M == 8) return (uint32_t)__builtin_amdgcn_update_dpp(x, x, 0x140, 0xf, 0xf, false); // row_mirror
-    if constexpr (M == 16) return (uint32_t)__builtin_amdgcn_ds_swizzle(x, 0x401F);                   // lane ^ 16
-    return (uint32_t)__shfl_xor(x, 32);
-}
-template <int M> __device__ __forceinline__ float lane_exchange(float v) {
-    return __builtin_bit_cast(float, lane_exchange<M>(__builtin_bit_cast(uint32_t, v)));
+    if constexpr (M == 1) return {v, (uint32_t)__builtin_amdgcn_mov_dpp(x, 0xB1, 0xf, 0xf, true)};  // quad_perm 1,0,3,2
+    if constexpr (M == 2) return {v, (uint32_t)__builtin_amdgcn_mov_dpp(x, 0x4E, 0xf, 0xf, true)};  // quad_perm 2,3,0,1
+    if constexpr (M == 4) return {v, (uint32_t)__builtin_amdgcn_mov_dpp(x, 0x141, 0xf, 0xf, true)}; // row_half_mirror
+    if constexpr (M == 8) return {v, (uint32_t)__builtin_amdgcn_mov_dpp(x, 0x140, 0xf, 0xf, true)}; // row_mirror
+    if constexpr (M == 16) {
+        const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+        return {r[0], r[1]};
+    }
+    if constexpr (M == 32) {
+        const auto r = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+        return {r[0], r[1]};
+    }
 }
 
 // all-reduce over the G lanes of a group; op(a, b) must be commutative and associative
-template <int G, int M = 1, typename V, typename Op> __device__ __forceinline__ V group_reduce(V v, Op op) {
+template <int G, int M = 1, typename Op> __device__ __forceinline__ uint32_t group_reduce(uint32_t v, Op op) {
     if constexpr (M < G) {
-        v = op(v, lane_exchange<M>(v));
-        return group_reduce<G, M * 2>(v, op);
+        const LanePair p = pair_exchange<M>(v);
+        return group_reduce<G, M * 2>(op(p.a, p.b), op);
     } else
         return v;
 }
 template <int G> __device__ __forceinline__ float group_sum(float v) {
-    return group_reduce<G>(v, [](float a, float b) { return a + b; });
+    const uint32_t r = group_reduce<G>(__builtin_bit_cast(uint32_t, v), [](uint32_t a, uint32_t b) {
+        return __builtin_bit_cast(uint32_t, __builtin_bit_cast(float, a) + __builtin_bit_cast(float, b));
+    });
+    return __builtin_bit_cast(float, r);
 }
 
 // softmax over the values held by lanes 0..k-1 of a group; lane 0 holds the largest (NaN propagates like in torch)
@@ -128,8 +139,9 @@ template <> struct Cand<XMA_ROCM_F32> {
     __device__ __forceinline__ float value() const { return key_value(key); }
     template <int G, int M = 1> __device__ __forceinline__ Cand group_best() const {
         if constexpr (M < G) {
-            const Cand o = {lane_exchange<M>(key), (int)lane_exchange<M>((uint32_t)idx)};
-            const Cand w = o.beats(*this) ? o : *this;
+            const LanePair pk = pair_exchange<M>(key), pi = pair_exchange<M>((uint32_t)idx);
+            const Cand a = {pk.a, (int)pi.a}, b = {pk.b, (int)pi.b};
+            const Cand w = b.beats(a) ? b : a;
             return w.template group_best<G, M * 2>();
         } else
             return *this;
@@ -231,6 +243,71 @@ __global__ __launch_bounds__(RT_THREADS) void router_topk_bwd_kernel(const void 
 // The four partial results meet in LDS; wave w then owns 8 of the 32 tokens: their logits sit across the 32 lanes of a
 // half-wave, NB per lane, exactly the layout the selection network of router_topk_kernel works on (G = 32).
 // ------------------------------------------------------------------------------------------------
+// S accumulator slots of the gate product at once: in a slot the lanes of a half-wave hold one token's logits, lane r
+// the experts 32 b + r (sum_of(s, b) = fp32 sum of block b of slot s; token_of(s) = the token of this lane's half).
+// Rounds them to the activation dtype, stores them, selects the k largest (lowest index among equals), and stores
+// fp32-softmax weights and expert ids.  A round of the selection is a chain of dependent cross-lane exchanges; the S
+// slots are S independent chains for the scheduler to interleave.
+template <typename T, int DT, int NB, int S, typename TokenOf, typename SumOf>
+__device__ __forceinline__ void gate_finish_slots(int64_t n_tokens, int r, int lane, int E, int k, TokenOf token_of,
+                                                  SumOf sum_of, uint16_t *__restrict__ logits, int64_t ldl,
+                                                  void *__restrict__ weights, void *__restrict__ ids, int ids_i64) {
+    const int g = r;
+    int64_t t[S];
+    bool live[S];
+    Cand<DT> c[S][NB], mine[S];
+    // all sums are read before anything is decided on them: the empty asm statements keep the compiler from sinking
+    // each read into the predicated region of its store, where every one of them would be waited for on its own
+    float sum[S][NB];
+#pragma unroll
+    for (int s = 0; s < S; ++s)
+#pragma unroll
+        for (int b = 0; b < NB; ++b) sum[s][b] = sum_of(s, b);
+#pragma unroll
+    for (int s = 0; s < S; ++s)
+#pragma unroll
+        for (int b = 0; b < NB; ++b) asm volatile("" : "+v"(sum[s][b]));
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        t[s] = token_of(s);
+        live[s] = t[s] < n_tokens;
+        mine[s] = Cand<DT>::none();
+#pragma unroll
+        for (int b = 0; b < NB; ++b) {
+            const uint32_t bits = Elem<T>::pack(sum[s][b], 0.f) & 0xffffu;
+            const int e = b * 32 + r;
+            if (live[s] && e < E) logits[t[s] * ldl + e] = (uint16_t)bits;
+            c[s][b] = (live[s] && e < E) ? Cand<DT>::from_bits(bits, e) : Cand<DT>::none();
+        }
+    }
+    for (int round = 0; round < k; ++round) {
+#pragma unroll
+        for (int s = 0; s < S; ++s) {
+            Cand<DT> best = c[s][0];
+#pragma unroll
+            for (int b = 1; b < NB; ++b)
+                if (c[s][b].beats(best)) best = c[s][b];
+            best = best.template group_best<32>();
+            const int be = best.index();
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+                if (b * 32 + r == be && !best.is_none()) c[s][b] = Cand<DT>::none(); // taken
+            if (g == round) mine[s] = best;
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < S; ++s) {
+        const float w = group_softmax<32>(mine[s].value(), g, k, lane - g);
+        if (live[s] && g < k) {
+            Scalar<DT>::store(weights, t[s] * k + g, w);
+            if (ids_i64)
+                ((int64_t *)ids)[t[s] * k + g] = mine[s].index();
+            else
+                ((int32_t *)ids)[t[s] * k + g] = mine[s].index();
+        }
+    }
+}
+
 constexpr int RG_THREADS = 256, RG_TOKENS = 32, RG_MAX_E = 128, RG_MAX_K = 32;
 
 template <typename T, int DT, int NB>
@@ -241,7 +318,8 @@ __global__ __launch_bounds__(RG_THREADS) void router_gate_topk_kernel(const uint
                                                                       void *__restrict__ weights, void *__restrict__ ids,
                                                                       int ids_i64) {
     __shared__ float s_part[4][16 * NB][64];
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6); // a scalar: K ranges and their branches are uniform
     const int r = lane & 31, half = lane >> 5;
     const int64_t t0 = (int64_t)blockIdx.x * RG_TOKENS;
     const int64_t my_t = (t0 + r < n_tokens) ? t0 + r : n_tokens - 1; // clamped: rows past the end are never stored
@@ -249,26 +327,38 @@ __global__ __launch_bounds__(RG_THREADS) void router_gate_topk_kernel(const uint
     const int s_begin = wave * steps / 4, s_end = (wave + 1) * steps / 4;
     const uint16_t *xrow = x + my_t * ldx + half * 32;
     const uint16_t *wrow[NB];
-    bool w_ok[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
-        const int e = b * 32 + r;
-        w_ok[b] = e < E;
-        wrow[b] = wg + (int64_t)(w_ok[b] ? e : E - 1) * ldw + half * 32;
+        const int e = b * 32 + r; // lanes past E read row E - 1: their accumulator columns are never looked at
+        wrow[b] = wg + (int64_t)(e < E ? e : E - 1) * ldw + half * 32;
     }
     struct Stage {
         u32x4 xa[4];
         u32x4 wb[NB][4];
     };
     const u32x4 zero4 = {0u, 0u, 0u, 0u};
+    // Steps inside H are plain loads, nothing selected and no branch per lane, so the compiler can count the loads in
+    // flight and wait only for the stage it multiplies.  The last step of an H that is no multiple of 64 runs apart
+    // from the loop: it reads each 16-byte chunk only where it lies inside the row (H is a multiple of 8) and takes
+    // zeros elsewhere.
+    const int steps_full = H / 64;
     auto fetch = [&](Stage &st, int step) {
         const int k0 = step * 64;
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const bool in = k0 + half * 32 + 8 * q < H; // H is a multiple of 8: a 16-byte chunk is inside or outside
+            st.xa[q] = *(const u32x4 *)(xrow + k0 + 8 * q);
+#pragma unroll
+            for (int b = 0; b < NB; ++b) st.wb[b][q] = *(const u32x4 *)(wrow[b] + k0 + 8 * q);
+        }
+    };
+    auto fetch_partial = [&](Stage &st, int step) {
+        const int k0 = step * 64;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const bool in = k0 + half * 32 + 8 * q < H;
             st.xa[q] = in ? *(const u32x4 *)(xrow + k0 + 8 * q) : zero4;
 #pragma unroll
-            for (int b = 0; b < NB; ++b) st.wb[b][q] = (in && w_ok[b]) ? *(const u32x4 *)(wrow[b] + k0 + 8 * q) : zero4;
+            for (int b = 0; b < NB; ++b) st.wb[b][q] = in ? *(const u32x4 *)(wrow[b] + k0 + 8 * q) : zero4;
         }
     };
     f32x16 acc[NB];
@@ -284,14 +374,19 @@ __global__ __launch_bounds__(RG_THREADS) void router_gate_topk_kernel(const uint
     };
     // two stages of operands in registers: the loads of step s + 1 are in flight while step s multiplies
     Stage s0, s1;
-    if (s_begin < s_end) fetch(s0, s_begin);
-    for (int step = s_begin; step < s_end; step += 2) {
-        if (step + 1 < s_end) fetch(s1, step + 1);
+    const int f_end = s_end < steps_full ? s_end : steps_full;
+    if (s_begin < f_end) fetch(s0, s_begin);
+    for (int step = s_begin; step < f_end; step += 2) {
+        if (step + 1 < f_end) fetch(s1, step + 1);
         multiply(s0);
-        if (step + 1 < s_end) {
-            if (step + 2 < s_end) fetch(s0, step + 2);
+        if (step + 1 < f_end) {
+            if (step + 2 < f_end) fetch(s0, step + 2);
             multiply(s1);
         }
+    }
+    if (s_end > steps_full) { // the last wave, when H is no multiple of 64
+        fetch_partial(s0, steps_full);
+        multiply(s0);
     }
 #pragma unroll
     for (int b = 0; b < NB; ++b)
@@ -301,62 +396,186 @@ __global__ __launch_bounds__(RG_THREADS) void router_gate_topk_kernel(const uint
 
     // wave w finishes accumulator slots v = 4 w .. 4 w + 3: in slot v the lanes of half h hold token
     // 8 (v / 4) + 4 h + v % 4 of the tile, lane r of the half the experts 32 b + r
-    const int g = r;
-    for (int vv = 0; vv < 4; ++vv) {
-        const int v = 4 * wave + vv;
-        const int64_t t = t0 + 8 * (v >> 2) + 4 * half + (v & 3);
-        const bool live = t < n_tokens;
-        Cand<DT> c[NB];
+    gate_finish_slots<T, DT, NB, 4>(
+        n_tokens, r, lane, E, k, [&](int s) { return t0 + 8 * wave + 4 * half + s; },
+        [&](int s, int b) {
+            const int v = 4 * wave + s;
+            return (s_part[0][b * 16 + v][lane] + s_part[1][b * 16 + v][lane]) +
+                   (s_part[2][b * 16 + v][lane] + s_part[3][b * 16 + v][lane]);
+        },
+        logits, ldl, weights, ids, ids_i64);
+}
+
+// The same product for layers of more than 32 experts, where Wg no longer is a small operand: every lane fetching its
+// own expert row per K step (32 rows of 64 bytes per load instruction, NB times per step) makes the texture path, not
+// HBM, the limit.  Here a workgroup takes 64 tokens, two waves of 32, and each K step's slice of Wg (32 NB rows x 64 k)
+// is loaded once for both with coalesced 16-byte loads (8 lanes per row), kept in LDS in two stages and read from there
+// as MFMA operands; a row of the slice takes 144 bytes of LDS, so the 16 lanes of a ds_read_b128 phase fall into 16
+// different 4-bank groups.  x still comes straight from global memory, 64 contiguous bytes per lane and step, DEPTH
+// steps ahead in registers.  With KS = 2 the workgroup has a second pair of waves that takes the other half of the K
+// range (with its own slices), which puts a wave on every SIMD when the layer has too few tokens for that otherwise.
+// The accumulators pass through LDS; the pairs share out the 16 accumulator slots for the selection, which adds the
+// KS partial sums as it reads them.
+constexpr int RL_TOKENS = 64, RL_ROW = 72;
+constexpr int64_t RL_SPLIT_K_BELOW = 24576; // tokens: fewer leave SIMDs of a 256-CU device idle at one wave per 32 tokens
+
+template <int NB, int KS> constexpr int rl_lds_bytes() { return 2 * KS * NB * 32 * RL_ROW * 2; }
+
+template <typename T, int DT, int NB, int KS>
+__global__ __launch_bounds__(128 * KS) void router_gate_topk_lds_kernel(const uint16_t *__restrict__ x, int64_t ldx,
+                                                                        const uint16_t *__restrict__ wg, int64_t ldw,
+                                                                        int64_t n_tokens, int H, int E, int k,
+                                                                        uint16_t *__restrict__ logits, int64_t ldl,
+                                                                        void *__restrict__ weights, void *__restrict__ ids,
+                                                                        int ids_i64) {
+    constexpr int SLICE = NB * 32 * RL_ROW;      // halfwords of one slice
+    constexpr int DEPTH = NB <= 2 ? 8 : 4;       // steps of x in flight: what fits beside the accumulators at 2 waves per SIMD
+    constexpr int W_CHUNKS = NB * 32 * 8 / 128;  // 16-byte chunks of a slice per thread of the pair that loads it
+    static_assert(rl_lds_bytes<NB, KS>() >= 2 * KS * NB * 16 * 64 * 4, "the accumulators pass through the operand stages");
+    extern __shared__ __attribute__((aligned(16))) uint16_t s_w[]; // [2 stages][KS][SLICE]
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int tb = wave & 1, kh = wave >> 1, ptid = tid & 127; // token block, K range, thread of the pair
+    const int r = lane & 31, half = lane >> 5;
+    const int64_t t0 = (int64_t)blockIdx.x * RL_TOKENS + tb * 32;
+    const int64_t my_t = (t0 + r < n_tokens) ? t0 + r : n_tokens - 1; // clamped: rows past the end are never stored
+    const uint16_t *xrow = x + my_t * ldx + half * 32;
+    const u32x4 zero4 = {0u, 0u, 0u, 0u};
+
+    f32x16 acc[NB];
 #pragma unroll
-        for (int b = 0; b < NB; ++b) {
-            const float sum = (s_part[0][b * 16 + v][lane] + s_part[1][b * 16 + v][lane]) +
-                              (s_part[2][b * 16 + v][lane] + s_part[3][b * 16 + v][lane]);
-            const uint32_t bits = Elem<T>::pack(sum, 0.f) & 0xffffu;
-            const int e = b * 32 + r;
-            if (live && e < E) logits[t * ldl + e] = (uint16_t)bits;
-            c[b] = (live && e < E) ? Cand<DT>::from_bits(bits, e) : Cand<DT>::none();
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[b][v] = 0.f;
+
+    // Steps inside H are plain loads (nothing selected, no branch per lane: the compiler counts the loads in flight
+    // and waits only for what a step uses); loads for steps past the pair's last one re-read step 0 and are never
+    // used.  Rows of the slice past E re-read row E - 1: their accumulator columns are never looked at.
+    const int steps_full = H / 64, per = (steps_full + KS - 1) / KS; // every pair runs `per` rounds of barriers
+    const int s_lo = kh * per, my_steps = steps_full - s_lo < per ? (steps_full - s_lo > 0 ? steps_full - s_lo : 0) : per;
+    auto fetch_x = [&](u32x4(&d)[4], int i) {
+        const int k0 = (i < my_steps ? s_lo + i : 0) * 64;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) d[q] = *(const u32x4 *)(xrow + k0 + 8 * q);
+    };
+    // chunk c of a slice: expert row c / 8, k offset 8 (c % 8)
+    auto fetch_w = [&](u32x4(&d)[W_CHUNKS], int i) {
+        const int k0 = (s_lo + i) * 64;
+#pragma unroll
+        for (int j = 0; j < W_CHUNKS; ++j) {
+            const int c = ptid + 128 * j, e = c >> 3;
+            d[j] = *(const u32x4 *)(wg + (int64_t)(e < E ? e : E - 1) * ldw + k0 + 8 * (c & 7));
         }
-        Cand<DT> mine = Cand<DT>::none();
-        for (int round = 0; round < k; ++round) {
-            Cand<DT> best = c[0];
+    };
+    auto store_w = [&](const u32x4(&d)[W_CHUNKS], int buf) {
 #pragma unroll
-            for (int b = 1; b < NB; ++b)
-                if (c[b].beats(best)) best = c[b];
-            best = best.template group_best<32>();
-            const int be = best.index();
-#pragma unroll
-            for (int b = 0; b < NB; ++b)
-                if (b * 32 + r == be && !best.is_none()) c[b] = Cand<DT>::none(); // taken
-            if (g == round) mine = best;
+        for (int j = 0; j < W_CHUNKS; ++j) {
+            const int c = ptid + 128 * j;
+            *(u32x4 *)(s_w + (buf * KS + kh) * SLICE + (c >> 3) * RL_ROW + 8 * (c & 7)) = d[j];
         }
-        const float w = group_softmax<32>(mine.value(), g, k, lane - g);
-        if (live && g < k) {
-            Scalar<DT>::store(weights, t * k + g, w);
-            if (ids_i64)
-                ((int64_t *)ids)[t * k + g] = mine.index();
-            else
-                ((int32_t *)ids)[t * k + g] = mine.index();
+    };
+    auto multiply = [&](const u32x4(&xa)[4], int buf) {
+        const uint16_t *ws = s_w + (buf * KS + kh) * SLICE + r * RL_ROW + half * 32;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                const u32x4 wb = *(const u32x4 *)(ws + b * 32 * RL_ROW + 8 * q);
+                acc[b] = Elem<T>::mfma(xa[q], wb, acc[b]);
+            }
+    };
+
+    u32x4 xs[DEPTH][4];
+    u32x4 wr[W_CHUNKS];
+    if (steps_full > 0) {
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) fetch_x(xs[d], d);
+        if (my_steps > 0) {
+            fetch_w(wr, 0);
+            store_w(wr, 0);
         }
     }
+    __syncthreads();
+    for (int base = 0; base < per; base += DEPTH) {
+#pragma unroll
+        for (int u = 0; u < DEPTH; ++u) {
+            const int i = base + u;
+            if (i < per) { // uniform over the workgroup; what follows is uniform over the pair
+                const bool more = i + 1 < my_steps;
+                if (more) fetch_w(wr, i + 1);
+                if (i < my_steps) multiply(xs[u], u & 1);
+                fetch_x(xs[u], i + DEPTH);
+                if (more) store_w(wr, (u + 1) & 1);
+                __syncthreads();
+            }
+        }
+    }
+    if (steps_full * 64 < H) {
+        // the last, partial step of an H that is no multiple of 64, taken by the first pair: a 16-byte chunk lies
+        // inside the row or outside (H is a multiple of 8); the chunks outside are zeros in both operands
+        const int k0 = steps_full * 64, buf = per & 1; // this stage was last read before the previous barrier
+        u32x4 xa[4];
+        if (kh == 0) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+                xa[q] = (k0 + half * 32 + 8 * q < H) ? *(const u32x4 *)(xrow + k0 + 8 * q) : zero4;
+#pragma unroll
+            for (int j = 0; j < W_CHUNKS; ++j) {
+                const int c = ptid + 128 * j, e = c >> 3, kk = k0 + 8 * (c & 7);
+                wr[j] = (kk < H) ? *(const u32x4 *)(wg + (int64_t)(e < E ? e : E - 1) * ldw + kk) : zero4;
+            }
+            store_w(wr, buf);
+        }
+        __syncthreads();
+        if (kh == 0) multiply(xa, buf);
+        __syncthreads();
+    }
+    // after the last barrier nobody reads the operand stages any more
+    float *s_acc = (float *)s_w;
+#pragma unroll
+    for (int b = 0; b < NB; ++b)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) s_acc[(wave * NB * 16 + b * 16 + v) * 64 + lane] = acc[b][v];
+    if constexpr (KS > 1) __syncthreads(); // with one pair every lane reads back only what it wrote itself
+    for (int v0 = kh * (16 / KS); v0 < (kh + 1) * (16 / KS); v0 += 4)
+        gate_finish_slots<T, DT, NB, 4>(
+            n_tokens, r, lane, E, k, [&](int s) { return t0 + 2 * v0 + 4 * half + s; },
+            [&](int s, int b) {
+                float sum = s_acc[(tb * NB * 16 + b * 16 + v0 + s) * 64 + lane];
+#pragma unroll
+                for (int h = 1; h < KS; ++h) sum += s_acc[((2 * h + tb) * NB * 16 + b * 16 + v0 + s) * 64 + lane];
+                return sum;
+            },
+            logits, ldl, weights, ids, ids_i64);
 }
 
 template <typename T, int DT>
 int router_gate_launch(const void *x, int64_t ldx, const void *wg, int64_t ldw, int64_t n_tokens, int H, int E, int k,
                        void *logits, int64_t ldl, void *weights, void *ids, int ids_i64, hipStream_t st) {
-    const unsigned grid = (unsigned)((n_tokens + RG_TOKENS - 1) / RG_TOKENS);
-#define RG_LAUNCH(NB)                                                                                                   \
-    router_gate_topk_kernel<T, DT, NB><<<grid, RG_THREADS, 0, st>>>((const uint16_t *)x, ldx, (const uint16_t *)wg, ldw, \
-                                                                    n_tokens, H, E, k, (uint16_t *)logits, ldl, weights, \
-                                                                    ids, ids_i64)
+#define RG_ARGS                                                                                                    \
+    (const uint16_t *)x, ldx, (const uint16_t *)wg, ldw, n_tokens, H, E, k, (uint16_t *)logits, ldl, weights, ids, ids_i64
+#define RL_LAUNCH(NB, KS)                                                                                          \
+    {                                                                                                              \
+        auto kernel = router_gate_topk_lds_kernel<T, DT, NB, KS>;                                                  \
+        if (int rc = xma_set_max_lds_once((const void *)kernel, rl_lds_bytes<NB, KS>())) return rc;                \
+        kernel<<<(unsigned)((n_tokens + RL_TOKENS - 1) / RL_TOKENS), 128 * KS, rl_lds_bytes<NB, KS>(), st>>>(RG_ARGS); \
+    }
+#define RL_LAUNCH_NB(NB)          \
+    if (split_k)                  \
+        RL_LAUNCH(NB, 2)          \
+    else                          \
+        RL_LAUNCH(NB, 1)
+    const bool split_k = n_tokens < RL_SPLIT_K_BELOW;
     if (E <= 32)
-        RG_LAUNCH(1);
+        router_gate_topk_kernel<T, DT, 1><<<(unsigned)((n_tokens + RG_TOKENS - 1) / RG_TOKENS), RG_THREADS, 0, st>>>(RG_ARGS);
     else if (E <= 64)
-        RG_LAUNCH(2);
+        RL_LAUNCH_NB(2)
     else if (E <= 96)
-        RG_LAUNCH(3);
+        RL_LAUNCH_NB(3)
     else
-        RG_LAUNCH(4);
-#undef RG_LAUNCH
+        RL_LAUNCH_NB(4)
+#undef RL_LAUNCH_NB
+#undef RL_LAUNCH
+#undef RG_ARGS
     return xma_check_launch("router_gate_topk_kernel");
 }
 

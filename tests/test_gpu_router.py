@@ -153,6 +153,10 @@ GATE_CASES = [  # T, H, E, k
     (100, 200, 100, 32),
     (65, 8, 33, 5),
     (8192, 4096, 8, 2),
+    (4133, 1032, 96, 4),
+    (2085, 2048, 128, 8),
+    (24613, 136, 40, 3),  # enough tokens for the variant without a K split
+    (24577, 64, 128, 8),
 ]
 
 
