@@ -117,6 +117,7 @@ template <int DT> struct Cand {
         return {(key << 16) | (0xffffu - (uint32_t)e)};
     }
     __device__ __forceinline__ bool beats(const Cand &o) const { return packed > o.packed; }
+    __device__ __forceinline__ bool same(const Cand &o) const { return packed == o.packed; } // value and index
     __device__ __forceinline__ bool is_none() const { return packed == 0u; }
     __device__ __forceinline__ int index() const { return (int)(0xffffu - (packed & 0xffffu)); }
     __device__ __forceinline__ float value() const {
@@ -134,6 +135,7 @@ template <> struct Cand<XMA_ROCM_F32> {
     static __device__ __forceinline__ Cand none() { return {0u, 0x7fffffff}; }
     static __device__ __forceinline__ Cand make(const void *row, int e) { return {order_key(((const float *)row)[e]), e}; }
     __device__ __forceinline__ bool beats(const Cand &o) const { return key > o.key || (key == o.key && idx < o.idx); }
+    __device__ __forceinline__ bool same(const Cand &o) const { return key == o.key && idx == o.idx; }
     __device__ __forceinline__ bool is_none() const { return key == 0u; }
     __device__ __forceinline__ int index() const { return idx; }
     __device__ __forceinline__ float value() const { return key_value(key); }
@@ -171,10 +173,9 @@ __global__ __launch_bounds__(RT_THREADS) void router_topk_kernel(const void *__r
         for (int v = 1; v < VPL; ++v)
             if (c[v].beats(best)) best = c[v];
         best = best.template group_best<G>();
-        const int be = best.index();
 #pragma unroll
         for (int v = 0; v < VPL; ++v)
-            if (g + v * G == be && !best.is_none()) c[v] = Cand<DT>::none(); // taken
+            if (c[v].same(best)) c[v] = Cand<DT>::none(); // taken (an index occurs once: at most one lane and slot matches)
         if (g == r) mine = best;
     }
     const float w = group_softmax<G>(mine.value(), g, k, lane - g);
@@ -288,10 +289,9 @@ __device__ __forceinline__ void gate_finish_slots(int64_t n_tokens, int r, int l
             for (int b = 1; b < NB; ++b)
                 if (c[s][b].beats(best)) best = c[s][b];
             best = best.template group_best<32>();
-            const int be = best.index();
 #pragma unroll
             for (int b = 0; b < NB; ++b)
-                if (b * 32 + r == be && !best.is_none()) c[s][b] = Cand<DT>::none(); // taken
+                if (c[s][b].same(best)) c[s][b] = Cand<DT>::none(); // taken (an index occurs once: at most one match)
             if (g == round) mine[s] = best;
         }
     }
