@@ -1,6 +1,6 @@
 """MoE hot-path benchmark on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c5|c2|copy|mfma_peak]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c5|c2|copy|mfma_peak|library_gemm]
 
 Default workload: the Mixtral-shaped layer (T=8192, H=4096, I=14336, E=8, top-2, packed SwiGLU, bf16).
 A step is one forward + backward of the layer behind the gate: router (top-k + softmax + expert ids from the
@@ -486,12 +486,49 @@ def run_mfma_peak(args):
                       "results": res}))
 
 
+def run_library_gemm(args):
+    """For comparison, not part of the product path: the stock dense bf16 GEMM of this PyTorch build (hipBLASLt) on the
+    dense equivalents of the C3 GEMMs - every token through one expert's weights, no gather, no scatter, no activation -
+    in the three operand forms the layer uses: x @ W^T (forward), dy @ W (dX) and dy^T @ x (dW).  Same value distribution
+    as the layer's operands (activations ~ N(0, 1), weights ~ N(0, 0.02))."""
+    g = torch.Generator(device="cuda").manual_seed(0)
+
+    def rn(*shape, std=1.0):
+        return (torch.randn(*shape, device="cuda", generator=g) * std).to(torch.bfloat16)
+
+    Tk, H, I = 16384, 4096, 14336
+    res = {}
+
+    def timed(name, fn, flops):
+        ms = _time_gpu(fn, max(args.steps, 5), warmup=max(args.warmup, 2))
+        res[name] = {"ms": round(ms, 4), "tflops": round(flops / ms / 1e9, 1), "frac_mfma_peak": round(flops / ms / 1e9 / PEAK_BF16_TFLOPS, 4)}
+
+    x, w1 = rn(Tk, H), rn(2 * I, H, std=0.02)
+    timed("up-projection form: x (Tk,H) @ W1 (2I,H)^T", lambda: torch.nn.functional.linear(x, w1), 4.0 * Tk * H * I)
+    dz = rn(Tk, 2 * I)
+    timed("dX1 form: dz (Tk,2I) @ W1 (2I,H)", lambda: dz @ w1, 4.0 * Tk * H * I)
+    timed("dW1 form: dz (Tk,2I)^T @ x (Tk,H)", lambda: dz.t() @ x, 4.0 * Tk * H * I)
+    del dz, w1
+    h, w2 = rn(Tk, I), rn(H, I, std=0.02)
+    timed("down-projection form: h (Tk,I) @ W2 (H,I)^T", lambda: torch.nn.functional.linear(h, w2), 2.0 * Tk * H * I)
+    dy = rn(Tk, H)
+    timed("dX2 form: dy (Tk,H) @ W2 (H,I)", lambda: dy @ w2, 2.0 * Tk * H * I)
+    timed("dW2 form: dy (Tk,H)^T @ h (Tk,I)", lambda: dy.t() @ h, 2.0 * Tk * H * I)
+    total_ms = sum(v["ms"] for v in res.values())
+    print(json.dumps({"metric": "library_dense_gemm_tflops", "value": round(18.0 * Tk * H * I / total_ms / 1e9, 1),
+                      "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(total_ms, 4),
+                      "higher_is_better": True, "dtype": "bf16",
+                      "config": {"workload": "library_gemm: stock dense bf16 GEMMs (torch -> hipBLASLt) on the dense equivalents of "
+                                             "the six C3 GEMMs, Tk=16384 H=4096 I=14336, no routing and no epilogue work"},
+                      "results": res}))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "copy", "mfma_peak"])
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "copy", "mfma_peak", "library_gemm"])
     ap.add_argument("--zipf", action="store_true", help="c2 only: Zipf(s=1.1) ids instead of uniform")
     ap.add_argument("--kernel-iters", type=int, default=5)
     ap.add_argument("--cpu-fraction", type=int, default=1, help="CPU baseline runs on T / this many tokens")
@@ -508,6 +545,8 @@ def main():
         run_copy(args)
     elif args.workload == "mfma_peak":
         run_mfma_peak(args)
+    elif args.workload == "library_gemm":
+        run_library_gemm(args)
     elif args.workload == "c2":
         run_routing(args)
     else:
