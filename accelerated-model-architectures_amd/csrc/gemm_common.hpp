@@ -17,6 +17,8 @@ struct FwdArgs {
     int64_t ldo;
     uint16_t *aux;
     int64_t ldaux;
+    uint16_t *aux2; // SWIGLU_BWD only, may be NULL: (M, N) = swiglu_packed(z) * row_scale in grouped order
+    int64_t ldaux2;
     const uint16_t *scale;
     int64_t M;
     int N, K, E, fan_out, x_grouped, y_grouped;

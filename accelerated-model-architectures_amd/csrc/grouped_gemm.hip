@@ -568,6 +568,12 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
         };
         const int i_first = only_i >= 0 ? only_i : 0, i_last = only_i >= 0 ? only_i : 3;
         if (wq + i_first * 32 < rows_valid) load_block(i_first);
+        // HS: a second output, the activations scaled by the row scale, (M, N) in grouped order.  A lane keeps its 128
+        // values of a block packed in 32 registers until the dz rows have left, then the block takes the same way out
+        // through the staging area (32 rows of 128 columns, the layout of the plain store epilogue).  Storing each quad
+        // straight from registers instead (8 bytes per lane, 16 bytes of 32 rows per instruction, no registers held)
+        // measured no faster.
+        auto blocks = [&](auto HS) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             if (wq + i * 32 >= rows_valid) break; // wave-uniform
@@ -577,6 +583,7 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
             if (i < i_last && wq + (i + 1) * 32 < rows_valid) load_block(i + 1);
             wave_lds_sync();
             const float sc = sc_i[i];
+            u32x2 hs[HS.value ? 16 : 1];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -584,14 +591,17 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
                     u32x4 *zp = (u32x4 *)(mine + (j * 32 + g * 8) * 4);
                     const u32x4 z = *zp;
                     u32x4 o;
+                    float hv[4];
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         const float dh = acc[j][i][4 * g + q] * sc;
                         const float gg = Elem<T>::lo(z[q]), uu = Elem<T>::hi(z[q]);
                         const float sg = sigmoidf_fast(gg), silu = gg * sg;
                         o[q] = Elem<T>::pack(dh * uu * (sg + silu * (1.f - sg)), dh * silu);
+                        hv[q] = uu * silu * sc;
                     }
                     *zp = o;
+                    if constexpr (HS.value != 0) hs[j * 4 + g] = u32x2{Elem<T>::pack(hv[0], hv[1]), Elem<T>::pack(hv[2], hv[3])};
                 }
             }
             wave_lds_sync();
@@ -602,7 +612,29 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
                 if (r < rows_valid && col_ok) *(u32x4 *)(a.out + (row0 + r) * a.ldo + cz) = v;
             }
             wave_lds_sync(); // the next block overwrites the area
+            if constexpr (HS.value != 0) {
+                unsigned char *h_w = stage + lrow * EPI_Z_STRIDE + lhalf * 8;
+                const unsigned char *h_r = stage + (lane >> 4) * EPI_Z_STRIDE + (lane & 15) * 16;
+                const int ch = n0 + wp + (lane & 15) * 8; // this lane's 8 activation columns on the way out
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) *(u32x2 *)(h_w + (j * 32 + g * 8) * 2) = hs[j * 4 + g];
+                wave_lds_sync();
+#pragma unroll
+                for (int it = 0; it < 8; ++it) {
+                    const int r = wq + i * 32 + 4 * it + (lane >> 4);
+                    const u32x4 v = *(const u32x4 *)(h_r + it * 4 * EPI_Z_STRIDE);
+                    if (r < rows_valid && ch < a.N) *(u32x4 *)(a.aux2 + (row0 + r) * a.ldaux2 + ch) = v;
+                }
+                wave_lds_sync();
+            }
         }
+        };
+        if (a.aux2)
+            blocks(IC<1>{});
+        else
+            blocks(IC<0>{});
     }
 }
 
@@ -1576,12 +1608,12 @@ inline bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
 
 using namespace xma_rocm;
 
-extern "C" int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *W, int64_t w_expert_stride, int64_t ldw,
-                                        int w_is_kn, const int64_t *sorted_scattered_idxs,
-                                        const int64_t *expert_offsets, void *out, int64_t ldo, void *aux, int64_t ldaux,
-                                        const void *row_scale, int64_t M, int32_t N, int32_t K, int32_t E,
-                                        int32_t fan_out, int x_grouped, int y_grouped, int epilogue, int dtype,
-                                        void *workspace, size_t workspace_bytes, void *stream) {
+static int scatter2scatter_impl(const void *X, int64_t ldx, const void *W, int64_t w_expert_stride, int64_t ldw,
+                                int w_is_kn, const int64_t *sorted_scattered_idxs, const int64_t *expert_offsets,
+                                void *out, int64_t ldo, void *aux, int64_t ldaux, void *aux2, int64_t ldaux2,
+                                const void *row_scale, int64_t M, int32_t N, int32_t K, int32_t E, int32_t fan_out,
+                                int x_grouped, int y_grouped, int epilogue, int dtype, void *workspace,
+                                size_t workspace_bytes, void *stream) {
     XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16 || dtype == XMA_ROCM_F32, XMA_ROCM_EUNSUPPORTED,
                 "scatter2scatter: dtype %d", dtype);
     XMA_REQUIRE(epilogue >= XMA_ROCM_EPI_STORE && epilogue <= XMA_ROCM_EPI_SWIGLU_BWD, XMA_ROCM_EINVAL,
@@ -1607,6 +1639,9 @@ extern "C" int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *
         XMA_REQUIRE(out && aux && aligned16(out) && aligned16(aux) && ldaux % 8 == 0 && y_grouped, XMA_ROCM_EINVAL,
                     "scatter2scatter: SWIGLU_BWD needs out, aux (z) and y_grouped");
     }
+    XMA_REQUIRE(!aux2 || (epilogue == XMA_ROCM_EPI_SWIGLU_BWD && dtype != XMA_ROCM_F32 && aligned16(aux2) && ldaux2 % 8 == 0 &&
+                          ldaux2 >= N),
+                XMA_ROCM_EINVAL, "scatter2scatter: scaled activations go with SWIGLU_BWD in bf16 / fp16, 16-byte aligned rows");
     FwdArgs a;
     a.X = (const uint16_t *)X;
     a.ldx = ldx;
@@ -1619,6 +1654,8 @@ extern "C" int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *
     a.ldo = ldo;
     a.aux = (uint16_t *)aux;
     a.ldaux = ldaux;
+    a.aux2 = (uint16_t *)aux2;
+    a.ldaux2 = ldaux2;
     a.scale = (const uint16_t *)row_scale;
     a.M = M;
     a.N = N;
@@ -1649,6 +1686,32 @@ extern "C" int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *
     hipStream_t st = (hipStream_t)stream;
     if (dtype == XMA_ROCM_BF16) return dispatch_fwd<__bf16>(a, w_is_kn ? 1 : 0, epilogue, st);
     return dispatch_fwd<_Float16>(a, w_is_kn ? 1 : 0, epilogue, st);
+}
+
+extern "C" int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *W, int64_t w_expert_stride, int64_t ldw,
+                                        int w_is_kn, const int64_t *sorted_scattered_idxs,
+                                        const int64_t *expert_offsets, void *out, int64_t ldo, void *aux, int64_t ldaux,
+                                        const void *row_scale, int64_t M, int32_t N, int32_t K, int32_t E,
+                                        int32_t fan_out, int x_grouped, int y_grouped, int epilogue, int dtype,
+                                        void *workspace, size_t workspace_bytes, void *stream) {
+    return scatter2scatter_impl(X, ldx, W, w_expert_stride, ldw, w_is_kn, sorted_scattered_idxs, expert_offsets, out, ldo,
+                                aux, ldaux, nullptr, 0, row_scale, M, N, K, E, fan_out, x_grouped, y_grouped, epilogue,
+                                dtype, workspace, workspace_bytes, stream);
+}
+
+extern "C" int xma_rocm_down_projection_dx_swiglu(const void *dY, int64_t lddy, const void *W, int64_t w_expert_stride,
+                                                  int64_t ldw, int w_is_kn, const int64_t *sorted_scattered_idxs,
+                                                  const int64_t *expert_offsets, const void *z, int64_t ldz, void *dz,
+                                                  int64_t lddz, void *scaled_act, int64_t ld_scaled_act,
+                                                  const void *row_scale, int64_t M, int32_t N, int32_t K, int32_t E,
+                                                  int32_t fan_out, int dtype, void *workspace, size_t workspace_bytes,
+                                                  void *stream) {
+    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED,
+                "down_projection_dx_swiglu: dtype %d (bf16 and fp16 only)", dtype);
+    XMA_REQUIRE(row_scale && scaled_act, XMA_ROCM_EINVAL, "down_projection_dx_swiglu: row_scale and scaled_act are required");
+    return scatter2scatter_impl(dY, lddy, W, w_expert_stride, ldw, w_is_kn, sorted_scattered_idxs, expert_offsets, dz, lddz,
+                                const_cast<void *>(z), ldz, scaled_act, ld_scaled_act, row_scale, M, N, K, E, fan_out, 0, 1,
+                                XMA_ROCM_EPI_SWIGLU_BWD, dtype, workspace, workspace_bytes, stream);
 }
 
 #ifdef XMA_PST_TIMING

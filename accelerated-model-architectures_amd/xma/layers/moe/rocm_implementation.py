@@ -11,7 +11,9 @@ Differences from the reference's data flow, all of which remove HBM passes:
   * dW reads its gathered operand through the index instead of a materialised
     ``grouped_x`` / ``grouped_grad_out`` copy, and writes every element of dW
     (no zeros_like fill);
-  * the router-weight scaling of dy is applied in the dX2 epilogue (dW2 reads one scaled grouped copy of dy);
+  * the router-weight scaling of dy is applied in the dX2 epilogue; dW2 reads one scaled grouped copy of dy, or, from
+    four experts per token on in the fused SwiGLU path, dy through the index and activations that the dX2 epilogue
+    wrote already scaled (then h is not kept for the backward either);
   * backward reuses the un-weighted expert outputs saved by forward instead of
     recomputing them with another GEMM (triton_implementation/__init__.py:117-128);
   * combine and its backward are dedicated coalesced kernels, not bmm.
@@ -164,6 +166,15 @@ def _scaled_grouped_dy(grad_out: torch.Tensor, sorted_scattered_idxs: torch.Tens
     return out
 
 
+def _scale_activations_for_dw2(top_k: int, grad_out: torch.Tensor) -> bool:
+    """Whether the fused SwiGLU backward scales h (in the dX2 epilogue) rather than dy (with `group`) for dW2.  The scaled
+    grouped copy of dy is top_k times the size of dy and goes through HBM twice; from four experts per token on that
+    costs more than the extra output of the epilogue (measured on the whole forward + backward step, two boxes: -2.4 / -3.1 % at
+    top-8 with H = 2048, I = 768; -1.0 / -1.4 % at top-6 with I = 1408; +0.7 / +1.0 % at top-2 with H = 4096, I = 14336).  h then is not kept for
+    the backward.  16-bit only: the fp32 kernels have no such epilogue."""
+    return top_k >= 4 and grad_out.dtype in (torch.bfloat16, torch.float16)
+
+
 # ----------------------------------------------------------------------------------------- autograd
 class _UpProjectionExperts(torch.autograd.Function):
     """x (T, H) -> grouped (T*k, out); counterpart of triton_implementation/__init__.py:12-72."""
@@ -249,7 +260,10 @@ class _FusedSwiGLUExperts(torch.autograd.Function):
         router_weights = router_weights.contiguous()
         y = torch.empty(T, expert_out.size(1), device=x.device, dtype=x.dtype)
         ops.combine_rocm(expert_out, router_weights, y, top_k)
-        ctx.save_for_backward(x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets, z, h, expert_out)
+        # h is an operand of dW2 only where dW2 takes the scaled grouped copy of dy; otherwise the backward rebuilds it,
+        # scaled, from z in the dX2 epilogue and h lives until the end of this forward only
+        kept_h = h.new_empty(0) if _scale_activations_for_dw2(top_k, x) else h
+        ctx.save_for_backward(x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets, z, kept_h, expert_out)
         return y
 
     @staticmethod
@@ -263,12 +277,22 @@ class _FusedSwiGLUExperts(torch.autograd.Function):
         ops.combine_bwd_rocm(expert_out, grad_out, d_router_weights)
 
         dz = torch.empty_like(z)
-        ops.down_projection_dx_swiglu_rocm(
-            grad_out, w_proj.permute(0, 2, 1), sorted_scattered_idxs, expert_offsets, z, dz, flat_w, top_k
-        )
         d_w_proj = _empty_dw_like(w_proj)
-        ops.group_bwd_W_rocm(_scaled_grouped_dy(grad_out, sorted_scattered_idxs, flat_w, top_k), h, sorted_scattered_idxs,
-                             expert_offsets, d_w_proj, None, 0, 0)
+        if h.numel() == 0 and z.numel() != 0:  # the forward decided (_scale_activations_for_dw2) not to keep h
+            # dW2 = sum_n (w_n dy_n)^T h_n = sum_n dy_n^T (w_n h_n): the dX2 epilogue, which has z and w_n at hand, writes
+            # w_n h_n (T*k, I), and dW2 takes dy unscaled through the index - instead of a scaled, grouped copy of dy
+            # (T*k, H) written by `group` and read back by the GEMM
+            scaled_h = torch.empty(z.size(0), z.size(1) // 2, dtype=z.dtype, device=z.device)
+            ops.down_projection_dx_swiglu_scaled_act_rocm(
+                grad_out, w_proj.permute(0, 2, 1), sorted_scattered_idxs, expert_offsets, z, dz, scaled_h, flat_w, top_k
+            )
+            ops.group_bwd_W_rocm(grad_out, scaled_h, sorted_scattered_idxs, expert_offsets, d_w_proj, None, top_k, 0)
+        else:
+            ops.down_projection_dx_swiglu_rocm(
+                grad_out, w_proj.permute(0, 2, 1), sorted_scattered_idxs, expert_offsets, z, dz, flat_w, top_k
+            )
+            ops.group_bwd_W_rocm(_scaled_grouped_dy(grad_out, sorted_scattered_idxs, flat_w, top_k), h,
+                                 sorted_scattered_idxs, expert_offsets, d_w_proj, None, 0, 0)
         d_w_fc = _empty_dw_like(w_fc)
         ops.group_bwd_W_rocm(dz, x, sorted_scattered_idxs, expert_offsets, d_w_fc, None, 0, top_k)
 

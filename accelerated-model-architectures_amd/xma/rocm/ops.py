@@ -217,6 +217,42 @@ def down_projection_dx_swiglu_rocm(
                      EPI_SWIGLU_BWD, M, N, K)
 
 
+@torch.library.custom_op("xma_rocm::down_projection_dx_swiglu_scaled_act", mutates_args={"dz", "scaled_act"})
+def down_projection_dx_swiglu_scaled_act_rocm(
+    dY: torch.Tensor,
+    W: torch.Tensor,
+    sorted_scattered_idxs: torch.Tensor,
+    expert_offsets: torch.Tensor,
+    z: torch.Tensor,
+    dz: torch.Tensor,
+    scaled_act: torch.Tensor,
+    row_scale: torch.Tensor,
+    FAN_OUT: int,
+) -> None:
+    """down_projection_dx_swiglu with a second output, scaled_act[n] = swiglu_packed(z[n]) * row_scale[idx[n]] (M, N) in
+    grouped order: the X operand of dW2 = sum_n dY[idx[n] // k]^T scaled_act[n], which then needs no scaled grouped copy
+    of dY."""
+    M = sorted_scattered_idxs.numel()
+    E, K, N = W.shape
+    assert dY.size(1) == K and dY.size(0) * FAN_OUT == M
+    assert z.shape == (M, 2 * N) and dz.shape == (M, 2 * N) and scaled_act.shape == (M, N)
+    assert W.dtype == dY.dtype == z.dtype == dz.dtype == scaled_act.dtype == row_scale.dtype and row_scale.is_contiguous()
+    assert sorted_scattered_idxs.dtype == torch.int64 and sorted_scattered_idxs.is_contiguous()
+    assert expert_offsets.dtype == torch.int64 and expert_offsets.is_contiguous() and expert_offsets.numel() == E
+    w_is_kn, w_es, ldw = _weight_layout(W)
+    lib = get_library()
+    ws_bytes = scatter2scatter_workspace_bytes(M, N, K, E, dY.device.index or 0)
+    workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dY.device) if ws_bytes else None
+    check(
+        lib.xma_rocm_down_projection_dx_swiglu(
+            _ptr(dY), _rows(dY, "dY"), _ptr(W), w_es, ldw, w_is_kn, _ptr(sorted_scattered_idxs), _ptr(expert_offsets),
+            _ptr(z), _rows(z, "z"), _ptr(dz), _rows(dz, "dz"), _ptr(scaled_act), _rows(scaled_act, "scaled_act"),
+            _ptr(row_scale), M, N, K, E, FAN_OUT, _code(dY), _ptr(workspace), ws_bytes, _stream(dY),
+        ),
+        "xma_rocm_down_projection_dx_swiglu",
+    )
+
+
 @torch.library.custom_op("xma_rocm::group_bwd_W", mutates_args={"DW"})
 def group_bwd_W_rocm(
     DY: torch.Tensor,

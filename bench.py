@@ -134,11 +134,19 @@ def _kernel_table(moe, x, rw, sel, grad, cfg, iters):
     f = 2.0 * Tk * H * I
     gemm("up_swiglu(grouped_gemm NT+SwiGLU)", lambda: ops.up_projection_swiglu_rocm(x, w_fc, ss, offs, z, h, k), 2 * f)
     gemm("down(grouped_gemm NT)", lambda: ops.scatter2scatter_rocm(h, w_proj, ss, offs, eo, None, 1, True, False), f)
-    gemm("dx2_swiglu_bwd(grouped_gemm NN)",
-         lambda: ops.down_projection_dx_swiglu_rocm(grad, w_proj.permute(0, 2, 1), ss, offs, z, dz, flat_w, k), f)
     gdy = torch.empty(Tk, H, device=dev, dtype=x.dtype)
     ops.group_rocm(grad, ss, gdy, flat_w, k)
-    gemm("dw2(grouped_gemm_dw)", lambda: ops.group_bwd_W_rocm(gdy, h, ss, offs, dw_proj, None, 0, 0), f)
+    if R._scale_activations_for_dw2(k, grad):
+        # from four experts per token on the step's dX2 also writes w * h, and its dW2 reads dy through the index
+        hs = torch.empty_like(h)
+        gemm("dx2_swiglu_bwd(grouped_gemm NN, + w*h out)",
+             lambda: ops.down_projection_dx_swiglu_scaled_act_rocm(grad, w_proj.permute(0, 2, 1), ss, offs, z, dz, hs, flat_w, k), f)
+        gemm("dw2(grouped_gemm_dw, dy gathered)", lambda: ops.group_bwd_W_rocm(grad, hs, ss, offs, dw_proj, None, k, 0), f)
+        del hs
+    else:
+        gemm("dx2_swiglu_bwd(grouped_gemm NN)",
+             lambda: ops.down_projection_dx_swiglu_rocm(grad, w_proj.permute(0, 2, 1), ss, offs, z, dz, flat_w, k), f)
+        gemm("dw2(grouped_gemm_dw)", lambda: ops.group_bwd_W_rocm(gdy, h, ss, offs, dw_proj, None, 0, 0), f)
     gemm("dw1(grouped_gemm_dw)", lambda: ops.group_bwd_W_rocm(dz, x, ss, offs, dw_fc, None, 0, k), 2 * f)
     gemm("dx1(grouped_gemm NN)", lambda: ops.scatter2scatter_rocm(dz, w_fc.permute(0, 2, 1), ss, offs, eo, None, 1, True, False), 2 * f)
     esz = 2
@@ -160,7 +168,7 @@ def _kernel_table(moe, x, rw, sel, grad, cfg, iters):
 
     mem("combine", rotating(lambda i: ops.combine_rocm(eos[i], rw, ys[i], k)), comb_bytes)
     mem("combine_bwd", rotating(lambda i: ops.combine_bwd_rocm(eos[i], grads[i], d_rw)), Tk * H * esz + T * H * esz + T * k * esz)
-    mem("group(dy*w)", rotating(lambda i: ops.group_rocm(grads[i], ss, gdys[i], flat_w, k)),
+    mem("group(dy*w)" if not R._scale_activations_for_dw2(k, grad) else "group(dy*w) [not part of this step: dW2 takes w*h]", rotating(lambda i: ops.group_rocm(grads[i], ss, gdys[i], flat_w, k)),
         T * H * esz + Tk * H * esz + Tk * (8 + esz))
     # what the machine does with the plainest kernels on the same buffers: a device-to-device copy and a fill of Tk x H
     mem("plain copy of (Tk,H) [torch copy_]", rotating(lambda i: gdys[i].copy_(eos[i])), 2 * Tk * H * esz)

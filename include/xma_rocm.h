@@ -135,6 +135,24 @@ XMA_API int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *W, 
                              size_t workspace_bytes, void *stream);
 
 /*
+ * dX of the down-projection with the SwiGLU backward in the epilogue (xma_rocm_scatter2scatter with
+ * XMA_ROCM_EPI_SWIGLU_BWD, x_grouped = 0, y_grouped = 1) and one more output:
+ *     dz (M, 2N)          = swiglu_packed'(z) * ((dY[idx[n] / fan_out] * row_scale[idx[n]]) @ B_e)
+ *     scaled_act (M, N)   = swiglu_packed(z) * row_scale[idx[n]]        (grouped order)
+ * scaled_act is the X operand of the down-projection's weight gradient when dY is taken unscaled through the index:
+ * sum_n (w_n dy_n)^T h_n = sum_n dy_n^T (w_n h_n).  It replaces the scaled, grouped copy of dY that the reference
+ * builds for that GEMM (`group` with coeff, xma/layers/moe/triton_implementation/__init__.py:134-140): k times fewer
+ * bytes are written when H > N, and h need not be kept for the backward.  bf16 / fp16; row_scale and scaled_act required.
+ */
+XMA_API int xma_rocm_down_projection_dx_swiglu(const void *dY, int64_t lddy, const void *W, int64_t w_expert_stride,
+                                               int64_t ldw, int w_is_kn, const int64_t *sorted_scattered_idxs,
+                                               const int64_t *expert_offsets, const void *z, int64_t ldz, void *dz,
+                                               int64_t lddz, void *scaled_act, int64_t ld_scaled_act,
+                                               const void *row_scale, int64_t M, int32_t N, int32_t K, int32_t num_experts,
+                                               int32_t fan_out, int dtype, void *workspace, size_t workspace_bytes,
+                                               void *stream);
+
+/*
  * Weight gradient of a grouped linear: for every expert e
  *     DW[e] (N_out, K_in) = sum_{n in expert e} DY[dsrc(n), :N_out]^T  X[xsrc(n), :K_in]
  *     dsrc(n) = n if dy_grouped else sorted_scattered_idxs[n] / dy_fan_out   (then scaled by dy_scale[idx[n]] if given)

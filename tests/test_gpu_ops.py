@@ -309,6 +309,62 @@ def test_swiglu_views_and_shapes():
         assert swiglu(empty, empty, kernel_backend=KernelBackend.rocm).shape == (0, 16)
 
 
+SCALED_ACT_CASES = [
+    # counts, k, H (= K of dX2), I (= N)
+    ((1, 31, 33, 65, 129, 257, 0, 512), 2, 256, 264),
+    ((256, 200, 700, 4), 4, 328, 512),
+    ((300, 260, 1, 255), 1, 1096, 72),  # few tiles and a long K with a tail: the tiles are split into K slices
+    ((3333, 259, 4000), 2, 64, 136),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", SCALED_ACT_CASES)
+def test_down_projection_dx_swiglu_scaled_act(dtype, case):
+    """dX2 + SwiGLU backward with the second output of its epilogue (xma_rocm_down_projection_dx_swiglu): dz bit-identical
+    to the launch without it; scaled_act[n] = swiglu_packed(z[n]) * w[idx[n]] against the oracle's activation in fp32
+    (one rounding); and dW2 from it, sum_n dy[idx[n] // k]^T scaled_act[n], against the oracle's weight gradient of the
+    scaled grouped dy, sum_n (w dy)[n]^T h[n], per expert."""
+    from xma.rocm import ops
+
+    counts, k, H, I = case
+    print(f"case counts={counts} k={k} H={H} I={I} {dtype}", flush=True)
+    sel, se, ss, offs = _routing_with_counts(counts, k, 21)
+    E, M = len(counts), sum(counts)
+    T = M // k
+    g = torch.Generator().manual_seed(22)
+    dy = torch.randn(T, H, generator=g).to(dtype)
+    W2 = (torch.randn(E, H, I, generator=g) * 0.1).to(dtype)  # c_proj.weight: (E, out = H, in = I)
+    z = torch.randn(M, 2 * I, generator=g).to(dtype)
+    w = torch.rand(M, generator=g).to(dtype)
+    dyd, W2d, zd, wd, ssd, offsd = dy.cuda(), W2.cuda(), z.cuda(), w.cuda(), ss.cuda(), offs.cuda()
+    dz0 = torch.full((M, 2 * I), float("nan"), dtype=dtype, device="cuda")
+    ops.down_projection_dx_swiglu_rocm(dyd, W2d, ssd, offsd, zd, dz0, wd, k)  # W logically (E, K = H, N = I)
+    dz1 = torch.full_like(dz0, float("nan"))
+    hs = torch.full((M, I), float("nan"), dtype=dtype, device="cuda")
+    ops.down_projection_dx_swiglu_scaled_act_rocm(dyd, W2d, ssd, offsd, zd, dz1, hs, wd, k)
+    torch.cuda.synchronize()
+    assert torch.equal(dz0, dz1) and torch.isfinite(dz1).all()
+    h32 = oracle.swiglu_packed(z.float())
+    want_hs = h32 * w.float()[ss][:, None]
+    assert torch.isfinite(hs).all()
+    assert nerr(hs, want_hs) <= _tol(dtype)
+    row_err = (hs.cpu().float() - want_hs).abs().amax(dim=1) / want_hs.abs().amax(dim=1).clamp_min(1e-6)
+    assert row_err.max() <= 4 * _tol(dtype), int(row_err.argmax())
+    # dW2 both ways against the oracle (grouped scaled dy, unscaled h)
+    gdy = (dy.float()[ss // k] * w.float()[ss][:, None]).to(dtype)
+    want_dw = oracle.group_bwd_W(gdy, h32.to(dtype), offs, E)  # (E, I, H)
+    dw = torch.full((E, H, I), float("nan"), dtype=dtype, device="cuda").permute(0, 2, 1)
+    ops.group_bwd_W_rocm(dyd, hs, ssd, offsd, dw, None, k, 0)
+    torch.cuda.synchronize()
+    assert torch.isfinite(dw).all()
+    for e in range(E):
+        if counts[e] == 0:
+            assert torch.count_nonzero(dw[e]) == 0
+        else:
+            assert nerr(dw[e], want_dw[e]) <= 2 * _tol(dtype), e  # two roundings (w h, then the sum) against (w dy, h)
+
+
 def test_scatter2scatter_with_and_without_workspace():
     """The same launch through the C ABI with the scratch for splitting the last round of tiles along K and without
     it (every tile by one workgroup): both within tolerance of the oracle; the workspace query and its error code."""
