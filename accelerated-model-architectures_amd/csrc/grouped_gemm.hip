@@ -236,6 +236,9 @@ __device__ __forceinline__ uint32_t lds_addr_of(const void *p) {
 // Epilogue staging in LDS, private to a wave: one 32-row block of its 128 x 128 corner as 16-bit values (rows padded
 // by 16 bytes against bank conflicts), followed by the 32 x 64 block of SwiGLU activations.
 constexpr int EPI_Z_STRIDE = 128 * 2 + 16, EPI_H_STRIDE = 64 * 2 + 16;
+// Internal epilogue code beside the public XMA_ROCM_EPI_*: SWIGLU_BWD with the second output FwdArgs::aux2.  A variant of
+// its own, so that the launches without that output keep their code and register allocation unchanged.
+constexpr int EPI_SWIGLU_BWD_SCALED_ACT = 3;
 constexpr int EPI_WAVE_BYTES = 32 * EPI_Z_STRIDE + 32 * EPI_H_STRIDE;
 // SwiGLU backward stages 32 rows of 256 pre-activation columns per wave
 constexpr int EPI_BWD_STRIDE = 256 * 2 + 16, EPI_BWD_WAVE_BYTES = 32 * EPI_BWD_STRIDE;
@@ -312,7 +315,7 @@ constexpr int ROLE_TILES = 0, ROLE_SLICES = 1, ROLE_FIXUP = 2;
 // benchmark shapes; the up-projection gains or loses about 1 % depending on the shape and the plain-store launches
 // lose 1 % (their tail is cut into K slices by a launch of its own), so those stay as they are.
 __host__ __device__ constexpr bool fwd_persistent(int epi, int role) {
-    return role == ROLE_TILES && epi == XMA_ROCM_EPI_SWIGLU_BWD;
+    return role == ROLE_TILES && (epi == XMA_ROCM_EPI_SWIGLU_BWD || epi == EPI_SWIGLU_BWD_SCALED_ACT);
 }
 template <int ROLE>
 __device__ __forceinline__ bool locate_tile(const FwdArgs &a, unsigned char *smem, int *s_sched, TileSched &ts,
@@ -437,7 +440,7 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
     // lane owns row (lane & 31) of each 32-row block; quad g of tile (j, i) holds
     //      columns n0 + wp + 32 j + 8 g + 4 (lane >> 5) + {0..3}
     const int lrow = lane & 31, lhalf = lane >> 5;
-    if constexpr (EPI != XMA_ROCM_EPI_SWIGLU_BWD) {
+    if constexpr (EPI != XMA_ROCM_EPI_SWIGLU_BWD && EPI != EPI_SWIGLU_BWD_SCALED_ACT) {
         // A store instruction of the accumulator layout would touch 32 rows with 16 bytes each.  Instead every
         // 32-row block goes through a wave-private LDS area and leaves as whole rows: 16 lanes x 16 bytes per row of
         // 128 columns (8 lanes per row of the 64 activation columns), i.e. full 128-byte lines.
@@ -569,10 +572,21 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
         const int i_first = only_i >= 0 ? only_i : 0, i_last = only_i >= 0 ? only_i : 3;
         if (wq + i_first * 32 < rows_valid) load_block(i_first);
         // HS: a second output, the activations scaled by the row scale, (M, N) in grouped order.  A lane keeps its 128
-        // values of a block packed in 32 registers until the dz rows have left, then the block takes the same way out
-        // through the staging area (32 rows of 128 columns, the layout of the plain store epilogue).  Storing each quad
-        // straight from registers instead (8 bytes per lane, 16 bytes of 32 rows per instruction, no registers held)
-        // measured no faster.
+        // values of a block, packed in 32 registers, until the dz rows have left; then the block takes the same way out
+        // through the staging area (32 rows of 128 columns, the layout of the plain store epilogue).  The 32 registers
+        // are accumulation registers - the 64 of the block's own accumulators are free by then - written and read with
+        // v_accvgpr moves: as ordinary variables they push the kernel's register allocation into spilling.  (Storing
+        // each quad straight from registers, 8 bytes per lane = 16 bytes of 32 rows per instruction, measured slower.)
+        auto park = [](uint32_t v) {
+            uint32_t r;
+            asm volatile("v_accvgpr_write_b32 %0, %1" : "=a"(r) : "v"(v));
+            return r;
+        };
+        auto unpark = [](uint32_t r) {
+            uint32_t v;
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(v) : "a"(r));
+            return v;
+        };
         auto blocks = [&](auto HS) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -583,7 +597,7 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
             if (i < i_last && wq + (i + 1) * 32 < rows_valid) load_block(i + 1);
             wave_lds_sync();
             const float sc = sc_i[i];
-            u32x2 hs[HS.value ? 16 : 1];
+            uint32_t hs[HS.value ? 32 : 1];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
 #pragma unroll
@@ -601,7 +615,10 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
                         hv[q] = uu * silu * sc;
                     }
                     *zp = o;
-                    if constexpr (HS.value != 0) hs[j * 4 + g] = u32x2{Elem<T>::pack(hv[0], hv[1]), Elem<T>::pack(hv[2], hv[3])};
+                    if constexpr (HS.value != 0) {
+                        hs[2 * (j * 4 + g)] = park(Elem<T>::pack(hv[0], hv[1]));
+                        hs[2 * (j * 4 + g) + 1] = park(Elem<T>::pack(hv[2], hv[3]));
+                    }
                 }
             }
             wave_lds_sync();
@@ -619,7 +636,8 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
 #pragma unroll
-                    for (int g = 0; g < 4; ++g) *(u32x2 *)(h_w + (j * 32 + g * 8) * 2) = hs[j * 4 + g];
+                    for (int g = 0; g < 4; ++g)
+                        *(u32x2 *)(h_w + (j * 32 + g * 8) * 2) = u32x2{unpark(hs[2 * (j * 4 + g)]), unpark(hs[2 * (j * 4 + g) + 1])};
                 wave_lds_sync();
 #pragma unroll
                 for (int it = 0; it < 8; ++it) {
@@ -631,10 +649,7 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
             }
         }
         };
-        if (a.aux2)
-            blocks(IC<1>{});
-        else
-            blocks(IC<0>{});
+        blocks(IC<(EPI == EPI_SWIGLU_BWD_SCALED_ACT) ? 1 : 0>{});
     }
 }
 
@@ -1575,6 +1590,7 @@ template <typename T> int dispatch_fwd(const FwdArgs &a, int wt, int epi, hipStr
     }
     if (epi == XMA_ROCM_EPI_STORE) return launch_fwd<T, 1, XMA_ROCM_EPI_STORE>(a, st);
     if (epi == XMA_ROCM_EPI_SWIGLU) return launch_fwd<T, 1, XMA_ROCM_EPI_SWIGLU>(a, st);
+    if (a.aux2) return launch_fwd<T, 1, EPI_SWIGLU_BWD_SCALED_ACT>(a, st);
     return launch_fwd<T, 1, XMA_ROCM_EPI_SWIGLU_BWD>(a, st);
 }
 
@@ -1639,9 +1655,10 @@ static int scatter2scatter_impl(const void *X, int64_t ldx, const void *W, int64
         XMA_REQUIRE(out && aux && aligned16(out) && aligned16(aux) && ldaux % 8 == 0 && y_grouped, XMA_ROCM_EINVAL,
                     "scatter2scatter: SWIGLU_BWD needs out, aux (z) and y_grouped");
     }
-    XMA_REQUIRE(!aux2 || (epilogue == XMA_ROCM_EPI_SWIGLU_BWD && dtype != XMA_ROCM_F32 && aligned16(aux2) && ldaux2 % 8 == 0 &&
-                          ldaux2 >= N),
-                XMA_ROCM_EINVAL, "scatter2scatter: scaled activations go with SWIGLU_BWD in bf16 / fp16, 16-byte aligned rows");
+    XMA_REQUIRE(!aux2 || (epilogue == XMA_ROCM_EPI_SWIGLU_BWD && aligned16(aux2) && ldaux2 % 8 == 0 && ldaux2 >= N),
+                XMA_ROCM_EINVAL, "scatter2scatter: scaled activations go with SWIGLU_BWD, 16-byte aligned rows");
+    XMA_REQUIRE(!aux2 || (dtype != XMA_ROCM_F32 && w_is_kn), XMA_ROCM_EUNSUPPORTED,
+                "scatter2scatter: scaled activations need bf16 / fp16 and W[e] as (K, N) with N contiguous (dy @ W)");
     FwdArgs a;
     a.X = (const uint16_t *)X;
     a.ldx = ldx;
@@ -1700,7 +1717,7 @@ extern "C" int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *
 }
 
 extern "C" int xma_rocm_down_projection_dx_swiglu(const void *dY, int64_t lddy, const void *W, int64_t w_expert_stride,
-                                                  int64_t ldw, int w_is_kn, const int64_t *sorted_scattered_idxs,
+                                                  int64_t ldw, const int64_t *sorted_scattered_idxs,
                                                   const int64_t *expert_offsets, const void *z, int64_t ldz, void *dz,
                                                   int64_t lddz, void *scaled_act, int64_t ld_scaled_act,
                                                   const void *row_scale, int64_t M, int32_t N, int32_t K, int32_t E,
@@ -1709,7 +1726,7 @@ extern "C" int xma_rocm_down_projection_dx_swiglu(const void *dY, int64_t lddy, 
     XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED,
                 "down_projection_dx_swiglu: dtype %d (bf16 and fp16 only)", dtype);
     XMA_REQUIRE(row_scale && scaled_act, XMA_ROCM_EINVAL, "down_projection_dx_swiglu: row_scale and scaled_act are required");
-    return scatter2scatter_impl(dY, lddy, W, w_expert_stride, ldw, w_is_kn, sorted_scattered_idxs, expert_offsets, dz, lddz,
+    return scatter2scatter_impl(dY, lddy, W, w_expert_stride, ldw, 1, sorted_scattered_idxs, expert_offsets, dz, lddz,
                                 const_cast<void *>(z), ldz, scaled_act, ld_scaled_act, row_scale, M, N, K, E, fan_out, 0, 1,
                                 XMA_ROCM_EPI_SWIGLU_BWD, dtype, workspace, workspace_bytes, stream);
 }

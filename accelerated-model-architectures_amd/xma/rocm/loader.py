@@ -44,7 +44,7 @@ SIGNATURES = {
     ),
     "xma_rocm_down_projection_dx_swiglu": (
         _int,
-        [_p, _i64, _p, _i64, _i64, _int, _p, _p, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _i32, _i32, _i32, _i32, _int,
+        [_p, _i64, _p, _i64, _i64, _p, _p, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _i32, _i32, _i32, _i32, _int,
          _p, _sz, _p],
     ),
     "xma_rocm_group_bwd_W": (

@@ -240,12 +240,13 @@ def down_projection_dx_swiglu_scaled_act_rocm(
     assert sorted_scattered_idxs.dtype == torch.int64 and sorted_scattered_idxs.is_contiguous()
     assert expert_offsets.dtype == torch.int64 and expert_offsets.is_contiguous() and expert_offsets.numel() == E
     w_is_kn, w_es, ldw = _weight_layout(W)
+    assert w_is_kn == 1, "W should be the down-projection parameter as stored, (E, H, I) with I contiguous"
     lib = get_library()
     ws_bytes = scatter2scatter_workspace_bytes(M, N, K, E, dY.device.index or 0)
     workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dY.device) if ws_bytes else None
     check(
         lib.xma_rocm_down_projection_dx_swiglu(
-            _ptr(dY), _rows(dY, "dY"), _ptr(W), w_es, ldw, w_is_kn, _ptr(sorted_scattered_idxs), _ptr(expert_offsets),
+            _ptr(dY), _rows(dY, "dY"), _ptr(W), w_es, ldw, _ptr(sorted_scattered_idxs), _ptr(expert_offsets),
             _ptr(z), _rows(z, "z"), _ptr(dz), _rows(dz, "dz"), _ptr(scaled_act), _rows(scaled_act, "scaled_act"),
             _ptr(row_scale), M, N, K, E, FAN_OUT, _code(dY), _ptr(workspace), ws_bytes, _stream(dY),
         ),

@@ -142,10 +142,11 @@ XMA_API int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *W, 
  * scaled_act is the X operand of the down-projection's weight gradient when dY is taken unscaled through the index:
  * sum_n (w_n dy_n)^T h_n = sum_n dy_n^T (w_n h_n).  It replaces the scaled, grouped copy of dY that the reference
  * builds for that GEMM (`group` with coeff, xma/layers/moe/triton_implementation/__init__.py:134-140): k times fewer
- * bytes are written when H > N, and h need not be kept for the backward.  bf16 / fp16; row_scale and scaled_act required.
+ * bytes are written when H > N, and h need not be kept for the backward.  bf16 / fp16; row_scale and scaled_act required;
+ * W[e] is (K, N) with N contiguous (the parameter of the down-projection as stored, B_e = W[e]).
  */
 XMA_API int xma_rocm_down_projection_dx_swiglu(const void *dY, int64_t lddy, const void *W, int64_t w_expert_stride,
-                                               int64_t ldw, int w_is_kn, const int64_t *sorted_scattered_idxs,
+                                               int64_t ldw, const int64_t *sorted_scattered_idxs,
                                                const int64_t *expert_offsets, const void *z, int64_t ldz, void *dz,
                                                int64_t lddz, void *scaled_act, int64_t ld_scaled_act,
                                                const void *row_scale, int64_t M, int32_t N, int32_t K, int32_t num_experts,
