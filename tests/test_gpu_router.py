@@ -213,3 +213,33 @@ def test_router_gate_topk_strided_rows_and_fallback():
     assert not ops.router_gate_topk_supported(512, 64, 33, torch.bfloat16)
     assert not ops.router_gate_topk_supported(516, 64, 2, torch.bfloat16)
     assert not ops.router_gate_topk_supported(512, 64, 2, torch.float32)
+
+
+def test_router_gate_backward_with_a_loss_on_the_logits():
+    """The gate's gradients with and without a loss on the returned router logits (an auxiliary loss adds its gradient to
+    the router's d_logits; without one that output's gradient arrives as None), against the fp32 chain."""
+    from tests.utils import nerr
+    from xma.layers.moe import rocm_implementation as R
+
+    g = torch.Generator().manual_seed(5)
+    T, H, E, k = 257, 512, 16, 4
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    wg = (torch.randn(E, H, generator=g) * H**-0.5).to(torch.bfloat16)
+    dw = torch.randn(T, k, generator=g).to(torch.bfloat16)
+    dl = torch.randn(T, E, generator=g).to(torch.bfloat16)
+    for with_logits in (False, True):
+        xd, wd = x.cuda().requires_grad_(), wg.cuda().requires_grad_()
+        logits, w, ids = R.router_gate_topk(xd, wd, k)
+        loss = (w * dw.cuda()).sum()
+        if with_logits:
+            loss = loss + (logits * dl.cuda()).sum()
+        loss.backward()
+        xf, wf = x.float().requires_grad_(), wg.float().requires_grad_()
+        lg = xf @ wf.t()
+        lg = lg + (logits.detach().cpu().float() - lg).detach()  # the device's logit values, the fp32 chain's derivative
+        rw = torch.softmax(lg.gather(-1, ids.cpu().long()), -1)
+        ref = (rw * dw.float()).sum()
+        if with_logits:
+            ref = ref + (lg * dl.float()).sum()
+        ref.backward()
+        assert nerr(xd.grad, xf.grad) <= 2e-2 and nerr(wd.grad, wf.grad) <= 2e-2, with_logits
