@@ -95,8 +95,21 @@ class _RouterGateTopK(torch.autograd.Function):
             if d_logits_out is not None:  # the caller also used the returned router logits (an auxiliary loss)
                 d_logits = d_logits + d_logits_out
         d_x = d_logits @ gate_weight if ctx.needs_input_grad[0] else None
-        d_w = d_logits.t() @ x if ctx.needs_input_grad[1] else None
+        d_w = _gate_weight_grad(d_logits, x) if ctx.needs_input_grad[1] else None
         return d_x, d_w, None
+
+
+def _gate_weight_grad(d_logits: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """d_Wg = d_logits^T @ x, (E, T) x (T, H): an output of E x H elements with a reduction over all tokens, for which the
+    stock GEMM launches few workgroups.  From 32 experts and 8192 tokens on the tokens are cut into 32 slices whose
+    products run as one batched GEMM and are added in fp32 (measured 158 -> 51 us at T = 32768, E = 128, H = 2048;
+    104 -> 38 us at T = 16384, E = 64; with 8 experts the single GEMM is faster)."""
+    T, E = d_logits.shape
+    slices = 32
+    if E >= 32 and T >= 8192 and T % slices == 0 and x.is_contiguous() and d_logits.is_contiguous():
+        partial = torch.bmm(d_logits.view(slices, T // slices, E).transpose(1, 2), x.view(slices, T // slices, x.size(1)))
+        return partial.sum(0, dtype=torch.float32).to(x.dtype)
+    return d_logits.t() @ x
 
 
 def router_gate_topk(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int):

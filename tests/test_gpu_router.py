@@ -156,6 +156,7 @@ GATE_CASES = [  # T, H, E, k
     (4133, 1032, 96, 4),
     (2085, 2048, 128, 8),
     (24613, 136, 40, 3),  # enough tokens for the variant without a K split
+    (8192, 256, 64, 4),  # the gate's weight gradient as a batched GEMM over slices of the tokens
     (24577, 64, 128, 8),
 ]
 
