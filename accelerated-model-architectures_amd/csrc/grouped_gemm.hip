@@ -547,10 +547,18 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
         // the same way.  The z rows of block i + 1 are requested before the stores of block i go out: loads and
         // stores retire in order, so a load issued behind the stores would wait for them.
         unsigned char *stage = smem + wave * EPI_BWD_WAVE_BYTES;
-        unsigned char *row_io = stage + (lane >> 5) * EPI_BWD_STRIDE + (lane & 31) * 16; // + 2 it rows
+        unsigned char *row_io = stage + (lane >> 5) * EPI_BWD_STRIDE + (lane & 31) * 16; // + 2 it rows (way in)
         unsigned char *mine = stage + lrow * EPI_BWD_STRIDE + lhalf * 16;                // + (32 j + 8 g) * 4 bytes
-        const int cz = 2 * (n0 + wp) + (lane & 31) * 8; // this lane's 8 columns of z / dz on the way in and out
-        const bool col_ok = cz < 2 * a.N;
+        // Loads and stores of this epilogue are unconditional: a lane whose row or column lies outside the tile's valid
+        // part repeats the access of a lane inside it (same address, and for stores the same data, read from the same place
+        // of the staging area).  Memory operations under a per-lane condition sit in branches, and the compiler then waits
+        // for all of them (vmcnt(0)) where it would otherwise count: every block would wait for the stores of the one
+        // before it to complete before it could bring its own rows of z into LDS.
+        // this wave's 128 columns lie past N: nothing to do, and nothing in here joins other waves (the value is uniform;
+        // readfirstlane tells the compiler so, which keeps the branch scalar)
+        if (__builtin_amdgcn_readfirstlane(n0 + wp) >= a.N) return;
+        const int piece = (2 * (n0 + wp) + (lane & 31) * 8 < 2 * a.N) ? (lane & 31) : 0; // piece 0 is inside N
+        const int cz = 2 * (n0 + wp) + piece * 8; // this lane's 8 columns of z / dz on the way in and out
         float sc_i[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -565,8 +573,7 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
             for (int it = 0; it < 16; ++it) {
                 int r = wq + i * 32 + 2 * it + (lane >> 5);
                 if (r >= rows_valid) r = rows_valid - 1;
-                zin[it] = u32x4{0u, 0u, 0u, 0u};
-                if (col_ok) zin[it] = *(const u32x4 *)(a.aux + (row0 + r) * a.ldaux + cz);
+                zin[it] = *(const u32x4 *)(a.aux + (row0 + r) * a.ldaux + cz);
             }
         };
         const int i_first = only_i >= 0 ? only_i : 0, i_last = only_i >= 0 ? only_i : 3;
@@ -624,15 +631,16 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
             wave_lds_sync();
 #pragma unroll
             for (int it = 0; it < 16; ++it) {
-                const int r = wq + i * 32 + 2 * it + (lane >> 5);
-                const u32x4 v = *(const u32x4 *)(row_io + 2 * it * EPI_BWD_STRIDE);
-                if (r < rows_valid && col_ok) *(u32x4 *)(a.out + (row0 + r) * a.ldo + cz) = v;
+                int br = 2 * it + (lane >> 5); // row of the block; the block's first row is valid
+                if (wq + i * 32 + br >= rows_valid) br = rows_valid - 1 - (wq + i * 32);
+                const u32x4 v = *(const u32x4 *)(stage + br * EPI_BWD_STRIDE + piece * 16);
+                *(u32x4 *)(a.out + (row0 + wq + i * 32 + br) * a.ldo + cz) = v;
             }
             wave_lds_sync(); // the next block overwrites the area
             if constexpr (HS.value != 0) {
                 unsigned char *h_w = stage + lrow * EPI_Z_STRIDE + lhalf * 8;
-                const unsigned char *h_r = stage + (lane >> 4) * EPI_Z_STRIDE + (lane & 15) * 16;
-                const int ch = n0 + wp + (lane & 15) * 8; // this lane's 8 activation columns on the way out
+                const int hpiece = (n0 + wp + (lane & 15) * 8 < a.N) ? (lane & 15) : 0; // as above: no store is conditional
+                const int ch = n0 + wp + hpiece * 8; // this lane's 8 activation columns on the way out
 #pragma unroll
                 for (int j = 0; j < 4; ++j)
 #pragma unroll
@@ -641,9 +649,10 @@ __device__ __forceinline__ void tile_epilogue(const FwdArgs &a, f32x16 (&acc)[4]
                 wave_lds_sync();
 #pragma unroll
                 for (int it = 0; it < 8; ++it) {
-                    const int r = wq + i * 32 + 4 * it + (lane >> 4);
-                    const u32x4 v = *(const u32x4 *)(h_r + it * 4 * EPI_Z_STRIDE);
-                    if (r < rows_valid && ch < a.N) *(u32x4 *)(a.aux2 + (row0 + r) * a.ldaux2 + ch) = v;
+                    int br = 4 * it + (lane >> 4);
+                    if (wq + i * 32 + br >= rows_valid) br = rows_valid - 1 - (wq + i * 32);
+                    const u32x4 v = *(const u32x4 *)(stage + br * EPI_Z_STRIDE + hpiece * 16);
+                    *(u32x4 *)(a.aux2 + (row0 + wq + i * 32 + br) * a.ldaux2 + ch) = v;
                 }
                 wave_lds_sync();
             }
@@ -1115,8 +1124,13 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
         const char *base = (piece < 8) ? q_base + (int64_t)kt * (2 * BK) : p_base + (int64_t)kt * p_step_b; // uniform
         const uint32_t off = (piece < 8) ? q_off[piece] : p_off[piece - 8];
         if constexpr (FULL.value) {
+            // the base is uniform by construction; where the register allocation keeps it in vector registers all the
+            // same, the two readfirstlane bring it back (they fold away where it already is scalar)
+            const uint64_t b64 = (uint64_t)base;
+            const char *ubase = (const char *)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(b64 >> 32)) << 32) |
+                                               (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b64));
             asm volatile("s_add_i32 m0, %0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, %3" ::"s"(dst0), "s"(stage), "v"(off),
-                         "s"(base)
+                         "s"(ubase)
                          : "memory", "m0", "scc");
         } else {
             const char *src = base + off;
