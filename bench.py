@@ -46,7 +46,7 @@ WORKLOADS = {
 # 1.0: the factors a 1 GiB device copy, `--workload copy`, gives for the same counters).  bench.py cannot read hardware
 # counters itself: the figures are copied from the profile named beside them and are NOT measured in this run.
 MEASURED_TRAFFIC_BYTES = {
-    "c3": 9.47e9,  # up-projection + SwiGLU GEMM: 8.06 GB fetched + 1.41 GB written (3.42 GB algorithmic)
+    "c3": 9.00e9,  # up-projection + SwiGLU GEMM: 7.59 GB fetched + 1.41 GB written (3.42 GB algorithmic)
     "c2": 92.2e6,  # route: unit histogram 18.9 MB + scan 0.6 MB + scatter 72.7 MB (36.1 MB fetched + 56.2 MB written)
 }
 TRAFFIC_SOURCE = "profiles/hbm_traffic_c3_c2_pmc.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE; a constant, not measured in this run)"
