@@ -70,6 +70,31 @@ def _scratch_inside_mfma_loop(asm_path: str, which: re.Pattern) -> list[str]:
     return bad
 
 
+def _resource_usage_from_asm(asm_path: str) -> dict[str, dict[str, str]]:
+    """{kernel: {field: value}} from the kernel metadata at the end of a device ISA listing (a compile with -save-temps
+    prints no resource remarks, so the kernels that the check below exists for are read from their listing)"""
+    keys = {".vgpr_count": "VGPRs", ".agpr_count": "AGPRs", ".private_segment_fixed_size": "ScratchSize [bytes/lane]",
+            ".group_segment_fixed_size": "LDS Size [bytes/block]", ".vgpr_spill_count": "VGPR spills",
+            ".sgpr_spill_count": "SGPR spills", ".sgpr_count": "SGPRs"}
+    out: dict[str, dict[str, str]] = {}
+    cur: dict[str, str] = {}
+    with open(asm_path) as f:
+        for line in f:
+            m = re.match(r"^\s+(?:- )?(\.[a-z_]+):\s+(\S+)\s*$", line)
+            if not m:
+                continue
+            key, val = m.group(1), m.group(2)
+            if key == ".agpr_count":  # first field of a kernel's record
+                cur = {}
+            if key in keys:
+                cur[keys[key]] = val
+            elif key == ".name" and val.startswith("_Z"):
+                out[val] = cur
+    for v in out.values():  # the VGPR figure of the remarks counts both files, as the occupancy rule does
+        v.setdefault("Occupancy [waves/SIMD]", str(max(1, 512 // max(int(v.get("VGPRs", "512")), 1))))
+    return out
+
+
 def _resource_usage(stderr: str) -> dict[str, dict[str, str]]:
     """{kernel: {field: value}} from the -Rpass-analysis=kernel-resource-usage remarks"""
     out: dict[str, dict[str, str]] = {}
@@ -99,7 +124,8 @@ def _check_compiler(verbose: bool) -> None:
 
 def _compile(src: str, verbose: bool, defines: tuple[str, ...] = (), tag: str = "") -> str:
     obj = os.path.join(HERE, "build", src.replace(".hip", tag + ".o"))
-    extra = ["-save-temps=obj"] if src in LOOP_NO_SCRATCH else []  # keeps the device ISA next to the object
+    # keeps the device ISA next to the object (named after the source, so only the untagged build of a file may do this)
+    extra = ["-save-temps=obj"] if src in LOOP_NO_SCRATCH and not tag else []
     cmd = [HIPCC, *FLAGS, *extra, *defines, "-c", os.path.join(CSRC, src), "-o", obj]
     if verbose:
         print(" ".join(cmd), flush=True)
@@ -112,11 +138,12 @@ def _compile(src: str, verbose: bool, defines: tuple[str, ...] = (), tag: str = 
         raise RuntimeError(f"hipcc failed on {src}:\n{err}")
     if re.search(r"warning|error", err) and verbose:
         print(err, file=sys.stderr)
-    if src in LOOP_NO_SCRATCH:
-        asm = os.path.join(HERE, "build", src.replace(".hip", tag + "-hip-amdgcn-amd-amdhsa-gfx950.s"))
+    if extra:
+        asm = os.path.join(HERE, "build", src.replace(".hip", "-hip-amdgcn-amd-amdhsa-gfx950.s"))
         bad = _scratch_inside_mfma_loop(asm, LOOP_NO_SCRATCH[src])
         if bad:
             raise RuntimeError(f"{src}: scratch stores inside the MFMA loop of:\n  " + "\n  ".join(bad))
+        usage = _resource_usage_from_asm(asm)
     return obj, usage
 
 
@@ -130,8 +157,9 @@ def build(verbose: bool = False) -> str:
     with open(USAGE_REPORT, "w") as f:
         for _, usage in results:
             for k, v in usage.items():
+                spills = f" spilled VGPRs {v['VGPR spills']}" if v.get("VGPR spills", "0") != "0" else ""
                 f.write(f"{k}: VGPRs {v.get('VGPRs')} AGPRs {v.get('AGPRs')} scratch {v.get('ScratchSize [bytes/lane]')} "
-                        f"LDS {v.get('LDS Size [bytes/block]')} occupancy {v.get('Occupancy [waves/SIMD]')}\n")
+                        f"LDS {v.get('LDS Size [bytes/block]')} occupancy {v.get('Occupancy [waves/SIMD]')}{spills}\n")
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB, *objs]
     if verbose:
         print(" ".join(cmd), flush=True)

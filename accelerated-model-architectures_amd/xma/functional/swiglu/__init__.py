@@ -52,9 +52,13 @@ class _SwigluPackedROCm(torch.autograd.Function):
 
 
 def _row_major_2d(t: torch.Tensor) -> torch.Tensor:
-    """2-D view with contiguous rows (any row pitch is fine for the kernels; anything else is copied)"""
+    """2-D view with contiguous rows that do not overlap (any row pitch >= the row length is fine for the kernels).
+    Anything else is copied: transposed views, and the broadcast views autograd hands to a backward - the gradient of
+    ``y.sum(0)`` has strides (0, 1) - or a caller passes as an expanded operand."""
     t = t.reshape(-1, t.size(-1)) if t.dim() != 2 else t
-    return t if t.stride(1) == 1 or t.size(1) == 1 else t.contiguous()
+    rows_ok = t.stride(1) == 1 or t.size(1) == 1
+    pitch_ok = t.size(0) <= 1 or t.stride(0) >= t.size(1)
+    return t if rows_ok and pitch_ok else t.contiguous()
 
 
 class _SwigluROCm(torch.autograd.Function):

@@ -119,7 +119,12 @@ def router_gate_topk(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int):
 
 
 def router_gate_topk_supported(x: torch.Tensor, gate_weight: torch.Tensor, top_k: int) -> bool:
+    """Whether the fused kernel takes these tensors; anything else (mixed dtypes, tensors on different devices, a row
+    pitch that is no multiple of 16 bytes, a shape outside the kernel's range) goes through gate(x) + router_topk.  Only
+    properties a traced caller can evaluate are looked at; a tensor that starts off a 16-byte boundary is copied inside
+    the op.  Note that the fused path returns int32 expert ids, the fallback int64 like torch.topk: `route` reads either."""
     return x.is_cuda and x.dim() == 2 and x.stride(1) == 1 and x.stride(0) % 8 == 0 and gate_weight.is_contiguous() and \
+        gate_weight.dtype == x.dtype and gate_weight.device == x.device and gate_weight.dim() == 2 and \
         ops.router_gate_topk_supported(x.size(1), gate_weight.size(0), top_k, x.dtype)
 
 

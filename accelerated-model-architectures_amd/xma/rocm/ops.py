@@ -426,6 +426,11 @@ def router_gate_topk_rocm(x: torch.Tensor, gate_weight: torch.Tensor, logits: to
     assert x.dtype == gate_weight.dtype == logits.dtype == weights.dtype and ids.dtype in (torch.int32, torch.int64)
     assert weights.is_contiguous() and ids.is_contiguous()
     lib = get_library()
+    # the kernel reads 16-byte pieces: a view that starts off such a boundary (a column slice at an odd offset) is copied
+    if x.data_ptr() % 16:
+        x = x.contiguous()
+    if gate_weight.data_ptr() % 16:
+        gate_weight = gate_weight.clone()
     check(
         lib.xma_rocm_router_gate_topk(_ptr(x), _rows(x, "x"), _ptr(gate_weight), _rows(gate_weight, "gate_weight"), T, H, E, k,
                                       _code(x), _ptr(logits), _rows(logits, "logits"), _ptr(weights), _ptr(ids),

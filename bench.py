@@ -14,6 +14,7 @@ copied) that are resident in HBM before the timed region.  Prints ONE JSON line:
   cpu_baseline the CPU oracle (plain torch restatement of the reference's torch path) on a bounded
                sample of the same workload, on this box's host cores
   kernels      per-kernel duration / throughput table (extra, for the record)
+  other_configs (default workload only) c4, c5 and c2 measured in the same run and summarised
 """
 
 from __future__ import annotations
@@ -42,14 +43,36 @@ WORKLOADS = {
 }
 
 
-# HBM bytes per launch of each workload's dominant kernel, from two counter runs (FETCH_SIZE scaled by 2.0, WRITE_SIZE by
-# 1.0: the factors a 1 GiB device copy, `--workload copy`, gives for the same counters).  bench.py cannot read hardware
-# counters itself: the figures are copied from the profile named beside them and are NOT measured in this run.
+# HBM bytes per launch of the GEMM kernels of c3 and of c2's route, from two counter runs (FETCH_SIZE scaled by 2.0,
+# WRITE_SIZE by 1.0: the factors a 1 GiB device copy, `--workload copy`, gives for the same counters).  bench.py cannot
+# read hardware counters itself: the figures are copied from the profile named beside them and are NOT measured in this
+# run; the roofline block carries the one of the kernel it names.
 MEASURED_TRAFFIC_BYTES = {
-    "c3": 9.00e9,  # up-projection + SwiGLU GEMM: 7.59 GB fetched + 1.41 GB written (3.42 GB algorithmic)
+    "c3": {
+        "up_swiglu": 9.00e9,  # 7.59 GB fetched + 1.41 GB written (3.42 GB algorithmic)
+        "down": 3.69e9,  # three launches: whole tiles, K slices of the last round, their sum
+        "dx2_swiglu_bwd": 6.77e9,
+        "dw2": 3.76e9,
+        "dw1": 7.52e9,
+        "dx1": 7.39e9,  # three launches
+    },
     "c2": 92.2e6,  # route: unit histogram 18.9 MB + scan 0.6 MB + scatter 72.7 MB (36.1 MB fetched + 56.2 MB written)
 }
 TRAFFIC_SOURCE = "profiles/hbm_traffic_c3_c2_pmc.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE; a constant, not measured in this run)"
+
+
+def _host_cpu() -> dict:
+    """model name and logical CPU count of the host the CPU baseline runs on"""
+    model = "unknown"
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"cpu_model": model, "os_cpu_count": os.cpu_count()}
 
 
 def _time_gpu(fn, iters: int, warmup: int = 2) -> float:
@@ -199,7 +222,7 @@ def _kernel_table(moe, x, rw, sel, grad, cfg, iters):
     return table, notes
 
 
-def run_moe(args, cfg, name):
+def measure_moe(args, cfg, name, cpu_baseline=True):
     from oracle import moe as oracle_moe
     from xma import KernelBackend
 
@@ -250,11 +273,12 @@ def run_moe(args, cfg, name):
 
     table, notes = _kernel_table(moe, x, rw, sel, grad, cfg, args.kernel_iters)
     gemms = {n: v for n, v in table.items() if "tflops" in v}
-    # the dominant kernel: the up-projection + SwiGLU GEMM (4 Tk H I FLOP like dW1 and dX1, and the longest of the three
-    # or within a per cent of it; fixing the choice keeps the figure, the counters and the profile on one kernel)
-    dom = next(n for n in gemms if n.startswith("up_swiglu"))
+    # the dominant kernel: the GEMM launch (group) that takes longest in this run
+    dom = max(gemms, key=lambda n: gemms[n]["ms"])
     total_flops = sum(v["flops"] for v in gemms.values())
     total_ms = sum(v["ms"] for v in gemms.values())
+    traffic = MEASURED_TRAFFIC_BYTES.get(name)
+    dom_traffic = traffic.get(dom.split("(")[0]) if isinstance(traffic, dict) else None
     roofline = {
         "kernel": dom,
         "bound": "mfma",
@@ -262,16 +286,17 @@ def run_moe(args, cfg, name):
         "peak": PEAK_BF16_TFLOPS,
         "unit": "TFLOP/s",
         "frac": round(gemms[dom]["tflops"] / PEAK_BF16_TFLOPS, 4),
-        "traffic": MEASURED_TRAFFIC_BYTES.get(name) if dom.startswith("up_swiglu") else None,
-        "traffic_source": TRAFFIC_SOURCE if name in MEASURED_TRAFFIC_BYTES else None,
+        "traffic": dom_traffic,
+        "traffic_source": TRAFFIC_SOURCE if dom_traffic else None,
         "all_gemms_tflops": round(total_flops / total_ms / 1e9, 1),
         "all_gemms_frac": round(total_flops / total_ms / 1e9 / PEAK_BF16_TFLOPS, 4),
+        "gemm_fracs": {n.split("(")[0]: v["frac_mfma_peak"] for n, v in gemms.items()},
     }
 
     # CPU baseline: the oracle, bf16 like the reference's torch path, on the first T / cpu_fraction tokens with every other
     # dimension unchanged (same weights, bit-identical)
     cpu = None
-    if not args.no_cpu_baseline:
+    if cpu_baseline and not args.no_cpu_baseline:
         Ts = max(T // args.cpu_fraction, 1)
         w1, w2 = moe.c_fc.weight.detach().cpu(), moe.c_proj.weight.detach().cpu()
         xs, rws, sels, gs = x[:Ts].cpu(), rw[:Ts].cpu(), sel[:Ts].cpu(), grad[:Ts].cpu()
@@ -284,6 +309,7 @@ def run_moe(args, cfg, name):
             "value": round(Ts / dt, 1),
             "unit": "tokens/s",
             "cores": torch.get_num_threads(),
+            **_host_cpu(),
             "kind": "port",
             "sample": f"fwd+bwd of the torch-path oracle in bf16 on the first {Ts} of {T} tokens (all other dimensions and "
                       f"the weights unchanged), mean of {reps} runs of {dt:.1f} s",
@@ -309,18 +335,22 @@ def run_moe(args, cfg, name):
             "tokens": T,
             "rows_per_expert_min_mean_max": [int(counts.min()), float(counts.float().mean()), int(counts.max())],
             "step_tflops": round(18.0 * T * k * H * I / ms_per_step / 1e9, 1),
+            # what `value` and `ms_per_step` time: MoE._compute_experts behind given router logits (BASELINE's metric)
             "step": "router top-k/softmax/ids from the given logits + routing + experts fwd+bwd down to d_logits",
-            "whole_layer_ms": round(layer_ms, 4),  # MoE.forward + backward with the gate projection fused into the router
+            # for the record, the whole layer: MoE.forward + backward with the gate projection fused into the router
+            "whole_layer_ms": round(layer_ms, 4),
         },
         "roofline": roofline,
         "cpu_baseline": cpu,
         "kernels": table,
         "notes": notes,
     }
-    print(json.dumps(out))
+    del moe, x, logits, rw, sel, grad, xg, lg
+    torch.cuda.empty_cache()
+    return out
 
 
-def run_routing(args):
+def measure_routing(args, zipf, cpu_baseline=True):
     """configs[1]: continuous_count + routing on 4 Mi int32 ids over 64 experts (uniform; --zipf for the skewed run)"""
     from oracle import routing as oracle_routing
     from xma import KernelBackend
@@ -330,7 +360,7 @@ def run_routing(args):
 
     n, E = 4 * 1024 * 1024, 64
     g = torch.Generator().manual_seed(0)
-    if args.zipf:
+    if zipf:
         p = torch.arange(1, E + 1, dtype=torch.float64) ** (-1.1)
         ids_cpu = torch.multinomial(p / p.sum(), n, replacement=True, generator=g).to(torch.int32)
     else:
@@ -400,11 +430,12 @@ def run_routing(args):
     copy_ms = ref_graph_ms(lambda i: halves[i].copy_(halves[(i + 1) % nbuf]))
     read_ms = ref_graph_ms(lambda i: halves[0][:64].copy_(bufs[i].view(torch.uint8)[:64]))  # launch floor of one kernel
     del outs, halves
-    t1 = time.perf_counter()
-    reps = 3
-    for _ in range(reps):
-        oracle_routing.route(ids_cpu.numpy(), E)
-    dt = (time.perf_counter() - t1) / reps
+    reps, dt = 3, None
+    if cpu_baseline and not args.no_cpu_baseline:
+        t1 = time.perf_counter()
+        for _ in range(reps):
+            oracle_routing.route(ids_cpu.numpy(), E)
+        dt = (time.perf_counter() - t1) / reps
     out = {
         "metric": "routing_ids_per_s",
         "value": round(n / ms_per_step * 1e3, 1),
@@ -419,7 +450,7 @@ def run_routing(args):
         "dtype": "int32",
         "data": "synthetic",
         "config": {"workload": f"c2: counts + offsets + stable permutation of {n} int32 ids over E={E}, "
-                               f"{'Zipf(s=1.1)' if args.zipf else 'uniform'}, {nbuf} rotating input buffers"},
+                               f"{'Zipf(s=1.1)' if zipf else 'uniform'}, {nbuf} rotating input buffers"},
         "roofline": {
             "kernel": "route (3 kernels: unit histogram, scan, stable scatter), per call, replayed from a graph",
             "bound": "hbm",
@@ -427,11 +458,12 @@ def run_routing(args):
             "peak": PEAK_HBM_GBS,
             "unit": "GB/s",
             "frac": round(route_bytes / route_graph_ms / 1e6 / PEAK_HBM_GBS, 4),
-            "traffic": None if args.zipf else MEASURED_TRAFFIC_BYTES["c2"],
-            "traffic_source": None if args.zipf else TRAFFIC_SOURCE,
+            "traffic": None if zipf else MEASURED_TRAFFIC_BYTES["c2"],
+            "traffic_source": None if zipf else TRAFFIC_SOURCE,
         },
-        "cpu_baseline": {"value": round(n / dt, 1), "unit": "ids/s", "cores": 1, "kind": "port",
-                         "sample": f"numpy stable argsort + bincount + cumsum of the same {n} ids, mean of {reps}"},
+        "cpu_baseline": None if dt is None else {
+            "value": round(n / dt, 1), "unit": "ids/s", "cores": 1, **_host_cpu(), "kind": "port",
+            "sample": f"numpy stable argsort + bincount + cumsum of the same {n} ids, mean of {reps}"},
         "kernels": {
             "continuous_count_cold": {"ms": round(hist_ms, 5), "gbs": round(hist_bytes / hist_ms / 1e6, 1),
                                       "frac_hbm_peak": round(hist_bytes / hist_ms / 1e6 / PEAK_HBM_GBS, 4), "bytes": hist_bytes},
@@ -450,7 +482,37 @@ def run_routing(args):
             "one 64-byte copy kernel [graph]": {"ms": round(read_ms, 5)},
         },
     }
-    print(json.dumps(out))
+    del bufs
+    torch.cuda.empty_cache()
+    return out
+
+
+def _other_configs(args) -> dict:
+    """The configurations beside the headline one, measured in the same process and summarised: c4 and c5 (a few steps and
+    the per-kernel table each), c2 uniform and Zipf (route and continuous_count replayed from a graph)."""
+    res = {}
+    saved = (args.steps, args.warmup)
+    args.steps, args.warmup = max(3, min(args.steps, 5)), 2
+    for name in ("c4", "c5"):
+        r = measure_moe(args, WORKLOADS[name], name, cpu_baseline=False)
+        fr = r["roofline"]["gemm_fracs"]
+        low = min(fr, key=fr.get)
+        res[name] = {"ms_per_step": r["ms_per_step"], "tokens_per_s": r["value"], "step_tflops": r["config"]["step_tflops"],
+                     "whole_layer_ms": r["config"]["whole_layer_ms"], "all_gemms_frac": r["roofline"]["all_gemms_frac"],
+                     "gemm_fracs": fr, "lowest_gemm": low, "dominant_gemm": r["roofline"]["kernel"],
+                     "rows_per_expert_min_mean_max": r["config"]["rows_per_expert_min_mean_max"],
+                     "hbm_kernels_frac": {n.split("(")[0]: v["frac_hbm_peak"] for n, v in r["kernels"].items()
+                                          if "frac_hbm_peak" in v and not n.startswith("plain")}}
+    for label, zipf in (("c2_uniform", False), ("c2_zipf", True)):
+        r = measure_routing(args, zipf, cpu_baseline=False)
+        k = r["kernels"]
+        res[label] = {"route_graph_us": round(k["route_graph"]["ms"] * 1e3, 2), "route_frac_hbm": k["route_graph"]["frac_hbm_peak"],
+                      "continuous_count_graph_us": round(k["continuous_count_graph"]["ms"] * 1e3, 2),
+                      "continuous_count_frac_hbm": k["continuous_count_graph"]["frac_hbm_peak"],
+                      "continuous_count_op_us": round(k["continuous_count_cold"]["ms"] * 1e3, 2),
+                      "route_op_us": round(k["route"]["ms"] * 1e3, 2)}
+    args.steps, args.warmup = saved
+    return res
 
 
 def run_copy(args):
@@ -541,6 +603,7 @@ def main():
     ap.add_argument("--kernel-iters", type=int, default=5)
     ap.add_argument("--cpu-fraction", type=int, default=1, help="CPU baseline runs on T / this many tokens")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true", help="c3 only: leave out the summary of c4, c5 and c2")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus N with N > 1 is not supported (no collectives in the path)")
@@ -556,9 +619,12 @@ def main():
     elif args.workload == "library_gemm":
         run_library_gemm(args)
     elif args.workload == "c2":
-        run_routing(args)
+        print(json.dumps(measure_routing(args, args.zipf)))
     else:
-        run_moe(args, WORKLOADS[args.workload], args.workload)
+        out = measure_moe(args, WORKLOADS[args.workload], args.workload)
+        if args.workload == "c3" and not args.no_other_configs:
+            out["other_configs"] = _other_configs(args)
+        print(json.dumps(out))
 
 
 if __name__ == "__main__":

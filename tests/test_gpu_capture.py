@@ -64,6 +64,59 @@ def test_compiled_module_matches_eager(backend, k):
             assert torch.equal(got[name], want[name]), name
 
 
+@pytest.mark.parametrize("backend", ["aot_eager", "inductor"])
+def test_compiled_functionals_match_eager(backend):
+    """The functionals under torch.compile(fullgraph=True), as the reference's tests run them
+    (tests/functional/continuous_count_test.py:25, tests/functional/swiglu_test.py: eager and compiled function side by
+    side): continuous_count over sizes of the reference's 1-D rule in both id types against the oracle, swiglu and
+    swiglu_packed forward and backward bit-identical to their eager runs."""
+    from oracle import routing as oracle_routing
+    from tests.utils import get_1d_tensor_sizes, np_of
+    from xma import KernelBackend
+    from xma.functional import continuous_count, swiglu, swiglu_packed
+
+    torch._dynamo.reset()
+    g = torch.Generator().manual_seed(3)
+    bins = 72
+    try:
+        cc = torch.compile(continuous_count, fullgraph=True, backend=backend)
+        sizes = get_1d_tensor_sizes()
+        for n in sizes[:: max(1, len(sizes) // 10)] + [70000]:  # 70000: the two-pass path, its scratch allocated in the op
+            for dtype in (torch.int32, torch.int64):
+                ids = torch.randint(0, bins, (n,), generator=g, dtype=dtype)
+                got = cc(ids.cuda(), bins, kernel_backend=KernelBackend.rocm)
+                assert got.dtype == torch.uint32 and got.shape == (bins,)
+                assert np_of(got).tolist() == oracle_routing.continuous_count(ids.numpy(), bins).tolist(), (n, dtype)
+        assert np_of(cc(torch.zeros(5, dtype=torch.int32, device="cuda"), 1, kernel_backend=KernelBackend.rocm)).tolist() == [5]
+
+        csw = torch.compile(swiglu, fullgraph=True, backend=backend)
+        cswp = torch.compile(swiglu_packed, fullgraph=True, backend=backend)
+        for dtype in (torch.bfloat16, torch.float32):
+            for rows, cols in [(7, 9), (64, 64), (300, 1408), (1025, 513)]:
+                gate = torch.randn(rows, cols, generator=g).to(dtype).cuda()
+                up = torch.randn(rows, cols, generator=g).to(dtype).cuda()
+                dy = torch.randn(rows, cols, generator=g).to(dtype).cuda()
+                res = []
+                for fn in (swiglu, csw):
+                    gd, ud = gate.clone().requires_grad_(), up.clone().requires_grad_()
+                    y = fn(gd, ud, kernel_backend=KernelBackend.rocm)
+                    y.backward(dy)
+                    res.append((y.detach(), gd.grad, ud.grad))
+                assert all(torch.equal(a, b) for a, b in zip(*res)), (rows, cols, dtype)
+                xp = torch.randn(rows, 2 * cols, generator=g).to(dtype).cuda()
+                res = []
+                for fn in (swiglu_packed, cswp):
+                    xd = xp.clone().requires_grad_()
+                    y = fn(xd, kernel_backend=KernelBackend.rocm)
+                    y.backward(dy)
+                    res.append((y.detach(), xd.grad))
+                assert all(torch.equal(a, b) for a, b in zip(*res)), (rows, cols, dtype)
+    except torch._dynamo.exc.BackendCompilerFailed as err:  # the code generator's own toolchain, not the ops under test
+        if backend == "inductor":
+            pytest.skip(f"inductor cannot generate code on this machine: {str(err)[:300]}")
+        raise
+
+
 @pytest.mark.parametrize("k", [2, 4])
 def test_graph_capture_and_replay(k):
     """fwd + bwd of the router (behind the gate) and of the expert computation captured once and replayed on new

@@ -168,3 +168,35 @@ def test_full_size_shared_weights_equal_dense_mlp():
         e = nerr(got, ref)
         print(f"   {label}: nerr={e:.2e}", flush=True)
         assert e <= TOL, f"{label}: {e}"
+
+
+def test_full_size_layer_forward_with_fused_gate():
+    """MoE.forward on the Mixtral-shaped configuration: the gate projection runs inside the router kernel, and its int32
+    expert ids go straight into the routing kernels.  Router logits of sampled tokens against the fp32 product (one
+    rounding to bf16 plus the summation order); the layer's output rows of those tokens against the oracle run on the
+    experts and router weights that the oracle's top-k / softmax derive from the device's own logits (a 16-bit logit
+    that differs in its last place may legitimately pick another expert)."""
+    from xma import KernelBackend
+
+    print("full size c3: MoE.forward with the fused gate", flush=True)
+    T, H, I, E, k, _ = CONFIGS["c3"]
+    moe, x, _, _, _ = _inputs("c3")
+    g = torch.Generator(device="cuda").manual_seed(11)
+    with torch.no_grad():
+        moe.gate.weight.copy_((torch.randn(E, H, generator=g, device="cuda") * H**-0.5).to(torch.bfloat16))
+        y, logits = moe(x, kernel_backend=KernelBackend.rocm)
+    torch.cuda.synchronize()
+    assert y.shape == (T, H) and logits.shape == (T, E) and logits.dtype == torch.bfloat16
+    assert torch.isfinite(y).all() and torch.isfinite(logits).all()
+    gen = torch.Generator().manual_seed(1)
+    tok = torch.cat([torch.tensor([0, 1, 31, 32, 63, 64, T - 1]), torch.randint(0, T, (57,), generator=gen)]).unique()
+    xs = x[tok.cuda()].float().cpu()
+    dev_logits = logits[tok.cuda()].cpu()
+    lg = xs @ moe.gate.weight.detach().float().cpu().t()
+    assert (lg - dev_logits.float()).abs().max().item() <= 2.0**-7 * max(1.0, lg.abs().max().item())  # 2 ulp of bf16
+    rw, sel = oracle.routing_topk(dev_logits, k, torch.bfloat16)
+    want = oracle.experts_forward(xs, rw.float(), sel, moe.c_fc.weight.detach().float().cpu(),
+                                  moe.c_proj.weight.detach().float().cpu(), oracle.swiglu_packed)
+    e = nerr(y[tok.cuda()], want)
+    print(f"   {len(tok)} tokens: y nerr={e:.2e}", flush=True)
+    assert e <= TOL

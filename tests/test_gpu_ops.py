@@ -72,6 +72,60 @@ def test_scatter2scatter(dtype, case, w_kn, x_grouped, y_grouped):
         assert nerr(out, want) <= _tol(dtype)
 
 
+def test_scatter2scatter_launches_outside_the_persistent_kernel():
+    """Three launches that the layer itself never makes and that take the one-workgroup-per-tile kernel instead of the
+    persistent one: more experts than its schedule tables hold (E = 1100, most of them empty), a row scale that starts
+    off a 4-byte boundary (the persistent kernel fetches the aligned dword around a 16-bit scale), and dy @ W (W as
+    (K, N)) with the SwiGLU forward epilogue, reachable through the C ABI only."""
+    from xma.layers.moe import rocm_implementation as R
+    from xma.rocm.loader import get_library
+
+    dtype = torch.bfloat16
+    g = torch.Generator().manual_seed(31)
+    # (1) E = 1100
+    T, E, k, K, N = 700, 1100, 2, 136, 264
+    sel, se, ss, offs = _routing(T, E, k, 5, skew=2.0)
+    M = T * k
+    X = torch.randn(T, K, generator=g).to(dtype)
+    W = (torch.randn(E, N, K, generator=g) * 0.1).to(dtype)
+    want = oracle.scatter2scatter(X, W.permute(0, 2, 1), se, ss, k, False, True, None)
+    out = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+    R.scatter2scatter(X.cuda(), W.cuda().permute(0, 2, 1), se.cuda(), ss.cuda(), out, k, False, True, offs.cuda(), None)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all() and nerr(out, want) <= TOL
+    # (2) a row scale at an odd element offset, grouped rows in, scattered rows out
+    T, E, k, K, N = 300, 3, 2, 192, 320
+    sel, se, ss, offs = _routing(T, E, k, 6)
+    M = T * k
+    X = torch.randn(M, K, generator=g).to(dtype)
+    W = (torch.randn(E, N, K, generator=g) * 0.1).to(dtype)
+    scale_buf = torch.rand(M + 1, generator=g).to(dtype)
+    want = oracle.scatter2scatter(X, W.permute(0, 2, 1), se, ss, k, True, False, scale_buf[1:])
+    sd = scale_buf.cuda()[1:]
+    assert sd.data_ptr() % 4 == 2
+    out = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+    R.scatter2scatter(X.cuda(), W.cuda().permute(0, 2, 1), se.cuda(), ss.cuda(), out, k, True, False, offs.cuda(), sd)
+    torch.cuda.synchronize()
+    assert torch.isfinite(out).all() and nerr(out, want) <= TOL
+    # (3) W[e] as (K, N) with the SwiGLU forward epilogue: z and h = swiglu_packed(z), straight through the C ABI
+    lib = get_library()
+    K, N = 200, 272
+    X = torch.randn(T, K, generator=g).to(dtype)
+    Wkn = (torch.randn(E, K, N, generator=g) * 0.1).to(dtype)
+    want_z = oracle.scatter2scatter(X, Wkn, se, ss, k, False, True, None)
+    want_h = oracle.swiglu_packed(want_z.float())
+    Xd, Wd, ssd, offsd = X.cuda(), Wkn.cuda(), ss.cuda(), offs.cuda()
+    z = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+    h = torch.full((M, N // 2), float("nan"), dtype=dtype, device="cuda")
+    rc = lib.xma_rocm_scatter2scatter(Xd.data_ptr(), K, Wd.data_ptr(), K * N, N, 1, ssd.data_ptr(), offsd.data_ptr(),
+                                      z.data_ptr(), N, h.data_ptr(), N // 2, None, M, N, K, E, k, 0, 1, 1, 0, None, 0,
+                                      torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert rc == 0, lib.xma_rocm_last_error()
+    assert torch.isfinite(z).all() and torch.isfinite(h).all()
+    assert nerr(z, want_z) <= TOL and nerr(h, want_h) <= TOL
+
+
 def _routing_with_counts(counts, k, seed):
     """a routing whose experts own exactly `counts` rows (sum divisible by k): the slots are dealt out at random"""
     g = torch.Generator().manual_seed(seed)
@@ -307,6 +361,40 @@ def test_swiglu_views_and_shapes():
             assert nerr(xpd.grad, torch.stack([dg, du], dim=-1).flatten(-2)) <= _tol(dtype), cols
         empty = torch.empty(0, 16, dtype=dtype, device="cuda")
         assert swiglu(empty, empty, kernel_backend=KernelBackend.rocm).shape == (0, 16)
+
+
+def test_swiglu_broadcast_operands_and_gradients():
+    """Operands and upstream gradients whose rows overlap in memory: the gradient autograd hands back for ``y.sum(0)``
+    has strides (0, 1), an ``expand``-ed operand too.  The rocm path copies them (the kernels want rows that do not
+    overlap); results against the oracle's closed forms."""
+    from xma import KernelBackend
+    from xma.functional import swiglu, swiglu_packed
+
+    g = torch.Generator().manual_seed(13)
+    for dtype in (torch.bfloat16, torch.float32):
+        rows, cols = 37, 203
+        gate = (torch.randn(rows, cols, generator=g) * 2).to(dtype)
+        up = (torch.randn(rows, cols, generator=g) * 2).to(dtype)
+        v = torch.randn(cols, generator=g).to(dtype)
+        gd, ud, vd = gate.cuda().requires_grad_(), up.cuda().requires_grad_(), v.cuda()
+        (swiglu(gd, ud, kernel_backend=KernelBackend.rocm).sum(0) * vd).sum().backward()
+        dy = v.float().expand(rows, cols)  # what the sum over the rows hands back, up to the rounding of y.sum(0)
+        dg, du = oracle.swiglu_backward(gate.float(), up.float(), dy)
+        assert nerr(gd.grad, dg) <= _tol(dtype) and nerr(ud.grad, du) <= _tol(dtype)
+        # one row of `up` for all rows of `gate`, forward and backward
+        u1 = (torch.randn(1, cols, generator=g) * 2).to(dtype)
+        gd, u1d = gate.cuda().requires_grad_(), u1.cuda().requires_grad_()
+        y = swiglu(gd, u1d.expand(rows, cols), kernel_backend=KernelBackend.rocm)
+        y.backward(torch.ones_like(y))
+        assert nerr(y, oracle.swiglu(gate.float(), u1.float().expand(rows, cols))) <= _tol(dtype)
+        dg, du = oracle.swiglu_backward(gate.float(), u1.float().expand(rows, cols), torch.ones(rows, cols))
+        assert nerr(gd.grad, dg) <= _tol(dtype) and nerr(u1d.grad, du.sum(0, keepdim=True)) <= 2 * _tol(dtype)
+        # the packed form with the same kind of gradient
+        xp = (torch.randn(rows, 2 * cols, generator=g) * 2).to(dtype)
+        xpd = xp.cuda().requires_grad_()
+        (swiglu_packed(xpd, kernel_backend=KernelBackend.rocm).sum(0) * vd).sum().backward()
+        dg, du = oracle.swiglu_backward(xp[..., 0::2].float(), xp[..., 1::2].float(), dy)
+        assert nerr(xpd.grad, torch.stack([dg, du], dim=-1).flatten(-2)) <= _tol(dtype)
 
 
 SCALED_ACT_CASES = [

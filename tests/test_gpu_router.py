@@ -158,6 +158,8 @@ GATE_CASES = [  # T, H, E, k
     (24613, 136, 40, 3),  # enough tokens for the variant without a K split
     (8192, 256, 64, 4),  # the gate's weight gradient as a batched GEMM over slices of the tokens
     (24577, 64, 128, 8),
+    (16384, 2048, 64, 6),  # the two benchmark layers with more than 32 experts, at their exact shapes: two pairs of waves
+    (32768, 2048, 128, 8),  # per workgroup with a K split (below 24576 tokens) and without; 32 K steps through the LDS ring
 ]
 
 
@@ -214,6 +216,14 @@ def test_router_gate_topk_strided_rows_and_fallback():
     assert not ops.router_gate_topk_supported(512, 64, 33, torch.bfloat16)
     assert not ops.router_gate_topk_supported(516, 64, 2, torch.bfloat16)
     assert not ops.router_gate_topk_supported(512, 64, 2, torch.float32)
+    # a gate weight of another dtype is not taken by the fused kernel although the shape is covered: the layer then runs
+    # gate(x) + router_topk; rows that start off a 16-byte boundary are copied inside the op
+    assert not R.router_gate_topk_supported(x, wg.float(), 4)
+    xs = wide[:, 4 : 4 + 512]
+    assert R.router_gate_topk_supported(xs, wg, 4)
+    l3, w3, ids3 = R.router_gate_topk(xs, wg, 4)
+    l4, w4, ids4 = R.router_gate_topk(xs.contiguous(), wg, 4)
+    assert torch.equal(l3, l4) and torch.equal(w3, w4) and torch.equal(ids3, ids4)
 
 
 def test_router_gate_backward_with_a_loss_on_the_logits():
