@@ -152,6 +152,21 @@ __global__ __launch_bounds__(FTHREADS) void gemm_f32_kernel(const FwdArgs a) {
     f32x16 acc[2][2];
     zero_acc(acc);
     const int wq = (wave & 1) * 64, wp = (wave >> 1) * 64;
+    if (a.bias) { // the expert's bias is the first term of every sum (see the epilogue for a lane's columns)
+        const float *b = (const float *)a.bias + (int64_t)e * a.bias_es;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                int col = n0 + wp + j * 32 + g * 8 + (lane >> 5) * 4;
+                if (col > a.N - 4) col = a.N - 4;
+                const f32x4 v = *(const f32x4 *)(b + col);
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) acc[j][i][4 * g + q] = v[q];
+            }
+    }
     const int KT = (a.K + FBK - 1) / FBK;
     TileRegs rq, rp;
     load_kcontig(rq, q_row, 0, a.K, tid);

@@ -20,6 +20,8 @@ struct FwdArgs {
     uint16_t *aux2; // SWIGLU_BWD only, may be NULL: (M, N) = swiglu_packed(z) * row_scale in grouped order
     int64_t ldaux2;
     const uint16_t *scale;
+    const uint16_t *bias; // (E, N) added to the product before the epilogue, or NULL
+    int64_t bias_es;      // elements between the bias rows of two experts
     int64_t M;
     int N, K, E, fan_out, x_grouped, y_grouped;
     FastDiv fan_div; // division of a scattered index by fan_out (indices are below 2^31)

@@ -262,6 +262,33 @@ template <int N> __device__ __forceinline__ void zero_acc(f32x16 (&acc)[N][N]) {
             for (int v = 0; v < 16; ++v) acc[j][i][v] = 0.f;
 }
 
+// The experts' bias enters a tile as a rank-one update of the cleared accumulators, ones (rows) x bias (columns), through
+// the matrix pipe: one k16 step whose only non-zero k holds 1 in the Q fragments and the bias of the lane's column in the P
+// fragments.  The product 1 x b is exact and it is the first term of the fp32 sum, so the result is rounded once, as a
+// linear layer with a bias rounds it, and no epilogue has to know about the bias.  (Writing the bias into the
+// accumulators directly, 256 register writes from loaded values, made the register allocation spill around the main loop.)
+template <typename T> __device__ __forceinline__ uint32_t one_bits();
+template <> __device__ __forceinline__ uint32_t one_bits<__bf16>() { return 0x3f80u; }
+template <> __device__ __forceinline__ uint32_t one_bits<_Float16>() { return 0x3c00u; }
+template <typename T>
+__device__ __forceinline__ void add_bias(const FwdArgs &a, f32x16 (&acc)[4][4], int e, int n0, int wp, int lane) {
+    const uint16_t *b = a.bias + (int64_t)e * a.bias_es;
+    const bool k0 = lane < 32; // lanes 0..31 hold k = 0..7 of their row, lanes 32..63 k = 8..15
+    u32x4 q = {k0 ? one_bits<T>() : 0u, 0u, 0u, 0u};
+    u32x4 p[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        int col = n0 + wp + 32 * j + (lane & 31);
+        if (col >= a.N) col = a.N - 1; // columns past N are computed and never stored
+        const uint32_t v = b[col];
+        p[j] = u32x4{k0 ? v : 0u, 0u, 0u, 0u};
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[j][i] = Elem<T>::mfma(p[j], q, acc[j][i]);
+}
+
 // Which tile a workgroup works on.
 struct TileSched {
     int e, rows_valid, n0; // expert, valid rows of the row tile, first output column
@@ -310,10 +337,9 @@ constexpr int SPLIT_MIN_STEPS = 8; // a K slice is at least this many K steps
 // third launch (ROLE_FIXUP, workgroup b = split tile b) adds the slices.  ROLE_TILES takes all other tiles.  Returns
 // false if the workgroup has nothing to do.
 constexpr int ROLE_TILES = 0, ROLE_SLICES = 1, ROLE_FIXUP = 2;
-// Which launches are persistent (one workgroup per compute unit walking its tiles) instead of one workgroup per tile:
-// the dX of the down-projection with its long SwiGLU-backward epilogue measured 3-4 % faster that way on all three
-// benchmark shapes; the up-projection gains or loses about 1 % depending on the shape and the plain-store launches
-// lose 1 % (their tail is cut into K slices by a launch of its own), so those stay as they are.
+// grouped_gemm_kernel is the fallback of launch_fwd for launches that grouped_gemm_persistent_kernel does not take, and
+// the kernel of the K slices.  Its SwiGLU-backward instantiations also walk several tiles per workgroup (one workgroup
+// per compute unit), the others run one workgroup per tile.
 __host__ __device__ constexpr bool fwd_persistent(int epi, int role) {
     return role == ROLE_TILES && (epi == XMA_ROCM_EPI_SWIGLU_BWD || epi == EPI_SWIGLU_BWD_SCALED_ACT);
 }
@@ -752,6 +778,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_kernel(const Fwd
     f32x16 acc[4][4];
     zero_acc(acc);
     const int wq = (wave & 1) * 128, wp = (wave >> 1) * 128; // wave's 128 x 128 corner inside the tile
+    if (a.bias != nullptr && kt0 == 0) add_bias<T>(a, acc, e, n0, wp, lane); // the first K slice of a split tile only
     FragBase<0> qb;
     FragBase<WT> pb;
     make_frag_base<0>(qb, lds0, wq, lane);
@@ -927,11 +954,14 @@ __device__ __forceinline__ void lds_dma4_raw(const void *src, uint32_t lds_wave_
 #ifdef XMA_PST_TIMING
 constexpr int PST_TIMING_TILES = 48;
 __device__ uint64_t g_pst_times[256][PST_TIMING_TILES][8];
+__device__ uint64_t g_pst_cycles[256][PST_TIMING_TILES][8]; // the shader clock counter at the same points
 __device__ int g_pst_no_ovl; // A/B switch of the timing build: 1 = no tile overlaps its neighbours' set-up
 #define PST_STAMP(k)                                                                                   \
     do {                                                                                               \
-        if (threadIdx.x == 0 && blockIdx.x < 256 && tile_no < PST_TIMING_TILES)                        \
+        if (threadIdx.x == 0 && blockIdx.x < 256 && tile_no < PST_TIMING_TILES) {                      \
             g_pst_times[blockIdx.x][tile_no][k] = __builtin_amdgcn_s_memrealtime();                    \
+            g_pst_cycles[blockIdx.x][tile_no][k] = __builtin_amdgcn_s_memtime();                       \
+        }                                                                                              \
     } while (0)
 #else
 #define PST_STAMP(k) \
@@ -1214,6 +1244,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
         PST_STAMP(2);
         f32x16 acc[4][4];
         zero_acc(acc);
+        if (a.bias != nullptr) add_bias<T>(a, acc, cur.e, cur.n0, wp, lane);
         FragBase<0> qb;
         FragBase<WT> pb;
         make_frag_base<0>(qb, lds0, wq, lane);
@@ -1641,9 +1672,9 @@ using namespace xma_rocm;
 static int scatter2scatter_impl(const void *X, int64_t ldx, const void *W, int64_t w_expert_stride, int64_t ldw,
                                 int w_is_kn, const int64_t *sorted_scattered_idxs, const int64_t *expert_offsets,
                                 void *out, int64_t ldo, void *aux, int64_t ldaux, void *aux2, int64_t ldaux2,
-                                const void *row_scale, int64_t M, int32_t N, int32_t K, int32_t E, int32_t fan_out,
-                                int x_grouped, int y_grouped, int epilogue, int dtype, void *workspace,
-                                size_t workspace_bytes, void *stream) {
+                                const void *row_scale, const void *bias, int64_t bias_expert_stride, int64_t M, int32_t N,
+                                int32_t K, int32_t E, int32_t fan_out, int x_grouped, int y_grouped, int epilogue, int dtype,
+                                void *workspace, size_t workspace_bytes, void *stream) {
     XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16 || dtype == XMA_ROCM_F32, XMA_ROCM_EUNSUPPORTED,
                 "scatter2scatter: dtype %d", dtype);
     XMA_REQUIRE(epilogue >= XMA_ROCM_EPI_STORE && epilogue <= XMA_ROCM_EPI_SWIGLU_BWD, XMA_ROCM_EINVAL,
@@ -1673,7 +1704,13 @@ static int scatter2scatter_impl(const void *X, int64_t ldx, const void *W, int64
                 XMA_ROCM_EINVAL, "scatter2scatter: scaled activations go with SWIGLU_BWD, 16-byte aligned rows");
     XMA_REQUIRE(!aux2 || (dtype != XMA_ROCM_F32 && w_is_kn), XMA_ROCM_EUNSUPPORTED,
                 "scatter2scatter: scaled activations need bf16 / fp16 and W[e] as (K, N) with N contiguous (dy @ W)");
+    XMA_REQUIRE(!bias || (aligned16(bias) && bias_expert_stride % 8 == 0 && bias_expert_stride >= 0 &&
+                          epilogue != XMA_ROCM_EPI_SWIGLU_BWD),
+                XMA_ROCM_EINVAL, "scatter2scatter: bias (E, N) must be 16-byte aligned with an expert stride that is a "
+                                 "multiple of 8 elements, and goes with the STORE and SWIGLU epilogues");
     FwdArgs a;
+    a.bias = (const uint16_t *)bias;
+    a.bias_es = bias_expert_stride;
     a.X = (const uint16_t *)X;
     a.ldx = ldx;
     a.W = (const uint16_t *)W;
@@ -1726,8 +1763,20 @@ extern "C" int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *
                                         int32_t fan_out, int x_grouped, int y_grouped, int epilogue, int dtype,
                                         void *workspace, size_t workspace_bytes, void *stream) {
     return scatter2scatter_impl(X, ldx, W, w_expert_stride, ldw, w_is_kn, sorted_scattered_idxs, expert_offsets, out, ldo,
-                                aux, ldaux, nullptr, 0, row_scale, M, N, K, E, fan_out, x_grouped, y_grouped, epilogue,
-                                dtype, workspace, workspace_bytes, stream);
+                                aux, ldaux, nullptr, 0, row_scale, nullptr, 0, M, N, K, E, fan_out, x_grouped, y_grouped,
+                                epilogue, dtype, workspace, workspace_bytes, stream);
+}
+
+extern "C" int xma_rocm_scatter2scatter_bias(const void *X, int64_t ldx, const void *W, int64_t w_expert_stride,
+                                             int64_t ldw, int w_is_kn, const int64_t *sorted_scattered_idxs,
+                                             const int64_t *expert_offsets, void *out, int64_t ldo, void *aux,
+                                             int64_t ldaux, const void *row_scale, const void *bias,
+                                             int64_t bias_expert_stride, int64_t M, int32_t N, int32_t K, int32_t E,
+                                             int32_t fan_out, int x_grouped, int y_grouped, int epilogue, int dtype,
+                                             void *workspace, size_t workspace_bytes, void *stream) {
+    return scatter2scatter_impl(X, ldx, W, w_expert_stride, ldw, w_is_kn, sorted_scattered_idxs, expert_offsets, out, ldo,
+                                aux, ldaux, nullptr, 0, row_scale, bias, bias_expert_stride, M, N, K, E, fan_out, x_grouped,
+                                y_grouped, epilogue, dtype, workspace, workspace_bytes, stream);
 }
 
 extern "C" int xma_rocm_down_projection_dx_swiglu(const void *dY, int64_t lddy, const void *W, int64_t w_expert_stride,
@@ -1741,13 +1790,16 @@ extern "C" int xma_rocm_down_projection_dx_swiglu(const void *dY, int64_t lddy, 
                 "down_projection_dx_swiglu: dtype %d (bf16 and fp16 only)", dtype);
     XMA_REQUIRE(row_scale && scaled_act, XMA_ROCM_EINVAL, "down_projection_dx_swiglu: row_scale and scaled_act are required");
     return scatter2scatter_impl(dY, lddy, W, w_expert_stride, ldw, 1, sorted_scattered_idxs, expert_offsets, dz, lddz,
-                                const_cast<void *>(z), ldz, scaled_act, ld_scaled_act, row_scale, M, N, K, E, fan_out, 0, 1,
-                                XMA_ROCM_EPI_SWIGLU_BWD, dtype, workspace, workspace_bytes, stream);
+                                const_cast<void *>(z), ldz, scaled_act, ld_scaled_act, row_scale, nullptr, 0, M, N, K, E,
+                                fan_out, 0, 1, XMA_ROCM_EPI_SWIGLU_BWD, dtype, workspace, workspace_bytes, stream);
 }
 
 #ifdef XMA_PST_TIMING
 extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_times(void *host_out) {
     return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_pst_times), sizeof(g_pst_times));
+}
+extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_cycles(void *host_out) {
+    return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_pst_cycles), sizeof(g_pst_cycles));
 }
 extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_band(int v) {
     return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_pst_band), &v, sizeof(v));

@@ -107,7 +107,9 @@ __global__ __launch_bounds__(HIST_THREADS) void histogram_kernel(const IdT *__re
     }
 }
 
-// counts[b] += sum of row b of table[bins][units]; one workgroup per bin, four independent loads in flight per thread
+// counts[b] (+)= sum of row b of table[bins][units]; one workgroup per bin, four independent loads in flight per thread.
+// ACCUMULATE = 0 overwrites counts, so the caller need not clear them.
+template <int ACCUMULATE>
 __global__ __launch_bounds__(256) void histogram_reduce_kernel(const uint32_t *__restrict__ table, int units, int bins,
                                                                uint32_t *__restrict__ counts) {
     __shared__ uint32_t s_part[256 / WAVE];
@@ -121,7 +123,7 @@ __global__ __launch_bounds__(256) void histogram_reduce_kernel(const uint32_t *_
     for (int d = WAVE / 2; d > 0; d >>= 1) s += __shfl_xor(s, d);
     if (tid % WAVE == 0) s_part[tid / WAVE] = s;
     __syncthreads();
-    if (tid == 0) counts[b] += s_part[0] + s_part[1] + s_part[2] + s_part[3];
+    if (tid == 0) counts[b] = (ACCUMULATE ? counts[b] : 0u) + s_part[0] + s_part[1] + s_part[2] + s_part[3];
 }
 
 // bins too many for LDS: straight global atomics (not a MoE-sized case)
@@ -398,7 +400,26 @@ inline void hist_units(int64_t n, int64_t &chunk, int64_t &units) {
 
 template <typename IdT>
 int hist_launch_t(const IdT *ids, int64_t n, uint32_t *counts, int bins, uint32_t *table, size_t table_bytes,
-                  hipStream_t st) {
+                  hipStream_t st, bool overwrite = false) {
+    if (overwrite) {
+        // counts are written, not added to: per-unit histograms and a reduction that stores its sums.  A single unit's
+        // histogram is the result itself (a table of one column is the counts vector).
+        int copies, stride;
+        hist_lds_layout(bins, copies, stride);
+        int64_t chunk, units;
+        hist_units(n, chunk, units);
+        if (units < 1) units = 1;
+        const size_t lds = (size_t)copies * stride * sizeof(uint32_t);
+        if (units == 1) {
+            histogram_kernel<IdT, 1><<<1, HIST_THREADS, lds, st>>>(ids, n, chunk, counts, bins, copies, stride);
+            return xma_check_launch("histogram_kernel");
+        }
+        histogram_kernel<IdT, 1><<<(int)units, HIST_THREADS, lds, st>>>(ids, n, chunk, table, bins, copies, stride);
+        int rc = xma_check_launch("histogram_kernel");
+        if (rc) return rc;
+        histogram_reduce_kernel<0><<<bins, 256, 0, st>>>(table, (int)units, bins, counts);
+        return xma_check_launch("histogram_reduce_kernel");
+    }
     if (bins > HIST_LDS_WORDS) {
         int64_t blocks = (n + HIST_THREADS * 16 - 1) / (HIST_THREADS * 16);
         if (blocks > 2048) blocks = 2048;
@@ -424,7 +445,7 @@ int hist_launch_t(const IdT *ids, int64_t n, uint32_t *counts, int bins, uint32_
     histogram_kernel<IdT, 1><<<(int)units, HIST_THREADS, lds, st>>>(ids, n, chunk, table, bins, copies, stride);
     int rc = xma_check_launch("histogram_kernel");
     if (rc) return rc;
-    histogram_reduce_kernel<<<bins, 256, 0, st>>>(table, (int)units, bins, counts);
+    histogram_reduce_kernel<1><<<bins, 256, 0, st>>>(table, (int)units, bins, counts);
     return xma_check_launch("histogram_reduce_kernel");
 }
 
@@ -449,6 +470,28 @@ extern "C" int xma_rocm_continuous_count(const void *ids, int ids_are_int64, int
     if (ids_are_int64)
         return hist_launch_t<int64_t>((const int64_t *)ids, n, counts, bins, (uint32_t *)workspace, workspace_bytes, st);
     return hist_launch_t<int32_t>((const int32_t *)ids, n, counts, bins, (uint32_t *)workspace, workspace_bytes, st);
+}
+
+extern "C" size_t xma_rocm_continuous_count_set_workspace_bytes(int64_t n, int32_t bins) {
+    if (n <= UNIT_IDS || bins < 1 || bins > HIST_LDS_WORDS) return 0; // one workgroup writes the counts itself
+    int64_t chunk, units;
+    hist_units(n, chunk, units);
+    return (size_t)units * (size_t)bins * sizeof(uint32_t);
+}
+
+extern "C" int xma_rocm_continuous_count_set(const void *ids, int ids_are_int64, int64_t n, uint32_t *counts, int32_t bins,
+                                             void *workspace, size_t workspace_bytes, void *stream) {
+    XMA_REQUIRE(n >= 0 && bins >= 1 && bins <= HIST_LDS_WORDS, XMA_ROCM_EINVAL, "continuous_count_set: n=%lld bins=%d (bins <= %d)",
+                (long long)n, bins, HIST_LDS_WORDS);
+    XMA_REQUIRE(counts != nullptr && (ids != nullptr || n == 0), XMA_ROCM_EINVAL, "continuous_count_set: null pointer");
+    XMA_REQUIRE(((uintptr_t)ids % (ids_are_int64 ? 8 : 4)) == 0, XMA_ROCM_EINVAL, "continuous_count_set: misaligned ids");
+    const size_t need = xma_rocm_continuous_count_set_workspace_bytes(n, bins);
+    XMA_REQUIRE(need == 0 || (workspace && workspace_bytes >= need), XMA_ROCM_EWORKSPACE,
+                "continuous_count_set: workspace %zu < %zu bytes", workspace ? workspace_bytes : (size_t)0, need);
+    hipStream_t st = (hipStream_t)stream;
+    if (ids_are_int64)
+        return hist_launch_t<int64_t>((const int64_t *)ids, n, counts, bins, (uint32_t *)workspace, workspace_bytes, st, true);
+    return hist_launch_t<int32_t>((const int32_t *)ids, n, counts, bins, (uint32_t *)workspace, workspace_bytes, st, true);
 }
 
 extern "C" int xma_rocm_route_set_rank_method(int method) {

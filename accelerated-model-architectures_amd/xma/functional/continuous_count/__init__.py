@@ -31,10 +31,14 @@ def continuous_count(x: torch.Tensor, bins: int, *, kernel_backend: KernelBacken
         assert kernel_backend.verify_accelerator()
 
     if kernel_backend == KernelBackend.rocm:
-        from ...rocm.ops import continuous_count_rocm
+        from ...rocm.ops import CONTINUOUS_COUNT_SET_MAX_BINS, continuous_count_rocm, continuous_count_set_rocm
 
-        y = torch.zeros(bins, dtype=torch.uint32, device=x.device)
-        continuous_count_rocm(x=x.contiguous(), y=y, workspace=None)
+        if bins <= CONTINUOUS_COUNT_SET_MAX_BINS:  # the kernels write the counts: no zero fill
+            y = torch.empty(bins, dtype=torch.uint32, device=x.device)
+            continuous_count_set_rocm(x=x.contiguous(), y=y)
+        else:
+            y = torch.zeros(bins, dtype=torch.uint32, device=x.device)
+            continuous_count_rocm(x=x.contiguous(), y=y, workspace=None)
     elif kernel_backend == KernelBackend.torch:
         y = x.bincount(minlength=bins).to(torch.uint32)
     else:

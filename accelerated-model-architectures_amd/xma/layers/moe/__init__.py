@@ -76,6 +76,10 @@ class MoE(nn.Module):
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
         self.is_glu = is_glu
+        # rocm backend with the fused SwiGLU path only (not a constructor argument: the signature is the reference's).
+        # False: keep x and the pre-activations between forward and backward and recompute the activations and the expert
+        # outputs in the backward, as the reference's backward does (triton_implementation/__init__.py:117-128).
+        self.save_activations = True
 
         self.gate = nn.Linear(in_features=hidden_size, out_features=num_experts, bias=False)
         self.c_fc = Experts(
@@ -136,18 +140,23 @@ class MoE(nn.Module):
         if kernel_backend == KernelBackend.rocm:
             from . import rocm_implementation as R
 
-            assert self.c_fc.bias is None and self.c_proj.bias is None
             _, expert_offsets, _, sorted_expert_idxs, sorted_scattered_idxs = R.route(selected_experts, self.num_experts)
             x = x.contiguous()
             w_fc, w_proj = self.c_fc.weight.permute(0, 2, 1), self.c_proj.weight.permute(0, 2, 1)
+            # the experts' biases (the reference applies them on its torch path only, :96-100; its Triton path asserts
+            # that there are none, :53 and :75) enter the grouped GEMMs as the first term of their fp32 sums
+            b_fc, b_proj = self.c_fc.bias, self.c_proj.bias
 
             if self.is_glu and getattr(self.act, "_xma_fused_activation", None) == "swiglu_packed":
-                x = R.fused_swiglu_experts(x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets)
+                x = R.fused_swiglu_experts(x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets, b_fc,
+                                           b_proj, self.save_activations)
             else:
-                x = R.up_projection_experts(x, w_fc, self.top_k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets)
+                x = R.up_projection_experts(x, w_fc, self.top_k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets,
+                                            b_fc)
                 x = self.act(x)
                 x = R.down_projection_experts(
-                    x.contiguous(), w_proj, 1, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, router_weights
+                    x.contiguous(), w_proj, 1, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, router_weights,
+                    b_proj
                 )
         elif kernel_backend == KernelBackend.torch:
             # the reference's torch path (moe/__init__.py:210-211, 235-250)

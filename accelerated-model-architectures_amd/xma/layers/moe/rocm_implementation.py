@@ -201,25 +201,34 @@ def _scale_activations_for_dw2(top_k: int, grad_out: torch.Tensor) -> bool:
 
 
 # ----------------------------------------------------------------------------------------- autograd
+def _bias_grad(A, sorted_scattered_idxs, expert_offsets, bias, row_scale=None, fan_out=1):
+    """d_bias (E, out) = per-expert column sums of the grouped (or gathered and scaled) gradient rows"""
+    d_bias = torch.empty_like(bias, memory_format=torch.contiguous_format)
+    ops.expert_column_sums_rocm(A, sorted_scattered_idxs, expert_offsets, d_bias, row_scale, fan_out)
+    return d_bias
+
+
 class _UpProjectionExperts(torch.autograd.Function):
-    """x (T, H) -> grouped (T*k, out); counterpart of triton_implementation/__init__.py:12-72."""
+    """x (T, H) -> grouped (T*k, out); counterpart of triton_implementation/__init__.py:12-72, plus the experts' bias
+    that the reference has on its torch path only (moe/__init__.py:96-100)."""
 
     @staticmethod
-    def forward(ctx, x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets):
+    def forward(ctx, x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, bias=None):
         output = torch.empty(sorted_expert_idxs.size(0), expert_weights.size(-1), device=x.device, dtype=x.dtype)
-        ops.scatter2scatter_rocm(x, expert_weights, sorted_scattered_idxs, expert_offsets, output, None, k, False, True)
-        ctx.save_for_backward(x, expert_weights, sorted_scattered_idxs, expert_offsets)
+        ops.scatter2scatter_rocm(x, expert_weights, sorted_scattered_idxs, expert_offsets, output, None, k, False, True, bias)
+        ctx.save_for_backward(x, expert_weights, sorted_scattered_idxs, expert_offsets, bias)
         ctx.k = k
         return output
 
     @staticmethod
     def backward(ctx, grad_out):
-        x, expert_weights, sorted_scattered_idxs, expert_offsets = ctx.saved_tensors
+        x, expert_weights, sorted_scattered_idxs, expert_offsets, bias = ctx.saved_tensors
         k = ctx.k
         grad_out = grad_out.contiguous()
 
         d_weights = _empty_dw_like(expert_weights)
         ops.group_bwd_W_rocm(grad_out, x, sorted_scattered_idxs, expert_offsets, d_weights, None, 0, k)
+        d_bias = None if bias is None else _bias_grad(grad_out, None, expert_offsets, bias)
 
         scattered = torch.empty(sorted_scattered_idxs.size(0), x.size(1), dtype=x.dtype, device=x.device)
         ops.scatter2scatter_rocm(
@@ -227,7 +236,7 @@ class _UpProjectionExperts(torch.autograd.Function):
         )
         d_input = torch.empty_like(x)
         ops.combine_rocm(scattered, None, d_input, k)
-        return d_input, d_weights, None, None, None, None
+        return d_input, d_weights, None, None, None, None, d_bias
 
 
 class _DownProjectionExperts(torch.autograd.Function):
@@ -235,20 +244,20 @@ class _DownProjectionExperts(torch.autograd.Function):
     triton_implementation/__init__.py:75-162 (there called with k = 1 and router_weights (T, top_k))."""
 
     @staticmethod
-    def forward(ctx, x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, router_weights):
+    def forward(ctx, x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, router_weights, bias=None):
         assert k == 1
         T, top_k = router_weights.shape
         expert_out = torch.empty(sorted_expert_idxs.size(0), expert_weights.size(-1), device=x.device, dtype=x.dtype)
-        ops.scatter2scatter_rocm(x, expert_weights, sorted_scattered_idxs, expert_offsets, expert_out, None, 1, True, False)
+        ops.scatter2scatter_rocm(x, expert_weights, sorted_scattered_idxs, expert_offsets, expert_out, None, 1, True, False, bias)
         router_weights = router_weights.contiguous()
         y = torch.empty(T, expert_out.size(1), device=x.device, dtype=x.dtype)
         ops.combine_rocm(expert_out, router_weights, y, top_k)
-        ctx.save_for_backward(x, expert_weights, sorted_scattered_idxs, expert_offsets, router_weights, expert_out)
+        ctx.save_for_backward(x, expert_weights, sorted_scattered_idxs, expert_offsets, router_weights, expert_out, bias)
         return y
 
     @staticmethod
     def backward(ctx, grad_out):
-        x, expert_weights, sorted_scattered_idxs, expert_offsets, router_weights, expert_out = ctx.saved_tensors
+        x, expert_weights, sorted_scattered_idxs, expert_offsets, router_weights, expert_out, bias = ctx.saved_tensors
         top_k = router_weights.size(1)
         grad_out = grad_out.contiguous()
 
@@ -257,53 +266,69 @@ class _DownProjectionExperts(torch.autograd.Function):
 
         flat_w = router_weights.view(-1)
         d_weights = _empty_dw_like(expert_weights)
-        ops.group_bwd_W_rocm(_scaled_grouped_dy(grad_out, sorted_scattered_idxs, flat_w, top_k), x, sorted_scattered_idxs,
-                             expert_offsets, d_weights, None, 0, 0)
+        grouped_dy = _scaled_grouped_dy(grad_out, sorted_scattered_idxs, flat_w, top_k)
+        ops.group_bwd_W_rocm(grouped_dy, x, sorted_scattered_idxs, expert_offsets, d_weights, None, 0, 0)
+        d_bias = None if bias is None else _bias_grad(grouped_dy, None, expert_offsets, bias)
 
         d_input = torch.empty_like(x)
         ops.scatter2scatter_rocm(
             grad_out, expert_weights.permute(0, 2, 1), sorted_scattered_idxs, expert_offsets, d_input, flat_w, top_k, False, True
         )
-        return d_input, d_weights, None, None, None, None, d_router_weights
+        return d_input, d_weights, None, None, None, None, d_router_weights, d_bias
 
 
 class _FusedSwiGLUExperts(torch.autograd.Function):
     """Whole expert computation with packed SwiGLU in the GEMM epilogues:
-    forward  up-projection (+ SwiGLU) -> down-projection (scattered) -> combine
-    backward combine' -> dX2 (+ SwiGLU') -> dW2, dW1 -> dX1 (scattered) -> k-way sum."""
+    forward  up-projection (+ bias, SwiGLU) -> down-projection (+ bias, scattered) -> combine
+    backward combine' -> dX2 (+ SwiGLU') -> dW2, dW1 (and the bias gradients) -> dX1 (scattered) -> k-way sum.
+    save_activations = False keeps x and the pre-activations z only: the backward then recomputes h = swiglu_packed(z)
+    and the expert outputs (one more down-projection GEMM), as the reference's backward recomputes its expert outputs
+    (triton_implementation/__init__.py:117-128)."""
 
     @staticmethod
-    def forward(ctx, x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets):
+    def forward(ctx, x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets, b_fc=None, b_proj=None,
+                save_activations=True):
         # w_fc: (E, H, 2I) view, w_proj: (E, I, H) view (both permuted views of the parameters)
         T, top_k = router_weights.shape
         M = sorted_scattered_idxs.numel()
         z = torch.empty(M, w_fc.size(-1), device=x.device, dtype=x.dtype)
         h = torch.empty(M, w_fc.size(-1) // 2, device=x.device, dtype=x.dtype)
-        ops.up_projection_swiglu_rocm(x, w_fc, sorted_scattered_idxs, expert_offsets, z, h, top_k)
+        ops.up_projection_swiglu_rocm(x, w_fc, sorted_scattered_idxs, expert_offsets, z, h, top_k, b_fc)
         expert_out = torch.empty(M, w_proj.size(-1), device=x.device, dtype=x.dtype)
-        ops.scatter2scatter_rocm(h, w_proj, sorted_scattered_idxs, expert_offsets, expert_out, None, 1, True, False)
+        ops.scatter2scatter_rocm(h, w_proj, sorted_scattered_idxs, expert_offsets, expert_out, None, 1, True, False, b_proj)
         router_weights = router_weights.contiguous()
         y = torch.empty(T, expert_out.size(1), device=x.device, dtype=x.dtype)
         ops.combine_rocm(expert_out, router_weights, y, top_k)
         # h is an operand of dW2 only where dW2 takes the scaled grouped copy of dy; otherwise the backward rebuilds it,
         # scaled, from z in the dX2 epilogue and h lives until the end of this forward only
-        kept_h = h.new_empty(0) if _scale_activations_for_dw2(top_k, x) else h
-        ctx.save_for_backward(x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets, z, kept_h, expert_out)
+        kept_h = h if save_activations and not _scale_activations_for_dw2(top_k, x) else h.new_empty(0)
+        kept_out = expert_out if save_activations else expert_out.new_empty(0)
+        ctx.save_for_backward(x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets, z, kept_h, kept_out,
+                              b_fc, b_proj)
         return y
 
     @staticmethod
     def backward(ctx, grad_out):
-        x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets, z, h, expert_out = ctx.saved_tensors
+        (x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets, z, h, expert_out, b_fc,
+         b_proj) = ctx.saved_tensors
         top_k = router_weights.size(1)
         grad_out = grad_out.contiguous()
         flat_w = router_weights.view(-1)
+        scaled_act_path = _scale_activations_for_dw2(top_k, grad_out)
 
+        if expert_out.numel() == 0 and z.numel() != 0:  # not kept: recomputed from z
+            if h.numel() == 0:
+                h = torch.empty(z.size(0), z.size(1) // 2, dtype=z.dtype, device=z.device)
+                ops.swiglu_packed_forward_rocm(z, h)
+            expert_out = torch.empty(z.size(0), w_proj.size(-1), device=z.device, dtype=z.dtype)
+            ops.scatter2scatter_rocm(h, w_proj, sorted_scattered_idxs, expert_offsets, expert_out, None, 1, True, False, b_proj)
         d_router_weights = torch.empty_like(router_weights)
         ops.combine_bwd_rocm(expert_out, grad_out, d_router_weights)
 
         dz = torch.empty_like(z)
         d_w_proj = _empty_dw_like(w_proj)
-        if h.numel() == 0 and z.numel() != 0:  # the forward decided (_scale_activations_for_dw2) not to keep h
+        d_b_proj = None
+        if scaled_act_path and z.numel() != 0:
             # dW2 = sum_n (w_n dy_n)^T h_n = sum_n dy_n^T (w_n h_n): the dX2 epilogue, which has z and w_n at hand, writes
             # w_n h_n (T*k, I), and dW2 takes dy unscaled through the index - instead of a scaled, grouped copy of dy
             # (T*k, H) written by `group` and read back by the GEMM
@@ -312,31 +337,42 @@ class _FusedSwiGLUExperts(torch.autograd.Function):
                 grad_out, w_proj.permute(0, 2, 1), sorted_scattered_idxs, expert_offsets, z, dz, scaled_h, flat_w, top_k
             )
             ops.group_bwd_W_rocm(grad_out, scaled_h, sorted_scattered_idxs, expert_offsets, d_w_proj, None, top_k, 0)
+            if b_proj is not None:
+                d_b_proj = _bias_grad(grad_out, sorted_scattered_idxs, expert_offsets, b_proj, flat_w, top_k)
         else:
             ops.down_projection_dx_swiglu_rocm(
                 grad_out, w_proj.permute(0, 2, 1), sorted_scattered_idxs, expert_offsets, z, dz, flat_w, top_k
             )
-            ops.group_bwd_W_rocm(_scaled_grouped_dy(grad_out, sorted_scattered_idxs, flat_w, top_k), h,
-                                 sorted_scattered_idxs, expert_offsets, d_w_proj, None, 0, 0)
+            grouped_dy = _scaled_grouped_dy(grad_out, sorted_scattered_idxs, flat_w, top_k)
+            ops.group_bwd_W_rocm(grouped_dy, h, sorted_scattered_idxs, expert_offsets, d_w_proj, None, 0, 0)
+            if b_proj is not None:
+                d_b_proj = _bias_grad(grouped_dy, None, expert_offsets, b_proj)
         d_w_fc = _empty_dw_like(w_fc)
         ops.group_bwd_W_rocm(dz, x, sorted_scattered_idxs, expert_offsets, d_w_fc, None, 0, top_k)
+        d_b_fc = None if b_fc is None else _bias_grad(dz, None, expert_offsets, b_fc)
 
-        scattered = expert_out.new_empty(expert_out.shape)
+        scattered = torch.empty(z.size(0), x.size(1), dtype=x.dtype, device=x.device)
         ops.scatter2scatter_rocm(dz, w_fc.permute(0, 2, 1), sorted_scattered_idxs, expert_offsets, scattered, None, 1, True, False)
         d_x = torch.empty_like(x)
         ops.combine_rocm(scattered, None, d_x, top_k)
-        return d_x, d_w_fc, d_w_proj, d_router_weights, None, None
+        return d_x, d_w_fc, d_w_proj, d_router_weights, None, None, d_b_fc, d_b_proj, None
 
 
-def up_projection_experts(x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets):
-    return _UpProjectionExperts.apply(x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets)
+def up_projection_experts(x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, bias=None):
+    return _UpProjectionExperts.apply(x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, bias)
 
 
-def down_projection_experts(x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, router_weights):
+def down_projection_experts(x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, router_weights,
+                            bias=None):
     return _DownProjectionExperts.apply(
-        x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, router_weights
+        x, expert_weights, k, sorted_expert_idxs, sorted_scattered_idxs, expert_offsets, router_weights, bias
     )
 
 
-def fused_swiglu_experts(x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets):
-    return _FusedSwiGLUExperts.apply(x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets)
+def fused_swiglu_experts(x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets, b_fc=None, b_proj=None,
+                         save_activations=True):
+    """save_activations = False: the backward recomputes h and the expert outputs instead of keeping them, which frees
+    T k (H + I) elements per layer between forward and backward (Mixtral-shaped layer: 604 MB of 1.5 GB) for one more
+    down-projection GEMM."""
+    return _FusedSwiGLUExperts.apply(x, w_fc, w_proj, router_weights, sorted_scattered_idxs, expert_offsets, b_fc, b_proj,
+                                     save_activations)

@@ -31,6 +31,8 @@ SIGNATURES = {
     "xma_rocm_last_error": (ctypes.c_char_p, []),
     "xma_rocm_continuous_count_workspace_bytes": (_sz, [_i64, _i32]),
     "xma_rocm_continuous_count": (_int, [_p, _int, _i64, _p, _i32, _p, _sz, _p]),
+    "xma_rocm_continuous_count_set_workspace_bytes": (_sz, [_i64, _i32]),
+    "xma_rocm_continuous_count_set": (_int, [_p, _int, _i64, _p, _i32, _p, _sz, _p]),
     "xma_rocm_route_workspace_bytes": (_sz, [_i64, _i32]),
     "xma_rocm_route_set_rank_method": (_int, [_int]),
     "xma_rocm_route": (_int, [_p, _int, _i64, _i32, _p, _p, _p, _p, _p, _p, _sz, _p]),
@@ -42,6 +44,12 @@ SIGNATURES = {
         [_p, _i64, _p, _i64, _i64, _int, _p, _p, _p, _i64, _p, _i64, _p, _i64, _i32, _i32, _i32, _i32, _int, _int, _int, _int,
          _p, _sz, _p],
     ),
+    "xma_rocm_scatter2scatter_bias": (
+        _int,
+        [_p, _i64, _p, _i64, _i64, _int, _p, _p, _p, _i64, _p, _i64, _p, _p, _i64, _i64, _i32, _i32, _i32, _i32, _int, _int,
+         _int, _int, _p, _sz, _p],
+    ),
+    "xma_rocm_expert_column_sums": (_int, [_p, _i64, _p, _i32, _p, _p, _p, _i64, _i32, _i32, _int, _p]),
     "xma_rocm_down_projection_dx_swiglu": (
         _int,
         [_p, _i64, _p, _i64, _i64, _p, _p, _p, _i64, _p, _i64, _p, _i64, _p, _i64, _i32, _i32, _i32, _i32, _int,

@@ -81,6 +81,26 @@ def continuous_count_rocm(x: torch.Tensor, y: torch.Tensor, workspace: torch.Ten
     )
 
 
+CONTINUOUS_COUNT_SET_MAX_BINS = 8192
+
+
+@torch.library.custom_op("xma_rocm::continuous_count_set", mutates_args={"y"})
+def continuous_count_set_rocm(x: torch.Tensor, y: torch.Tensor) -> None:
+    """y (uint32, any contents) = histogram of x: the counts are written, not added to, so the caller allocates y with
+    torch.empty and no zero fill is launched (reference op: _continuous_count_cuda, which accumulates into torch.zeros,
+    continuous_count/__init__.py:41-45).  The scratch of large inputs is taken from torch's allocator inside the op."""
+    assert x.is_cuda and y.is_cuda and x.dim() == 1 and x.is_contiguous() and y.is_contiguous()
+    assert x.dtype in (torch.int32, torch.int64) and y.dtype == torch.uint32 and y.numel() <= CONTINUOUS_COUNT_SET_MAX_BINS
+    lib = get_library()
+    ws_bytes = lib.xma_rocm_continuous_count_set_workspace_bytes(x.numel(), y.numel())
+    workspace = torch.empty(ws_bytes // 4, dtype=torch.int32, device=x.device) if ws_bytes else None
+    check(
+        lib.xma_rocm_continuous_count_set(_ptr(x), int(x.dtype == torch.int64), x.numel(), _ptr(y), y.numel(), _ptr(workspace),
+                                          ws_bytes, _stream(x)),
+        "xma_rocm_continuous_count_set",
+    )
+
+
 # --------------------------------------------------------------------------- a2
 def route_workspace_elements(n: int, num_experts: int) -> int:
     return (get_library().xma_rocm_route_workspace_bytes(n, num_experts) + 3) // 4
@@ -135,8 +155,12 @@ def scatter2scatter_workspace_bytes(M: int, N: int, K: int, E: int, device_index
     return _S2S_WORKSPACE_BYTES[key]
 
 
-def _scatter2scatter(X, W, idx, offs, out, aux, scale, fan_out, x_grouped, y_grouped, epilogue, M, N, K):
+def _scatter2scatter(X, W, idx, offs, out, aux, scale, fan_out, x_grouped, y_grouped, epilogue, M, N, K, bias=None):
     w_is_kn, w_es, ldw = _weight_layout(W)
+    if bias is not None:  # (E, N): the experts' bias, the first term of every fp32 sum
+        assert bias.dtype == X.dtype and bias.shape == (W.size(0), N) and bias.is_cuda
+        assert bias.stride(1) == 1 and bias.stride(0) % 8 == 0 and bias.data_ptr() % 16 == 0, \
+            "bias rows should be contiguous, 16-byte aligned and a multiple of 8 elements apart"
     assert W.dtype == X.dtype
     assert idx.dtype == torch.int64 and idx.is_contiguous() and offs.dtype == torch.int64 and offs.is_contiguous()
     assert offs.numel() == W.size(0)
@@ -148,13 +172,13 @@ def _scatter2scatter(X, W, idx, offs, out, aux, scale, fan_out, x_grouped, y_gro
     ws_bytes = scatter2scatter_workspace_bytes(M, N, K, W.size(0), X.device.index or 0)
     workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=X.device) if ws_bytes else None
     check(
-        lib.xma_rocm_scatter2scatter(
+        lib.xma_rocm_scatter2scatter_bias(
             _ptr(X), _rows(X, "X"), _ptr(W), w_es, ldw, w_is_kn, _ptr(idx), _ptr(offs),
             _ptr(out), 0 if out is None else _rows(out, "out"), _ptr(aux), 0 if aux is None else _rows(aux, "aux"),
-            _ptr(scale), M, N, K, W.size(0), fan_out, int(x_grouped), int(y_grouped), epilogue, _code(X),
-            _ptr(workspace), ws_bytes, _stream(X),
+            _ptr(scale), _ptr(bias), 0 if bias is None else bias.stride(0), M, N, K, W.size(0), fan_out, int(x_grouped),
+            int(y_grouped), epilogue, _code(X), _ptr(workspace), ws_bytes, _stream(X),
         ),
-        "xma_rocm_scatter2scatter",
+        "xma_rocm_scatter2scatter_bias",
     )
 
 
@@ -169,14 +193,15 @@ def scatter2scatter_rocm(
     FAN_OUT: int,
     x_grouped: bool,
     y_grouped: bool,
+    bias: torch.Tensor | None = None,
 ) -> None:
-    """out[dst(n)] = X[src(n)] @ W[e(n)] (* row_scale[idx[n]]), W logically (E, K, N)."""
+    """out[dst(n)] = (bias[e(n)] + X[src(n)] @ W[e(n)]) (* row_scale[idx[n]]), W logically (E, K, N), bias (E, N) or None."""
     M = sorted_scattered_idxs.numel()
     E, K, N = W.shape
     assert X.size(1) == K and out.size(1) == N and out.size(0) == M
     assert X.size(0) * (1 if x_grouped else FAN_OUT) == M
     _scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, out, None, row_scale, FAN_OUT, x_grouped, y_grouped,
-                     EPI_STORE, M, N, K)
+                     EPI_STORE, M, N, K, bias)
 
 
 @torch.library.custom_op("xma_rocm::up_projection_swiglu", mutates_args={"z", "h"})
@@ -188,13 +213,14 @@ def up_projection_swiglu_rocm(
     z: torch.Tensor,
     h: torch.Tensor,
     FAN_OUT: int,
+    bias: torch.Tensor | None = None,
 ) -> None:
-    """z (grouped pre-activations, (Tk, 2I)) and h = swiglu_packed(z) (Tk, I) in one GEMM."""
+    """z (grouped pre-activations, (Tk, 2I), bias (E, 2I) included) and h = swiglu_packed(z) (Tk, I) in one GEMM."""
     M = sorted_scattered_idxs.numel()
     E, K, N = W.shape
     assert X.size(1) == K and X.size(0) * FAN_OUT == M
     assert z.shape == (M, N) and h.shape == (M, N // 2) and N % 2 == 0
-    _scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, z, h, None, FAN_OUT, False, True, EPI_SWIGLU, M, N, K)
+    _scatter2scatter(X, W, sorted_scattered_idxs, expert_offsets, z, h, None, FAN_OUT, False, True, EPI_SWIGLU, M, N, K, bias)
 
 
 @torch.library.custom_op("xma_rocm::down_projection_dx_swiglu", mutates_args={"dz"})
@@ -284,6 +310,32 @@ def group_bwd_W_rocm(
             N_out, K_in, E, _code(X), _stream(X),
         ),
         "xma_rocm_group_bwd_W",
+    )
+
+
+@torch.library.custom_op("xma_rocm::expert_column_sums", mutates_args={"out"})
+def expert_column_sums_rocm(
+    A: torch.Tensor,
+    sorted_scattered_idxs: torch.Tensor | None,
+    expert_offsets: torch.Tensor,
+    out: torch.Tensor,
+    row_scale: torch.Tensor | None,
+    fan_out: int,
+) -> None:
+    """out[e] = sum over the grouped rows n of expert e of A[src(n)] * row_scale[idx[n]], src(n) = n when no index is given,
+    else idx[n] // fan_out: the gradient of the experts' bias (autograd of F.linear's bias, moe/__init__.py:96-100)."""
+    E, N = out.shape
+    assert A.size(1) == N and A.dtype == out.dtype and expert_offsets.numel() == E and expert_offsets.dtype == torch.int64
+    assert out.stride(1) == 1 and expert_offsets.is_contiguous()
+    if sorted_scattered_idxs is not None:
+        assert sorted_scattered_idxs.dtype == torch.int64 and sorted_scattered_idxs.is_contiguous()
+    if row_scale is not None:
+        assert row_scale.dtype == A.dtype and row_scale.is_contiguous() and sorted_scattered_idxs is not None
+    lib = get_library()
+    check(
+        lib.xma_rocm_expert_column_sums(_ptr(A), _rows(A, "A"), _ptr(sorted_scattered_idxs), max(fan_out, 1), _ptr(row_scale),
+                                        _ptr(expert_offsets), _ptr(out), _rows(out, "out"), N, E, _code(A), _stream(A)),
+        "xma_rocm_expert_column_sums",
     )
 
 

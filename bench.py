@@ -1,6 +1,6 @@
 """MoE hot-path benchmark on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c5|c2|copy|mfma_peak|library_gemm]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c5|c2|small_t|copy|mfma_peak|library_gemm]
 
 Default workload: the Mixtral-shaped layer (T=8192, H=4096, I=14336, E=8, top-2, packed SwiGLU, bf16).
 A step is one forward + backward of the layer behind the gate: router (top-k + softmax + expert ids from the
@@ -384,11 +384,10 @@ def measure_routing(args, zipf, cpu_baseline=True):
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
 
     y = torch.zeros(E, dtype=torch.uint32, device="cuda")
-    hws = torch.empty(ops.continuous_count_workspace_elements(n, E), dtype=torch.int32, device="cuda")
 
-    def hist():
+    def hist():  # what the public functional runs: output from torch.empty, counts written by the kernels
         it[0] += 1
-        ops.continuous_count_rocm(bufs[it[0] % nbuf], y, hws)
+        continuous_count(bufs[it[0] % nbuf], E, kernel_backend=KernelBackend.rocm)
 
     def graph_ms(call, reps=20):
         """per-call time of `call(buffer)` replayed from one graph that holds a call per input buffer: GPU time without the
@@ -406,9 +405,9 @@ def measure_routing(args, zipf, cpu_baseline=True):
         return _time_gpu(g_.replay, reps, warmup=3) / len(bufs)
 
     route_graph_ms = graph_ms(lambda b: R.route(b, E))
-    hist_graph_ms = graph_ms(lambda b: ops.continuous_count_rocm(b, y, hws))
+    hist_graph_ms = graph_ms(lambda b: ops.continuous_count_set_rocm(b, y))
     hist_ms = _time_gpu(hist, args.kernel_iters * 10, warmup=5)
-    hist_warm_ms = _time_gpu(lambda: ops.continuous_count_rocm(bufs[0], y, hws), args.kernel_iters * 10, warmup=5)
+    hist_warm_ms = _time_gpu(lambda: ops.continuous_count_set_rocm(bufs[0], y), args.kernel_iters * 10, warmup=5)
     route_ms = _time_gpu(step, args.kernel_iters * 5, warmup=5)
     hist_bytes = n * 4 + E * 4
     route_bytes = n * 4 + n * 8 + n * 4 + E * 20
@@ -430,6 +429,17 @@ def measure_routing(args, zipf, cpu_baseline=True):
     copy_ms = ref_graph_ms(lambda i: halves[i].copy_(halves[(i + 1) % nbuf]))
     read_ms = ref_graph_ms(lambda i: halves[0][:64].copy_(bufs[i].view(torch.uint8)[:64]))  # launch floor of one kernel
     del outs, halves
+    # the same kernels with the launch cost amortised: 64 Mi ids (16 times the configuration), two alternating buffers
+    big_n = 64 * 1024 * 1024
+    big = [torch.randint(0, E, (big_n,), dtype=torch.int32, device="cuda") for _ in range(2)]
+    if zipf:
+        for b in big:
+            b.copy_(torch.multinomial((p / p.sum()).cuda().float(), big_n, replacement=True).to(torch.int32))
+    big_y = torch.empty(E, dtype=torch.uint32, device="cuda")
+    big_route_ms = _time_gpu(lambda: (it.__setitem__(0, it[0] + 1), R.route(big[it[0] % 2], E)), 10, warmup=2)
+    big_hist_ms = _time_gpu(lambda: (it.__setitem__(0, it[0] + 1), ops.continuous_count_set_rocm(big[it[0] % 2], big_y)), 10, warmup=2)
+    del big
+    torch.cuda.empty_cache()
     reps, dt = 3, None
     if cpu_baseline and not args.no_cpu_baseline:
         t1 = time.perf_counter()
@@ -480,6 +490,10 @@ def measure_routing(args, zipf, cpu_baseline=True):
                 "ms": round(copy_ms, 5), "gbs": round(route_bytes / copy_ms / 1e6, 1),
                 "frac_hbm_peak": round(route_bytes / copy_ms / 1e6 / PEAK_HBM_GBS, 4)},
             "one 64-byte copy kernel [graph]": {"ms": round(read_ms, 5)},
+            "route_64Mi_ids": {"ms": round(big_route_ms, 5), "gbs": round(route_bytes * 16 / big_route_ms / 1e6, 1),
+                               "frac_hbm_peak": round(route_bytes * 16 / big_route_ms / 1e6 / PEAK_HBM_GBS, 4)},
+            "continuous_count_64Mi_ids": {"ms": round(big_hist_ms, 5), "gbs": round(big_n * 4 / big_hist_ms / 1e6, 1),
+                                          "frac_hbm_peak": round(big_n * 4 / big_hist_ms / 1e6 / PEAK_HBM_GBS, 4)},
         },
     }
     del bufs
@@ -510,9 +524,71 @@ def _other_configs(args) -> dict:
                       "continuous_count_graph_us": round(k["continuous_count_graph"]["ms"] * 1e3, 2),
                       "continuous_count_frac_hbm": k["continuous_count_graph"]["frac_hbm_peak"],
                       "continuous_count_op_us": round(k["continuous_count_cold"]["ms"] * 1e3, 2),
-                      "route_op_us": round(k["route"]["ms"] * 1e3, 2)}
+                      "route_op_us": round(k["route"]["ms"] * 1e3, 2),
+                      "route_64Mi_frac_hbm": k["route_64Mi_ids"]["frac_hbm_peak"],
+                      "continuous_count_64Mi_frac_hbm": k["continuous_count_64Mi_ids"]["frac_hbm_peak"]}
     args.steps, args.warmup = saved
     return res
+
+
+def run_small_t(args):
+    """Latency of one forward + backward of the expert computation with a handful of tokens, the case the reference's
+    own test runs (7 tokens, tests/layers/moe_test.py:107) at its two size points (moe_test.py:26-53), and with 64
+    tokens: eager, and replayed from a HIP graph (no host launch overhead), beside the time the weights touched by the
+    step need to stream through HBM once per use at 8 TB/s (forward, dX and the dW store: three uses)."""
+    from xma import KernelBackend, set_seed
+    from xma.functional import swiglu_packed
+    from xma.layers import MoE
+    from xma.layers.moe import rocm_implementation as R
+
+    res = {}
+    for E, k, H, I in ((8, 2, 2048, 8192), (128, 8, 576, 256)):
+        set_seed(0)
+        moe = MoE(E, k, H, I, swiglu_packed, True, add_bias=False, std=0.02).to(torch.bfloat16).cuda()
+        for T in (7, 64):
+            x = torch.randn(T, H, device="cuda").to(torch.bfloat16).requires_grad_()
+            lg = torch.randn(T, E, device="cuda").to(torch.bfloat16).requires_grad_()
+            grad = torch.randn(T, H, device="cuda").to(torch.bfloat16)
+
+            def step():
+                for p_ in moe.parameters():
+                    p_.grad = None
+                x.grad = None
+                lg.grad = None
+                w, ids = R.router_topk(lg, k, ids_dtype=torch.int32)
+                y = moe._compute_experts(x, w, ids, kernel_backend=KernelBackend.rocm)
+                y.backward(grad)
+
+            eager_ms = _time_gpu(step, max(args.steps, 20), warmup=5)
+            side = torch.cuda.Stream()
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):
+                step()
+            torch.cuda.current_stream().wait_stream(side)
+            torch.cuda.synchronize()
+            g_ = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g_):
+                step()
+            graph_ms = _time_gpu(g_.replay, max(args.steps, 20), warmup=5)
+            _, sel = R.router_topk(lg.detach(), k)
+            touched = int(torch.unique(sel).numel())
+            wbytes = (2 * I * H + H * I) * 2  # both matrices of one expert
+            stream_bytes = 2 * touched * wbytes + E * wbytes  # forward and dX read the touched experts, dW writes all
+            res[f"E{E}_k{k}_H{H}_I{I}_T{T}"] = {
+                "eager_ms": round(eager_ms, 4), "graph_ms": round(graph_ms, 4), "experts_touched": touched,
+                "weight_stream_ms_at_8TBs": round(stream_bytes / PEAK_HBM_GBS / 1e6, 4),
+                "graph_over_stream": round(graph_ms / (stream_bytes / PEAK_HBM_GBS / 1e6), 2),
+            }
+        del moe
+        torch.cuda.empty_cache()
+    first = next(iter(res.values()))
+    print(json.dumps({"metric": "moe_small_t_fwd_bwd_latency_ms", "value": first["graph_ms"], "unit": "ms", "n_gpus": 1,
+                      "steps": args.steps, "warmup": args.warmup, "ms_per_step": first["graph_ms"], "higher_is_better": False,
+                      "dtype": "bf16", "data": "synthetic",
+                      "config": {"workload": "small_t: expert computation fwd+bwd (router top-k from given logits, routing, "
+                                             "experts, combine and all gradients) at T = 7 and 64 on the reference test's two "
+                                             "size points, bf16 packed SwiGLU"},
+                      "results": res}))
 
 
 def run_copy(args):
@@ -598,7 +674,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "copy", "mfma_peak", "library_gemm"])
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "small_t", "copy", "mfma_peak", "library_gemm"])
     ap.add_argument("--zipf", action="store_true", help="c2 only: Zipf(s=1.1) ids instead of uniform")
     ap.add_argument("--kernel-iters", type=int, default=5)
     ap.add_argument("--cpu-fraction", type=int, default=1, help="CPU baseline runs on T / this many tokens")
@@ -618,6 +694,8 @@ def main():
         run_mfma_peak(args)
     elif args.workload == "library_gemm":
         run_library_gemm(args)
+    elif args.workload == "small_t":
+        run_small_t(args)
     elif args.workload == "c2":
         print(json.dumps(measure_routing(args, args.zipf)))
     else:

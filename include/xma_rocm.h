@@ -4,8 +4,9 @@
  *
  * Conventions
  *   - every pointer is a DEVICE pointer owned by the caller (PyTorch's caching
- *     allocator in the Python host); the library allocates nothing and keeps no
- *     state between calls;
+ *     allocator in the Python host); the library allocates nothing.  What it keeps between calls: per-device
+ *     constants looked up once (compute units, a kernel's raised LDS limit, the address of xma_rocm_route_static's
+ *     scratch) and one process-wide switch, xma_rocm_route_set_rank_method;
  *   - `stream` is a hipStream_t passed as void*; all work is enqueued on it and
  *     no entry point synchronises;
  *   - return value 0 = enqueued, negative = XMA_ROCM_E* (argument errors are
@@ -65,6 +66,17 @@ XMA_API const char *xma_rocm_last_error(void);
 XMA_API size_t xma_rocm_continuous_count_workspace_bytes(int64_t n, int32_t bins);
 XMA_API int xma_rocm_continuous_count(const void *ids, int ids_are_int64, int64_t n, uint32_t *counts, int32_t bins,
                                       void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * The same histogram with counts OVERWRITTEN instead of added to, so that the caller need not clear them (one launch
+ * less per call): counts[b] = #{i : ids[i] == b}, b < bins <= 8192, ids outside the range ignored, n == 0 gives zeros.
+ * Inputs of more than 4096 ids need xma_rocm_continuous_count_set_workspace_bytes(n, bins) bytes of workspace.
+ * Same reference interface as xma_rocm_continuous_count (there the caller's torch.zeros, cuda_implementation.py callers
+ * at xma/functional/continuous_count/__init__.py:41-45, is a launch of its own).
+ */
+XMA_API size_t xma_rocm_continuous_count_set_workspace_bytes(int64_t n, int32_t bins);
+XMA_API int xma_rocm_continuous_count_set(const void *ids, int ids_are_int64, int64_t n, uint32_t *counts, int32_t bins,
+                                  void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * Routing in one op: counts, inclusive/exclusive expert offsets and the STABLE
@@ -133,6 +145,32 @@ XMA_API int xma_rocm_scatter2scatter(const void *X, int64_t ldx, const void *W, 
                              int32_t N, int32_t K, int32_t num_experts, int32_t fan_out, int x_grouped,
                              int y_grouped, int epilogue, int dtype, void *workspace,
                              size_t workspace_bytes, void *stream);
+
+/*
+ * xma_rocm_scatter2scatter with the experts' bias: acc[n, :] = bias[e(n), :N] + X[src(n), :K] @ B_e, the bias being the
+ * first term of the fp32 sum (one rounding, like a linear layer with a bias), then the epilogue; a row scale multiplies
+ * the biased row.  bias (E, N) with `bias_expert_stride` elements between experts (a multiple of 8), 16-byte aligned,
+ * NULL = no bias; STORE and SWIGLU epilogues.  Covers the bias of Experts that the reference applies on its torch path
+ * only, F.linear(x[e], weight[e], bias[e]) in xma/layers/moe/__init__.py:96-100 (its Triton path asserts there is none,
+ * :53 and :75).
+ */
+XMA_API int xma_rocm_scatter2scatter_bias(const void *X, int64_t ldx, const void *W, int64_t w_expert_stride, int64_t ldw,
+                                  int w_is_kn, const int64_t *sorted_scattered_idxs, const int64_t *expert_offsets,
+                                  void *out, int64_t ldo, void *aux, int64_t ldaux, const void *row_scale,
+                                  const void *bias, int64_t bias_expert_stride, int64_t M, int32_t N, int32_t K,
+                                  int32_t num_experts, int32_t fan_out, int x_grouped, int y_grouped, int epilogue,
+                                  int dtype, void *workspace, size_t workspace_bytes, void *stream);
+
+/*
+ * Gradient of the experts' bias: out[e, :N] = sum over the grouped rows n of expert e of A[src(n), :N] * scale, with
+ * src(n) = n (sorted_scattered_idxs == NULL) or sorted_scattered_idxs[n] / fan_out, scale = row_scale[idx[n]] or 1.
+ * fp32 sums in a fixed order; experts without rows get zeros; every element of out (E, N; row stride ldo) is written.
+ * Replaces what autograd derives for the bias of F.linear in the reference's torch path
+ * (xma/layers/moe/__init__.py:96-100).  N and the leading dimensions even, 8-byte aligned bases.
+ */
+XMA_API int xma_rocm_expert_column_sums(const void *A, int64_t lda, const int64_t *sorted_scattered_idxs, int32_t fan_out,
+                                const void *row_scale, const int64_t *expert_offsets, void *out, int64_t ldo, int32_t N,
+                                int32_t num_experts, int dtype, void *stream);
 
 /*
  * dX of the down-projection with the SwiGLU backward in the epilogue (xma_rocm_scatter2scatter with

@@ -122,6 +122,8 @@ def experts_forward_backward(
     act: Callable[[torch.Tensor], torch.Tensor],
     grad_out: torch.Tensor,
     compute_dtype: torch.dtype | None = None,
+    b_fc: torch.Tensor | None = None,
+    b_proj: torch.Tensor | None = None,
 ) -> dict[str, torch.Tensor]:
     """Forward and stock-autograd backward of ``experts_forward`` for an
     upstream gradient ``grad_out`` (the reference test uses ones,
@@ -131,9 +133,16 @@ def experts_forward_backward(
     cd = compute_dtype or x.dtype
     leaves = [t.detach().to(cd).clone().requires_grad_() for t in (x, router_weights, w_fc, w_proj)]
     xx, rw, w1, w2 = leaves
-    y = experts_forward(xx, rw, selected_experts, w1, w2, act)
+    b1 = None if b_fc is None else b_fc.detach().to(cd).clone().requires_grad_()
+    b2 = None if b_proj is None else b_proj.detach().to(cd).clone().requires_grad_()
+    y = experts_forward(xx, rw, selected_experts, w1, w2, act, b1, b2)
     y.backward(grad_out.to(cd))
-    return {"y": y.detach(), "dx": xx.grad, "d_router_weights": rw.grad, "dw_fc": w1.grad, "dw_proj": w2.grad}
+    out = {"y": y.detach(), "dx": xx.grad, "d_router_weights": rw.grad, "dw_fc": w1.grad, "dw_proj": w2.grad}
+    if b1 is not None:  # an expert without rows never enters the graph: its bias gradient is zero
+        out["db_fc"] = b1.grad if b1.grad is not None else torch.zeros_like(b1)
+    if b2 is not None:
+        out["db_proj"] = b2.grad if b2.grad is not None else torch.zeros_like(b2)
+    return out
 
 
 def normalised_max_error(got: torch.Tensor, want: torch.Tensor) -> float:
@@ -157,9 +166,11 @@ def scatter2scatter(
     y_grouped: bool,
     row_scale: torch.Tensor | None = None,
     compute_dtype: torch.dtype = torch.float32,
+    bias: torch.Tensor | None = None,  # (E, N)
 ) -> torch.Tensor:
     """out[dst(n)] = X[src(n)] @ W[e(n)] with src(n) = n or idx[n] // fan_out and dst(n) = n or idx[n]
-    (xma/layers/moe/triton_implementation/scatter_kernel.py:58-134: row selection :105-108, store :128-134)."""
+    (xma/layers/moe/triton_implementation/scatter_kernel.py:58-134: row selection :105-108, store :128-134); with
+    `bias`, the expert's bias row is added to the product as F.linear adds it (xma/layers/moe/__init__.py:96-100)."""
     M = sorted_scattered_idxs.numel()
     N = W.shape[-1]
     out = torch.zeros(M, N, dtype=compute_dtype)
@@ -170,6 +181,8 @@ def scatter2scatter(
         src = n if x_grouped else s // fan_out
         dst = n if y_grouped else s
         v = Xc[src] @ Wc[e]
+        if bias is not None:
+            v = v + bias[e].to(compute_dtype)
         if row_scale is not None:
             v = v * row_scale[s].to(compute_dtype)
         out[dst] = v

@@ -29,14 +29,21 @@ def _oracle_act(name):
     return {"swiglu_packed": oracle.swiglu_packed, "glu": nn.GLU(), "gelu": nn.GELU(approximate="tanh")}[name]
 
 
-def _run_case(dtype, T, E, k, H, I, act_name, skew=0.0, empty=(), seed=42):
+def _run_case(dtype, T, E, k, H, I, act_name, skew=0.0, empty=(), seed=42, add_bias=False, save_activations=True):
     from xma import KernelBackend, set_seed
     from xma.layers import MoE
 
     print(f"case {dtype} T={T} E={E} k={k} H={H} I={I} act={act_name} skew={skew} empty={empty}", flush=True)
     set_seed(seed)
     is_glu = act_name != "gelu"
-    moe = MoE(E, k, H, I, _act(act_name), is_glu, add_bias=False, std=0.02).to(dtype)
+    moe = MoE(E, k, H, I, _act(act_name), is_glu, add_bias=add_bias, std=0.02).to(dtype)
+    moe.save_activations = save_activations
+    b_fc = b_proj = None
+    if add_bias:  # the module zero-fills its biases; the test wants values that matter
+        with torch.no_grad():
+            moe.c_fc.bias.copy_((torch.randn(moe.c_fc.bias.shape) * 0.5).to(dtype))
+            moe.c_proj.bias.copy_((torch.randn(moe.c_proj.bias.shape) * 0.5).to(dtype))
+        b_fc, b_proj = moe.c_fc.bias.data, moe.c_proj.bias.data
     x = torch.randn(T, H).to(dtype)
     logits = torch.randn(T, E) + skew * torch.randn(E)
     for e in empty:
@@ -45,7 +52,8 @@ def _run_case(dtype, T, E, k, H, I, act_name, skew=0.0, empty=(), seed=42):
     grad = torch.randn(T, H).to(dtype)
 
     want = oracle.experts_forward_backward(
-        x, rw, sel, moe.c_fc.weight.data, moe.c_proj.weight.data, _oracle_act(act_name), grad, compute_dtype=torch.float32
+        x, rw, sel, moe.c_fc.weight.data, moe.c_proj.weight.data, _oracle_act(act_name), grad, compute_dtype=torch.float32,
+        b_fc=b_fc, b_proj=b_proj,
     )
 
     moe = moe.cuda()
@@ -56,6 +64,8 @@ def _run_case(dtype, T, E, k, H, I, act_name, skew=0.0, empty=(), seed=42):
     torch.cuda.synchronize()
 
     got = {"y": y, "dx": xd.grad, "d_router_weights": rwd.grad, "dw_fc": moe.c_fc.weight.grad, "dw_proj": moe.c_proj.weight.grad}
+    if add_bias:
+        got["db_fc"], got["db_proj"] = moe.c_fc.bias.grad, moe.c_proj.bias.grad
     for name, w in want.items():
         g = got[name]
         assert g is not None and g.dtype == dtype and g.shape == w.shape, name
@@ -99,6 +109,49 @@ def test_moe_tiles_split_along_k(act_name):
     up, in all three epilogues (up-projection K = H, dX2 K = H, down-projection K = I, dX1 K = 2 I)."""
     _run_case(torch.bfloat16, 64, 2, 1, 1024, 1536, act_name)
     _run_case(torch.float16, 300, 3, 2, 2048, 512, act_name, skew=1.0)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("act_name", ["swiglu_packed", "glu", "gelu"])
+def test_moe_with_expert_biases(dtype, act_name):
+    """add_bias=True: Experts.bias (E, out) on both projections, as the reference's torch path applies it
+    (F.linear(x[e], weight[e], bias[e]), moe/__init__.py:96-100), forward and all gradients including the two biases'
+    against the fp32 oracle: the reference's 7-token shape, ragged routing with empty experts (their bias gradient is
+    zero), top-4 (dW2 and the down-projection's bias gradient from unscaled dy through the index) and tiles split along K."""
+    _run_case(dtype, 7, 8, 2, 512, 1024, act_name, add_bias=True)
+    _run_case(dtype, 777, 16, 4, 264, 136, act_name, skew=2.0, empty=(0, 15), add_bias=True)
+    _run_case(dtype, 1500, 8, 2, 256, 384, act_name, skew=1.5, empty=(2,), add_bias=True)
+    _run_case(dtype, 300, 3, 2, 2048, 512, act_name, skew=1.0, add_bias=True)
+
+
+@pytest.mark.parametrize("k", [2, 4])
+def test_moe_recomputed_activations(k):
+    """save_activations = False: the backward recomputes h and the expert outputs from the kept pre-activations; the
+    results are those of the default path bit for bit (same kernels on the same operands), and within tolerance of the
+    oracle, with and without biases."""
+    from xma import KernelBackend, set_seed
+    from xma.layers import MoE
+
+    _run_case(torch.bfloat16, 777, 16, k, 264, 136, "swiglu_packed", skew=2.0, empty=(0, 15), save_activations=False)
+    _run_case(torch.bfloat16, 300, 8, k, 512, 256, "swiglu_packed", add_bias=True, save_activations=False)
+    set_seed(5)
+    T, E, H, I = 900, 8, 256, 384
+    moe = MoE(E, k, H, I, _act("swiglu_packed"), True, add_bias=False, std=0.02).to(torch.bfloat16).cuda()
+    x = torch.randn(T, H, device="cuda").to(torch.bfloat16)
+    rw, sel = oracle.routing_weights(torch.randn(T, E, device="cuda"), k, torch.bfloat16)
+    grad = torch.randn(T, H, device="cuda").to(torch.bfloat16)
+    res = []
+    for keep in (True, False):
+        moe.save_activations = keep
+        for p in moe.parameters():
+            p.grad = None
+        xd, rwd = x.clone().requires_grad_(), rw.clone().requires_grad_()
+        y = moe._compute_experts(xd, rwd, sel, kernel_backend=KernelBackend.rocm)
+        y.backward(grad)
+        torch.cuda.synchronize()
+        res.append([t.clone() for t in (y.detach(), xd.grad, rwd.grad, moe.c_fc.weight.grad, moe.c_proj.weight.grad)])
+    for a, b, name in zip(res[0], res[1], ("y", "dx", "d_router_weights", "dw_fc", "dw_proj")):
+        assert torch.equal(a, b), name
 
 
 def test_moe_plumbing_config_shape():

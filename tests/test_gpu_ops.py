@@ -126,6 +126,55 @@ def test_scatter2scatter_launches_outside_the_persistent_kernel():
     assert nerr(z, want_z) <= TOL and nerr(h, want_h) <= TOL
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+def test_scatter2scatter_bias_and_expert_column_sums(dtype):
+    """The experts' bias as the first term of the grouped GEMM's sums (plain store and SwiGLU epilogues, both weight
+    layouts, with and without a row scale, a tile split along K), and its gradient, the per-expert column sums of grouped
+    rows or of gathered and scaled rows; experts without rows give zero sums."""
+    from xma.rocm import ops
+
+    for T, E, k, K, N, skew, empty in [(300, 3, 2, 192, 320, 0.0, ()), (513, 6, 4, 72, 40, 2.0, (0, 5)), (300, 3, 2, 1096, 320, 0.0, ())]:
+        print(f"bias case T={T} E={E} k={k} K={K} N={N} {dtype}", flush=True)
+        sel, se, ss, offs = _routing(T, E, k, 3, skew, empty)
+        g = torch.Generator().manual_seed(4)
+        M = T * k
+        X = torch.randn(T, K, generator=g).to(dtype)
+        bias = torch.randn(E, N, generator=g).to(dtype)
+        scale = torch.rand(M, generator=g).to(dtype)
+        for w_kn in (False, True):
+            W = (torch.randn(E, K, N, generator=g) * 0.1).to(dtype)
+            Wd = W.cuda() if w_kn else W.permute(0, 2, 1).contiguous().cuda().permute(0, 2, 1)
+            for rs in (None, scale):
+                want = oracle.scatter2scatter(X, W, se, ss, k, False, True, rs, bias=bias)
+                out = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+                ops.scatter2scatter_rocm(X.cuda(), Wd, ss.cuda(), offs.cuda(), out, None if rs is None else rs.cuda(), k, False,
+                                         True, bias.cuda())
+                torch.cuda.synchronize()
+                assert torch.isfinite(out).all() and nerr(out, want) <= _tol(dtype), (w_kn, rs is None)
+            if not w_kn and N % 16 == 0:
+                want_z = oracle.scatter2scatter(X, W, se, ss, k, False, True, None, bias=bias)
+                z = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+                h = torch.full((M, N // 2), float("nan"), dtype=dtype, device="cuda")
+                ops.up_projection_swiglu_rocm(X.cuda(), Wd, ss.cuda(), offs.cuda(), z, h, k, bias.cuda())
+                torch.cuda.synchronize()
+                assert nerr(z, want_z) <= _tol(dtype) and nerr(h, oracle.swiglu_packed(want_z)) <= _tol(dtype)
+        # column sums: grouped rows; gathered rows times a scale
+        A = torch.randn(M, N, generator=g).to(dtype)
+        counts = torch.bincount(se, minlength=E).tolist()
+        want = torch.stack([a.float().sum(0) for a in A.split(counts)])
+        got = torch.full((E, N), float("nan"), dtype=dtype, device="cuda")
+        ops.expert_column_sums_rocm(A.cuda(), None, offs.cuda(), got, None, 1)
+        B = torch.randn(T, N, generator=g).to(dtype)
+        rows = B.float()[ss // k] * scale.float()[ss][:, None]
+        want2 = torch.stack([a.sum(0) for a in rows.split(counts)])
+        got2 = torch.full((E, N), float("nan"), dtype=dtype, device="cuda")
+        ops.expert_column_sums_rocm(B.cuda(), ss.cuda(), offs.cuda(), got2, scale.cuda(), k)
+        torch.cuda.synchronize()
+        assert nerr(got, want) <= _tol(dtype) and nerr(got2, want2) <= _tol(dtype)
+        for e in empty:
+            assert torch.count_nonzero(got[e]) == 0 and torch.count_nonzero(got2[e]) == 0
+
+
 def _routing_with_counts(counts, k, seed):
     """a routing whose experts own exactly `counts` rows (sum divisible by k): the slots are dealt out at random"""
     g = torch.Generator().manual_seed(seed)

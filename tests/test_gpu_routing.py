@@ -55,6 +55,24 @@ def test_continuous_count_edge_cases():
     assert continuous_count(z, 4, kernel_backend=_kb()).tolist() == [1, 1, 0, 2]
 
 
+def test_continuous_count_overwrites_or_accumulates():
+    """The two histogram ops behind the functional: continuous_count_set writes the counts whatever the output held
+    (one workgroup for up to 4096 ids, per-unit histograms plus a storing reduction beyond), continuous_count adds to
+    what the caller put there, as the reference's kernel does (cuda_implementation.py:139-145)."""
+    from xma.rocm import ops
+
+    for n in (0, 1, 4096, 4097, 70000, 300000):
+        ids = torch.randint(0, 72, (n,), device="cuda", dtype=torch.int32)
+        want = oracle.continuous_count(ids.cpu().numpy(), 72)
+        y = torch.full((72,), -559038737, dtype=torch.int32, device="cuda").view(torch.uint32)
+        ops.continuous_count_set_rocm(ids, y)
+        assert np.array_equal(np_of(y), want), n
+        acc = torch.zeros(72, dtype=torch.uint32, device="cuda")
+        ops.continuous_count_rocm(ids, acc, None)
+        ops.continuous_count_rocm(ids, acc, None)
+        assert np.array_equal(np_of(acc), 2 * want), n
+
+
 @pytest.mark.parametrize("dist", ["uniform", "zipf", "sorted"])
 @pytest.mark.parametrize("dtype", [torch.int32, torch.int64])
 def test_continuous_count_4m(dist, dtype):

@@ -130,6 +130,43 @@ def test_per_token_brute_force():
     assert torch.allclose(y, want, rtol=1e-10, atol=1e-12)
 
 
+def test_biases_per_token_brute_force_and_their_gradients():
+    """Experts.bias as the torch path applies it (moe/__init__.py:96-100): z = W1[e] x + b1[e], out = W2[e] h + b2[e].
+    Forward against a per-token loop; the bias gradients against their closed forms - db2[e] = sum over the (token, slot)
+    pairs routed to e of w * dy[token], db1[e] = sum of dz over the expert's rows (by finite differences) - and zero for
+    an expert that no token selects."""
+    x, rw, sel, w1, w2 = _random_case(10, 4, 2, 6, 5, seed=4)
+    sel = sel.clamp(max=2)  # expert 3 never selected
+    g = torch.Generator().manual_seed(9)
+    b1 = torch.randn(4, 10, generator=g, dtype=torch.float64)
+    b2 = torch.randn(4, 6, generator=g, dtype=torch.float64)
+    y = oracle.experts_forward(x, rw, sel, w1, w2, oracle.swiglu_packed, b1, b2)
+    want = torch.zeros_like(x)
+    for t in range(10):
+        for j in range(2):
+            e = int(sel[t, j])
+            z = w1[e] @ x[t] + b1[e]
+            h = torch.stack([z[2 * c + 1] * z[2 * c] / (1 + torch.exp(-z[2 * c])) for c in range(5)])
+            want[t] += rw[t, j] * (w2[e] @ h + b2[e])
+    assert torch.allclose(y, want, rtol=1e-10, atol=1e-12)
+    dy = torch.randn(10, 6, generator=g, dtype=torch.float64)
+    out = oracle.experts_forward_backward(x, rw, sel, w1, w2, oracle.swiglu_packed, dy, b_fc=b1, b_proj=b2)
+    want_db2 = torch.zeros(4, 6, dtype=torch.float64)
+    for t in range(10):
+        for j in range(2):
+            want_db2[int(sel[t, j])] += rw[t, j] * dy[t]
+    assert torch.allclose(out["db_proj"], want_db2, rtol=1e-10, atol=1e-12)
+    assert (out["db_fc"][3] == 0).all() and (out["db_proj"][3] == 0).all() and out["db_fc"][:3].abs().sum() > 0
+    eps = 1e-6
+    for e, c in ((0, 0), (1, 3), (2, 9)):
+        bp, bm = b1.clone(), b1.clone()
+        bp[e, c] += eps
+        bm[e, c] -= eps
+        fd = ((oracle.experts_forward(x, rw, sel, w1, w2, oracle.swiglu_packed, bp, b2) -
+               oracle.experts_forward(x, rw, sel, w1, w2, oracle.swiglu_packed, bm, b2)) * dy).sum() / (2 * eps)
+        assert abs(float(fd) - float(out["db_fc"][e, c])) <= 1e-6 * max(1.0, abs(float(fd)))
+
+
 def test_backward_gradcheck_and_empty_expert():
     x, rw, sel, w1, w2 = _random_case(6, 4, 2, 4, 3, seed=5)
     sel = sel.clamp(max=2)  # expert 3 never selected; duplicates inside a token are allowed by the math
