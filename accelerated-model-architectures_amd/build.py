@@ -172,11 +172,13 @@ def build(verbose: bool = False) -> str:
 TIMING_LIB = os.path.join(OUT_DIR, "libxma_rocm_timing.so")
 
 
-def build_timing(verbose: bool = False) -> str:
+def build_timing(verbose: bool = False, rebuild: bool = True) -> str:
     """A second library for diagnostics/tile_phases.py: grouped_gemm.hip compiled with -DXMA_PST_TIMING (the persistent
-    GEMM kernel stamps the real-time counter at six points of every tile), linked with the objects of the normal build.
+    GEMM kernel stamps the real-time counter and the shader clock counter at six points of every tile and behind every K
+    step of one tile), linked with the objects of the normal build (rebuild=False: those of the last build()).
     Not part of build(): nothing in the product loads it."""
-    build(verbose)
+    if rebuild:
+        build(verbose)
     obj, _ = _compile("grouped_gemm.hip", verbose, ("-DXMA_PST_TIMING",), "_timing")
     objs = [obj if s == "grouped_gemm.hip" else os.path.join(HERE, "build", s.replace(".hip", ".o")) for s in SOURCES]
     r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", TIMING_LIB, *objs], capture_output=True, text=True)
@@ -186,4 +188,7 @@ def build_timing(verbose: bool = False) -> str:
 
 
 if __name__ == "__main__":
-    print(build_timing(verbose=True) if "--timing" in sys.argv[1:] else build(verbose=True))
+    if "--timing-only" in sys.argv[1:]:
+        print(build_timing(verbose=True, rebuild=False))
+    else:
+        print(build_timing(verbose=True) if "--timing" in sys.argv[1:] else build(verbose=True))

@@ -289,6 +289,33 @@ __device__ __forceinline__ void add_bias(const FwdArgs &a, f32x16 (&acc)[4][4], 
         for (int i = 0; i < 4; ++i) acc[j][i] = Elem<T>::mfma(p[j], q, acc[j][i]);
 }
 
+// The accumulators of a tile set to its expert's bias, or to zero without one, by sixteen MFMAs of that rank-one product
+// onto a constant zero: the matrix pipe clears the 256 registers in half the cycles that 256 register writes take.
+template <typename T>
+__device__ __forceinline__ void init_acc(const FwdArgs &a, f32x16 (&acc)[4][4], int e, int n0, int wp, int lane) {
+    const bool k0 = lane < 32;
+    const u32x4 q = {k0 ? one_bits<T>() : 0u, 0u, 0u, 0u};
+    uint32_t v[4] = {0u, 0u, 0u, 0u};
+    if (a.bias != nullptr) { // uniform
+        const uint16_t *b = a.bias + (int64_t)e * a.bias_es;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            int col = n0 + wp + 32 * j + (lane & 31);
+            if (col >= a.N) col = a.N - 1;
+            v[j] = b[col];
+        }
+    }
+    f32x16 zero;
+#pragma unroll
+    for (int c = 0; c < 16; ++c) zero[c] = 0.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const u32x4 p = {k0 ? v[j] : 0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[j][i] = Elem<T>::mfma(p, q, zero);
+    }
+}
+
 // Which tile a workgroup works on.
 struct TileSched {
     int e, rows_valid, n0; // expert, valid rows of the row tile, first output column
@@ -936,6 +963,7 @@ constexpr int PST_STAGING_OFF = STAGE_CHUNKS * 16; // the epilogue's staging are
 constexpr int PST_ROWS_OFF = PST_STAGING_OFF + 4 * EPI_BWD_WAVE_BYTES;
 constexpr int PST_QR = 0, PST_ER = 8, PST_SC = 16, PST_ROW_ITEMS = 20;
 constexpr int PST_TABLE_OFF = PST_SMEM_BYTES - 2 * (PST_MAX_E + 1) * (int)sizeof(int);
+constexpr int PST_STEP_LDS_OFF = PST_ROWS_OFF + PST_ROW_ITEMS * 1024; // timing build: 8 bytes per K step, up to the tables
 static_assert(EPI_BWD_WAVE_BYTES >= EPI_WAVE_BYTES && PST_ROWS_OFF + PST_ROW_ITEMS * 1024 <= PST_TABLE_OFF,
               "epilogue staging and the prefetched rows must fit between stage 0 and the schedule tables");
 
@@ -956,6 +984,15 @@ constexpr int PST_TIMING_TILES = 48;
 __device__ uint64_t g_pst_times[256][PST_TIMING_TILES][8];
 __device__ uint64_t g_pst_cycles[256][PST_TIMING_TILES][8]; // the shader clock counter at the same points
 __device__ int g_pst_no_ovl; // A/B switch of the timing build: 1 = no tile overlaps its neighbours' set-up
+// the shader clock counter behind every K step of one tile per workgroup (the PST_STEP_TILE-th): written to a spare
+// corner of LDS inside the loop (a vector store to memory would enter the loop's vmcnt waits), copied out behind the tile
+constexpr int PST_STEP_TILE = 3, PST_MAX_STEPS = 240;
+__device__ uint64_t g_pst_steps[256][PST_MAX_STEPS];
+#define PST_STEP_STAMP(kt)                                                                             \
+    do {                                                                                               \
+        if (tile_no == PST_STEP_TILE && threadIdx.x == 0 && (kt) < PST_MAX_STEPS)                      \
+            ((uint64_t *)(smem + PST_STEP_LDS_OFF))[(kt)] = __builtin_amdgcn_s_memtime();             \
+    } while (0)
 #define PST_STAMP(k)                                                                                   \
     do {                                                                                               \
         if (threadIdx.x == 0 && blockIdx.x < 256 && tile_no < PST_TIMING_TILES) {                      \
@@ -966,6 +1003,9 @@ __device__ int g_pst_no_ovl; // A/B switch of the timing build: 1 = no tile over
 #else
 #define PST_STAMP(k) \
     do {             \
+    } while (0)
+#define PST_STEP_STAMP(kt) \
+    do {                   \
     } while (0)
 #endif
 
@@ -1215,7 +1255,10 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
         // epilogue have been handed over and its staging area is dead
         asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
         PST_STAMP(1);
-        static_for<DMA_N0>([&](auto P) { issue_piece(1, P, IC<0>{}); });
+        if (KT_full >= 2) // the second K step exists and is complete: the short form of the loads
+            static_for<DMA_N0>([&](auto P) { issue_piece(1, P, IC<1>{}); });
+        else
+            static_for<DMA_N0>([&](auto P) { issue_piece(1, P, IC<0>{}); });
 
         // One tile ahead: the next tile's schedule entry and rows, and this tile's row scales (their addresses are the
         // epilogue's row indices, fetched a tile ago); all of it lands in LDS during the main loop.  A full tile with an
@@ -1243,8 +1286,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
 
         PST_STAMP(2);
         f32x16 acc[4][4];
-        zero_acc(acc);
-        if (a.bias != nullptr) add_bias<T>(a, acc, cur.e, cur.n0, wp, lane);
+        init_acc<T>(a, acc, cur.e, cur.n0, wp, lane);
         FragBase<0> qb;
         FragBase<WT> pb;
         make_frag_base<0>(qb, lds0, wq, lane);
@@ -1256,7 +1298,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
                 static_for<4>([&](auto I) { f0.p[I.value] = read_frag<WT, I.value, 0>(pb); });
                 static_for<NI>([&](auto I) { f0.q[I.value] = read_frag<0, I.value, 0>(qb); });
             }
-            // One K step.  FULL: steps kt + 1 and kt + 2 exist and are complete.  MODE 1, the first step of a tile that
+            // One K step.  FULL = 1: steps kt + 1 and kt + 2 exist and are complete; FULL = 2: step kt + 1 exists and is
+            // complete and is the tile's last (nothing is loaded for kt + 2); FULL = 0: every piece checks.  MODE 1, the first step of a tile that
             // overlaps (`ovl`): the free slots of its second half take the next tile's schedule entry and the 16 row
             // items; they are the youngest loads at the step's barrier, which leaves exactly them in flight.  MODE 2, the
             // last step of such a tile (it lives in stage 1, stage 0 has been free since the barrier before): its slots
@@ -1266,14 +1309,21 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
                 constexpr int mode = MODE.value;
                 int kt_a = kt + 1, kt_b = kt + 2;
                 asm volatile("" : "+s"(kt_a), "+s"(kt_b));
+                // MODE 2: the next tile's eight gathered rows, read from the row area in one go in front of the step's MFMAs
+                // (one wait for all of them; read inside the slots, each would stall the MFMA stream for an LDS round trip)
+                [[maybe_unused]] uint32_t nxt_rows[8];
+                if constexpr (mode == 2) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i)
+                        nxt_rows[i] = need_q_idx ? row_item(PST_QR + i, tid) : (uint32_t)q_row(nxt, i, lane, wave);
+                }
                 mma_step<T, WT, 0, 1, NI>(f0, f1, pb, qb, acc, [&](auto G) {
                     if constexpr (mode == 2) {
                         // also when there is no next tile (all fields zero then: addresses that nothing is loaded from):
                         // a branch here would only add a join of sixteen registers to the loop
-                        make_pointer(nxt, G, lane, wave,
-                                     need_q_idx ? row_item(PST_QR + G.value, tid) : (uint32_t)q_row(nxt, G.value, lane, wave));
+                        make_pointer(nxt, G, lane, wave, nxt_rows[G.value]);
                     } else if constexpr (G.value < DMA_N1) {
-                        issue_piece(kt_a, IC<DMA_N0 + G.value>{}, FULL);
+                        issue_piece(kt_a, IC<DMA_N0 + G.value>{}, IC<(FULL.value != 0) ? 1 : 0>{});
                     }
                 });
                 mma_step<T, WT, 0, 2, NI>(f1, f0, pb, qb, acc, [&](auto G) {
@@ -1282,7 +1332,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
                     } else if constexpr (mode == 2) {
                         if (nxt.valid) issue_piece(0, G, IC<1>{});
                     } else if constexpr (G.value < DMA_N2) {
-                        issue_piece(kt_a, IC<DMA_N0 + DMA_N1 + G.value>{}, FULL);
+                        issue_piece(kt_a, IC<DMA_N0 + DMA_N1 + G.value>{}, IC<(FULL.value != 0) ? 1 : 0>{});
                     }
                 });
                 mma_step<T, WT, 0, 3, NI>(f0, f1, pb, qb, acc, [&](auto G) {
@@ -1300,11 +1350,12 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
                 flip_stage(pb);
                 flip_stage(qb);
                 mma_step<T, WT, 0, 0, NI, (mode == 2 ? 0 : 1)>(f1, f0, pb, qb, acc, [&](auto G) {
-                    if constexpr (mode != 2) {
+                    if constexpr (mode != 2 && FULL.value != 2) {
                         if constexpr (G.value < DMA_N0) issue_piece(kt_b, G, FULL);
                         if constexpr (G.value + 8 < DMA_N0) issue_piece(kt_b, IC<G.value + 8>{}, FULL);
                     }
                 });
+                PST_STEP_STAMP(kt);
             };
             int kt = 0, kt_end = KT;
             if constexpr (NI == 4) {
@@ -1313,6 +1364,10 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
                     kt = 1, kt_end = KT - 1;
                 }
                 for (; kt + 2 < KT_full && kt < kt_end; ++kt) k_step(kt, IC<1>{}, IC<0>{});
+                if (kt + 2 == KT && kt + 1 < KT_full && kt < kt_end) { // the step in front of a complete last step
+                    k_step(kt, IC<2>{}, IC<0>{});
+                    ++kt;
+                }
             }
             for (; kt < kt_end; ++kt) k_step(kt, IC<0>{}, IC<0>{});
             if constexpr (NI == 4) {
@@ -1363,6 +1418,10 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
         }
         tile_epilogue<T, EPI>(a, acc, smem + PST_STAGING_OFF, cur.row0, cur.rows_valid, cur.n0, tid_e, -1, &er);
         PST_STAMP(5);
+#ifdef XMA_PST_TIMING
+        if (tile_no == PST_STEP_TILE && threadIdx.x == 0 && blockIdx.x < 256)
+            for (int q = 0; q < KT && q < PST_MAX_STEPS; ++q) g_pst_steps[blockIdx.x][q] = ((uint64_t *)(smem + PST_STEP_LDS_OFF))[q];
+#endif
         if (!nxt.valid) break;
         cur = nxt;
         e_buf ^= 1;
@@ -1800,6 +1859,9 @@ extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_times(v
 }
 extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_cycles(void *host_out) {
     return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_pst_cycles), sizeof(g_pst_cycles));
+}
+extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_steps(void *host_out) {
+    return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_pst_steps), sizeof(g_pst_steps));
 }
 extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_band(int v) {
     return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_pst_band), &v, sizeof(v));

@@ -1,19 +1,22 @@
-"""Where a tile of the persistent grouped GEMM kernel spends its time.
+"""Where a tile of the persistent grouped GEMM kernel spends its time, in shader cycles and microseconds.
 
     python accelerated-model-architectures_amd/build.py --timing       (here, no GPU needed)
     python accelerated-model-architectures_amd/diagnostics/tile_phases.py [c3] [c4] [c5]    (on the GPU box)
 
 The timing build of the library (xma/rocm/libxma_rocm_timing.so, grouped_gemm.hip compiled with -DXMA_PST_TIMING) makes
-thread 0 of every workgroup write the 100 MHz real-time counter at six points of each of its first 48 tiles;
-xma_rocm_debug_pst_times copies the stamps out.  Per workload and forward-type GEMM this prints the mean duration of
-the phases of a tile, first and last tile of every workgroup left out:
+thread 0 of every workgroup read the 100 MHz real-time counter and the shader clock counter at six points of each of its
+first 48 tiles, and the shader clock counter behind every K step of its fourth tile.  Per workload and forward-type GEMM
+this prints
 
-    wait   top of the tile: its first K step and the rows of its epilogue have landed, all waves have met
-    setup  what precedes the main loop (second K step's first loads; for tiles that do not overlap: the next tile's
-           schedule entry and row indices)
-    loop   the K loop (for tiles that overlap it contains the next tile's set-up and the issue of its first K step)
-    issue  behind the loop: operand addresses and first K step of the next tile (tiles that do not overlap)
-    epi    the epilogue
+  phases   mean duration of the phases of a tile (first and last tile of every workgroup left out):
+           wait (top of the tile: its first K step has landed, all waves have met), setup (up to the main loop), loop,
+           issue (behind the loop: the next tile's first K step, for tiles that do not overlap it with their last step),
+           epi (the epilogue)
+  loop     shader cycles per K step (2048 = the 64 MFMAs of a step back to back) and the clock the loop ran at
+  steps    median cycles of the single K steps of one tile: the first step (which also looks up the next tile and
+           fetches its row indices), the following ones (loads of a fresh operand panel), the steady state, the last two
+           (the last one sets up and issues the next tile's first K step)
+  ends     when the workgroups finish (the launch ends with the slowest)
 """
 
 from __future__ import annotations
@@ -31,22 +34,25 @@ sys.path.insert(0, os.path.dirname(HERE))
 from xma.rocm.loader import SIGNATURES  # noqa: E402
 
 WORKLOADS = {"c3": (8192, 4096, 14336, 8, 2, 0.0), "c4": (16384, 2048, 1408, 64, 6, 1.5), "c5": (32768, 2048, 768, 128, 8, 0.0)}
-TILES, STAMPS = 48, 8
+TILES, STAMPS, MAX_STEPS, STEP_TILE = 48, 8, 240, 3
 
 
-def load():
-    path = os.path.join(os.path.dirname(HERE), "xma", "rocm", "libxma_rocm_timing.so")
+def load(path=None):
+    path = path or os.path.join(os.path.dirname(HERE), "xma", "rocm", "libxma_rocm_timing.so")
     if not os.path.isfile(path):
         sys.exit(f"{path} is missing: build it with `python accelerated-model-architectures_amd/build.py --timing`")
     lib = ctypes.CDLL(path)
     for name, (res, args) in SIGNATURES.items():
-        f = getattr(lib, name)
-        f.restype, f.argtypes = res, args
-    lib.xma_rocm_debug_pst_times.argtypes = [ctypes.c_void_p]
+        if hasattr(lib, name):
+            f = getattr(lib, name)
+            f.restype, f.argtypes = res, args
+    for name in ("xma_rocm_debug_pst_times", "xma_rocm_debug_pst_cycles", "xma_rocm_debug_pst_steps"):
+        getattr(lib, name).argtypes = [ctypes.c_void_p]
     return lib
 
 
-def run(lib, name):
+def make_ops(lib, name):
+    """the four forward-type GEMMs of a workload as closures, with their K step counts"""
     T, H, I, E, k, bias = WORKLOADS[name]
     dev, bf = "cuda", torch.bfloat16
     g = torch.Generator(device=dev).manual_seed(0)
@@ -65,39 +71,72 @@ def run(lib, name):
     eo = torch.empty(Tk, H, device=dev, dtype=bf)
     st = torch.cuda.current_stream().cuda_stream
     P = lambda t: t.data_ptr()  # noqa: E731
+    keep = (x, w1, w2, ss, offs, z, h, dz, dy, rw, eo)
 
     def s2s(*a):
         rc = lib.xma_rocm_scatter2scatter(*a, None, 0, st)
         assert rc == 0, lib.xma_rocm_last_error()
 
-    ops = {
-        "up-projection + SwiGLU": lambda: s2s(P(x), H, P(w1), 2 * I * H, H, 0, P(ss), P(offs), P(z), 2 * I, P(h), I, None, Tk, 2 * I, H, E, k, 0, 1, 1, 0),
-        "down-projection": lambda: s2s(P(h), I, P(w2), H * I, I, 0, P(ss), P(offs), P(eo), H, None, 0, None, Tk, H, I, E, 1, 1, 0, 0, 0),
-        "dX2 + SwiGLU backward": lambda: s2s(P(dy), H, P(w2), H * I, I, 1, P(ss), P(offs), P(dz), 2 * I, P(z), 2 * I, P(rw), Tk, I, H, E, k, 0, 1, 2, 0),
-        "dX1": lambda: s2s(P(dz), 2 * I, P(w1), 2 * I * H, H, 1, P(ss), P(offs), P(eo), H, None, 0, None, Tk, H, 2 * I, E, 1, 1, 0, 0, 0),
-    }
-    for what, op in ops.items():
-        for _ in range(3):
-            op()
-        torch.cuda.synchronize()
-        assert lib.xma_rocm_debug_pst_reset() == 0
-        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-        s.record()
+    return {
+        "up-projection + SwiGLU": (lambda: s2s(P(x), H, P(w1), 2 * I * H, H, 0, P(ss), P(offs), P(z), 2 * I, P(h), I, None, Tk, 2 * I, H, E, k, 0, 1, 1, 0), H // 64),
+        "down-projection": (lambda: s2s(P(h), I, P(w2), H * I, I, 0, P(ss), P(offs), P(eo), H, None, 0, None, Tk, H, I, E, 1, 1, 0, 0, 0), I // 64),
+        "dX2 + SwiGLU backward": (lambda: s2s(P(dy), H, P(w2), H * I, I, 1, P(ss), P(offs), P(dz), 2 * I, P(z), 2 * I, P(rw), Tk, I, H, E, k, 0, 1, 2, 0), H // 64),
+        "dX1": (lambda: s2s(P(dz), 2 * I, P(w1), 2 * I * H, H, 1, P(ss), P(offs), P(eo), H, None, 0, None, Tk, H, 2 * I, E, 1, 1, 0, 0, 0), 2 * I // 64),
+    }, keep
+
+
+def measure(lib, op, KT):
+    """one launch with cleared stamps -> dict of the figures this script prints"""
+    for _ in range(2):
         op()
-        e.record()
-        torch.cuda.synchronize()
-        buf = np.zeros((256, TILES, STAMPS), dtype=np.uint64)
-        assert lib.xma_rocm_debug_pst_times(buf.ctypes.data) == 0
-        t = buf.astype(np.int64)
-        n_tiles = (t[:, :, 5] > 0).sum(1)
-        rows = []
-        for b in range(256):
-            for i in range(1, min(n_tiles[b], TILES - 1) - 1):
-                rows.append([t[b, i, j + 1] - t[b, i, j] for j in range(5)] + [t[b, i + 1, 0] - t[b, i, 0]])
-        r = np.array(rows) * 0.01  # 100 MHz ticks -> microseconds
-        m = r.mean(0)
-        print(f"{name} {what}: launch {s.elapsed_time(e) * 1e3:.0f} us, {n_tiles.min()}-{n_tiles.max()} tiles per workgroup; per tile "
-              f"wait {m[0]:.2f} setup {m[1]:.2f} loop {m[2]:.2f} issue {m[3]:.2f} epi {m[4]:.2f} total {m[5]:.2f} us", flush=True)
+    torch.cuda.synchronize()
+    assert lib.xma_rocm_debug_pst_reset() == 0
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    op()
+    e.record()
+    torch.cuda.synchronize()
+    tb = np.zeros((256, TILES, STAMPS), dtype=np.uint64)
+    cb = np.zeros_like(tb)
+    sb = np.zeros((256, MAX_STEPS), dtype=np.uint64)
+    assert lib.xma_rocm_debug_pst_times(tb.ctypes.data) == 0 and lib.xma_rocm_debug_pst_cycles(cb.ctypes.data) == 0
+    assert lib.xma_rocm_debug_pst_steps(sb.ctypes.data) == 0
+    t, c, st = tb.astype(np.int64), cb.astype(np.int64), sb.astype(np.int64)
+    n_tiles = (t[:, :, 5] > 0).sum(1)
+    sel = [(b, i) for b in range(256) for i in range(1, min(n_tiles[b], TILES - 1) - 1)]
+    ph = np.array([[t[b, i, j + 1] - t[b, i, j] for j in range(5)] + [t[b, i + 1, 0] - t[b, i, 0]] for b, i in sel]) * 0.01
+    lc = np.array([c[b, i, 3] - c[b, i, 2] for b, i in sel], dtype=np.float64)
+    lt = ph[:, 2]
+    out = {"launch_us": s.elapsed_time(e) * 1e3, "tiles": (int(n_tiles.min()), int(n_tiles.max())), "phases_us": ph.mean(0),
+           "cycles_per_step": lc.mean() / KT, "clock_ghz": lc.sum() / lt.sum() / 1e3,
+           "behind_loop_cycles": float(np.mean([c[b, i, 5] - c[b, i, 3] for b, i in sel]))}
+    ok = n_tiles > 0
+    ends = np.array([t[b, min(n_tiles[b], TILES) - 1, 5] for b in range(256) if ok[b]]) - t[ok, 0, 0].min()
+    out["ends_us"] = (ends.min() * 0.01, np.median(ends) * 0.01, ends.max() * 0.01) if (n_tiles[ok] <= TILES).all() else None
+    n = min(KT, MAX_STEPS)
+    have = (st[:, n - 1] > 0) & (c[:, STEP_TILE, 5] > 0)
+    if have.any():
+        sv, cv = st[have], c[have]
+        d = np.median(np.diff(sv[:, :n], axis=1), axis=0)
+        out["steps"] = {"first": float(np.median(sv[:, 0] - cv[:, STEP_TILE, 2])), "next": d[:6], "steady": float(np.median(d[6:max(7, n - 4)])),
+                        "last": d[-2:], "top_to_loop": float(np.median(cv[:, STEP_TILE, 2] - cv[:, STEP_TILE, 0]))}
+    return out
+
+
+def run(lib, name):
+    ops, _keep = make_ops(lib, name)
+    for what, (op, KT) in ops.items():
+        r = measure(lib, op, KT)
+        m = r["phases_us"]
+        print(f"{name} {what}: launch {r['launch_us']:.0f} us, {r['tiles'][0]}-{r['tiles'][1]} tiles per workgroup", flush=True)
+        print(f"   phases (us): wait {m[0]:.2f} setup {m[1]:.2f} loop {m[2]:.2f} issue {m[3]:.2f} epi {m[4]:.2f} total {m[5]:.2f}")
+        print(f"   loop: {r['cycles_per_step']:.0f} shader cycles per K step at {r['clock_ghz']:.3f} GHz; behind the loop {r['behind_loop_cycles']:.0f} cycles")
+        if "steps" in r:
+            s = r["steps"]
+            print(f"   steps (cycles, {KT} per tile): top of tile to loop {s['top_to_loop']:.0f}; first {s['first']:.0f}; then "
+                  f"{' '.join(f'{v:.0f}' for v in s['next'])}; steady {s['steady']:.0f}; last two {' '.join(f'{v:.0f}' for v in s['last'])}")
+        if r["ends_us"]:
+            print(f"   workgroups end at (us from the first start): min {r['ends_us'][0]:.0f} median {r['ends_us'][1]:.0f} max {r['ends_us'][2]:.0f}")
 
 
 if __name__ == "__main__":

@@ -110,6 +110,8 @@ XMA_API int xma_rocm_route(const void *ids, int ids_are_int64, int64_t n, int32_
  * Limit: ceil(n / 4096) * num_experts <= xma_rocm_route_static_max_units_times_experts() (= 262144; e.g. 4 Mi ids
  * over 256 experts); larger problems return XMA_ROCM_EWORKSPACE and must use xma_rocm_route.  All calls on one GPU
  * share that array: calls that overlap on one GPU (two streams, two threads) race and must be serialised by the caller.
+ * The first call on a device looks up the array's address and raises a kernel's LDS limit, which are not stream
+ * operations: make one ordinary call per device before capturing this entry point in a graph.
  */
 XMA_API size_t xma_rocm_route_static_max_units_times_experts(void);
 XMA_API int xma_rocm_route_static(const void *ids, int ids_are_int64, int64_t n, int32_t num_experts, uint32_t *counts,
@@ -124,7 +126,9 @@ XMA_API int xma_rocm_route_static(const void *ids, int ids_are_int64, int64_t n,
  *     src(n)  = n                         if x_grouped else sorted_scattered_idxs[n] / fan_out
  *     dst(n)  = n                         if y_grouped else sorted_scattered_idxs[n]
  * followed by the epilogue (XMA_ROCM_EPI_*).  row_scale (may be NULL) is a
- * vector indexed in scattered order (the flattened (T, k) router weights).
+ * vector indexed in scattered order (the flattened (T, k) router weights); a 16-bit scale is fetched as the aligned
+ * 4-byte word around it, so the vector's allocation must extend to an even number of elements (a vector that starts
+ * off a 4-byte boundary is accepted and takes a slower kernel).
  * Replaces scatter2scatter, xma/layers/moe/triton_implementation/scatter_kernel.py:137-183
  * (kernel :58-134), the separate activation pass xma/layers/moe/__init__.py:226
  * and its autograd backward, and the coefficient pass of `group`

@@ -88,11 +88,12 @@ def test_moe_reference_grid_7_tokens(dtype, E, k, act_name):
     _run_case(dtype, 7, E, k, 512, 1024, act_name)
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 @pytest.mark.parametrize("act_name", ["swiglu_packed", "glu"])
-def test_moe_reference_sizes(act_name):
-    # the two size points of the reference grid (moe_test.py:31-32 and :43-46)
-    _run_case(torch.bfloat16, 7, 8, 2, 2048, 8192, act_name)
-    _run_case(torch.bfloat16, 7, 128, 8, 576, 256, act_name)
+def test_moe_reference_sizes(dtype, act_name):
+    # the two size points of the reference grid (moe_test.py:31-32 and :43-46) in its three dtypes
+    _run_case(dtype, 7, 8, 2, 2048, 8192, act_name)
+    _run_case(dtype, 7, 128, 8, 576, 256, act_name)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])

@@ -80,3 +80,37 @@ def test_route_static_rejects_sizes_beyond_its_scratch():
     assert b"static scratch" in lib.xma_rocm_last_error()
     torch.cuda.synchronize()
     assert int(pos.abs().sum()) == 0  # nothing ran
+
+
+def test_route_static_captured_in_a_graph_after_a_warm_up_call():
+    """The use the entry point exists for: one ordinary call per device first (it resolves the scratch's address and raises
+    the scatter kernel's LDS limit, neither of which is a stream operation), then the call is captured in a HIP graph and
+    replayed on new ids written into the same input buffer; every replay against xma_rocm_route, with eager work and
+    synchronisations between the replays."""
+    from xma.rocm import get_library
+    from xma.rocm.loader import check
+
+    lib = get_library()
+    n, E = 300000, 64
+    g = torch.Generator().manual_seed(9)
+    ids = torch.randint(0, E, (n,), generator=g, dtype=torch.int32).cuda()
+    _route(lib, ids, E, static=True)  # warm-up, outside any capture
+    counts = torch.zeros(E, dtype=torch.int32, device="cuda")
+    incl = torch.zeros(E, dtype=torch.int64, device="cuda")
+    excl = torch.zeros(E, dtype=torch.int64, device="cuda")
+    sorted_e = torch.zeros(n, dtype=torch.int32, device="cuda")
+    sorted_s = torch.zeros(n, dtype=torch.int64, device="cuda")
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        check(lib.xma_rocm_route_static(ids.data_ptr(), 0, n, E, counts.data_ptr(), incl.data_ptr(), excl.data_ptr(),
+                                        sorted_e.data_ptr(), sorted_s.data_ptr(), torch.cuda.current_stream().cuda_stream),
+              "xma_rocm_route_static")
+    for rep in range(3):
+        ids.copy_(torch.randint(0, E, (n,), generator=g, dtype=torch.int32))
+        graph.replay()
+        torch.cuda.synchronize()
+        want = _route(lib, ids, E, static=False)  # eager work between the replays
+        assert np.array_equal(np_of(counts), want["counts"]) and np.array_equal(np_of(incl), want["incl"]), rep
+        assert np.array_equal(np_of(excl), want["excl"]) and np.array_equal(np_of(sorted_e), want["sorted_e"]), rep
+        assert np.array_equal(np_of(sorted_s), want["sorted_s"]), rep
