@@ -1434,6 +1434,21 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_persistent_kerne
 //   GQ / GP = 1: the rows of dY / X are taken through sorted_scattered_idxs (index / fan_out); 0: grouped order
 // ------------------------------------------------------------------------------------------------
 constexpr int DW_BAND = 4;
+#ifdef XMA_PST_TIMING
+// timing build: shader clock counter of the first DW_TIMING_TILES workgroups at the start of the kernel, in front of and
+// behind the K loop and at the end, and the tile's K step count
+constexpr int DW_TIMING_TILES = 8192;
+__device__ uint64_t g_dw_cycles[DW_TIMING_TILES][6];
+#define DW_STAMP(k)                                                                   \
+    do {                                                                              \
+        if (threadIdx.x == 0 && blockIdx.x < DW_TIMING_TILES)                          \
+            g_dw_cycles[blockIdx.x][k] = (k) == 4 ? (uint64_t)KT : __builtin_amdgcn_s_memtime(); \
+    } while (0)
+#else
+#define DW_STAMP(k) \
+    do {            \
+    } while (0)
+#endif
 template <typename T, int GQ, int GP>
 __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const DwArgs a) {
     constexpr int GATHER = GQ | GP;
@@ -1470,6 +1485,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
     const int64_t row_lo = e ? a.offs[e - 1] : 0, row_hi = a.offs[e];
     const int rows = (int)(row_hi - row_lo);
     const int KT = (rows + BK - 1) / BK;
+    DW_STAMP(0);
+    DW_STAMP(4);
     const uint16_t *zero = (const uint16_t *)g_zero_page;
     const int q_max_chunk = ((a.N_out - o0) >> 3) - 1, p_max_chunk = ((a.K_in - i0) >> 3) - 1;
     const int kr_lane = wave * 16 + (lane >> 5); // this lane's k-rows of a step: kr_lane + 2 j, j = 0..7
@@ -1580,6 +1597,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
             asm volatile("s_waitcnt vmcnt(0)\n\ts_barrier" ::: "memory");
         Frags f0, f1;
         load_frags<1, 1, 0>(f0, pb, qb);
+        DW_STAMP(1);
         // one K step; FULL: steps kt + 1 and kt + 2 lie completely inside the expert's rows
         auto k_step = [&](int kt, auto FULL) {
             // idx_next holds the indices of step kt + 1 here; the second half of that step's loads goes out now, then
@@ -1600,6 +1618,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
         for (; kt + 2 < KT_full; ++kt) k_step(kt, IC<1>{});
         for (; kt < KT; ++kt) k_step(kt, IC<0>{});
         XMA_WAIT_ALL_LOADS();
+        DW_STAMP(2);
     }
 
     // lane owns DW row o (from the Q tile), 4 consecutive in-features per quad; each 32-row block is staged in a
@@ -1632,6 +1651,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 1) void grouped_gemm_dw_kernel(const 
         }
         wave_lds_sync(); // the next block overwrites the area
     }
+    DW_STAMP(3);
 }
 
 inline int device_cus();
@@ -1714,9 +1734,12 @@ inline int device_cus() {
 // Launches of fewer rounds than this may split the tiles of their last round over the idle CUs.
 constexpr int64_t SPLIT_MAX_ROUNDS = 12;
 
-inline size_t fwd_workspace_bytes(int64_t M, int32_t N, int32_t E) {
+inline size_t fwd_workspace_bytes(int64_t M, int32_t N, int32_t K, int32_t E) {
     const int cus = device_cus();
     if (cus <= 0) return 0;
+    // a tile is cut into at least two slices of SPLIT_MIN_STEPS K steps or not at all: short K never splits, and the two
+    // launches that would find nothing to do are not made
+    if ((K + BK - 1) / BK < 2 * SPLIT_MIN_STEPS) return 0;
     const int64_t tiles = (M / BM + E) * ((N + BN - 1) / BN);
     if (tiles > SPLIT_MAX_ROUNDS * cus) return 0;
     return (size_t)cus * BM * BN * sizeof(float);
@@ -1803,7 +1826,7 @@ static int scatter2scatter_impl(const void *X, int64_t ldx, const void *W, int64
     a.grid_main = (int)grid;
     a.partial = nullptr;
     a.split_cus = 0;
-    const size_t ws_need = fwd_workspace_bytes(M, N, E);
+    const size_t ws_need = fwd_workspace_bytes(M, N, K, E);
     if (workspace && ws_need) {
         XMA_REQUIRE(workspace_bytes >= ws_need && aligned16(workspace), XMA_ROCM_EWORKSPACE,
                     "scatter2scatter: workspace of %zu bytes, %zu needed (16-byte aligned)", workspace_bytes, ws_need);
@@ -1863,6 +1886,9 @@ extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_cycles(
 extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_steps(void *host_out) {
     return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_pst_steps), sizeof(g_pst_steps));
 }
+extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_dw_cycles(void *host_out) {
+    return (int)hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_dw_cycles), sizeof(g_dw_cycles));
+}
 extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_band(int v) {
     return (int)hipMemcpyToSymbol(HIP_SYMBOL(g_pst_band), &v, sizeof(v));
 }
@@ -1877,9 +1903,8 @@ extern "C" __attribute__((visibility("default"))) int xma_rocm_debug_pst_reset(v
 #endif
 
 extern "C" size_t xma_rocm_scatter2scatter_workspace_bytes(int64_t M, int32_t N, int32_t K, int32_t E) {
-    (void)K;
-    if (M <= 0 || N <= 0 || E <= 0) return 0;
-    return fwd_workspace_bytes(M, N, E);
+    if (M <= 0 || N <= 0 || K <= 0 || E <= 0) return 0;
+    return fwd_workspace_bytes(M, N, K, E);
 }
 
 extern "C" int xma_rocm_group_bwd_W(const void *DY, int64_t lddy, int dy_grouped, int32_t dy_fan_out,

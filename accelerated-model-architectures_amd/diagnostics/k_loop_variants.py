@@ -4,7 +4,7 @@
     python accelerated-model-architectures_amd/diagnostics/k_loop_variants.py build         (here, no GPU needed)
     python accelerated-model-architectures_amd/diagnostics/k_loop_variants.py run [c3] [c5] (on the GPU box)
 
-`build` writes patched copies of csrc/grouped_gemm.hip to build/variants/, compiles each with -DXMA_PST_TIMING (bf16,
+`build` writes patched copies of csrc/grouped_gemm.hip to diagnostics/variants/, compiles each with -DXMA_PST_TIMING (bf16,
 forward-type kernels only) and links it with the other objects of the normal build.  The patches touch the steady K steps
 only (complete steps in the middle of a tile; the first and last steps of a tile keep every wait), and all variants but
 `base` compute WRONG RESULTS on purpose - they exist to be timed, nothing else loads them:
@@ -29,7 +29,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.dirname(HERE)
-OUT = os.path.join(PKG, "build", "variants")
+OUT = os.path.join(HERE, "variants")  # generated sources and libraries: not tracked, but they travel to the GPU box
 VARIANTS = ["base", "novm", "nowait", "nodma", "noreads", "lead2"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 OTHER_OBJECTS = ["api", "routing", "elementwise", "grouped_gemm_staged", "fp32", "router", "swiglu", "bias", "diagnostics"]
@@ -129,7 +129,7 @@ def run(workloads):
     for name in workloads:
         for tag in VARIANTS:
             lib = tile_phases.load(os.path.join(OUT, f"grouped_gemm_{tag}.so"))
-            ops, _keep = tile_phases.make_ops(lib, name)
+            ops, _dw_ops, _keep = tile_phases.make_ops(lib, name)
             for what, (op, KT) in ops.items():
                 if "SwiGLU backward" in what:
                     continue  # not among the three instantiations of the variants

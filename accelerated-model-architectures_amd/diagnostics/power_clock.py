@@ -79,6 +79,11 @@ def main():
     lib = get_library()
     paths = sensors()
     print("power sensor:", paths[0] if paths else "none found (the watt columns are nan)", flush=True)
+    for cap in glob.glob("/sys/class/drm/card*/device/hwmon/hwmon*/power1_cap"):
+        try:
+            print(f"board power limit ({cap}): {int(open(cap).read().strip()) * 1e-6:.0f} W", flush=True)
+        except (OSError, ValueError):
+            pass
     measure("idle (no kernel)", lambda: None, 0, paths, secs=1.0)
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     st = torch.cuda.current_stream().cuda_stream
@@ -88,10 +93,12 @@ def main():
     rnd = (torch.rand(16 * 256 * 8, device="cuda") * 4 - 2).to(torch.bfloat16)
     for label, opnd in (("MFMA stream, random operands", rnd), ("MFMA stream, zero operands", torch.zeros_like(rnd))):
         measure(label, lambda: check(lib.xma_rocm_diag_mfma_stream(opnd.data_ptr(), iters, out.data_ptr(), cus, st), "diag"), stream_flops, paths)
-    ops, keep = tile_phases.make_ops(lib, "c3")
+    ops, dw_ops, keep = tile_phases.make_ops(lib, "c3")
     T, H, I, E, k, _ = tile_phases.WORKLOADS["c3"]
     f = 2.0 * T * k * H * I
     for (what, (op, _kt)), fl in zip(ops.items(), (2 * f, f, f, 2 * f)):
+        measure("grouped " + what, op, fl, paths)
+    for (what, op), fl in zip(dw_ops.items(), (f, 2 * f)):
         measure("grouped " + what, op, fl, paths)
     g = torch.Generator(device="cuda").manual_seed(0)
     Tk = T * k

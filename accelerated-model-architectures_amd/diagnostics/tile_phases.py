@@ -17,6 +17,9 @@ this prints
            fetches its row indices), the following ones (loads of a fresh operand panel), the steady state, the last two
            (the last one sets up and issues the next tile's first K step)
   ends     when the workgroups finish (the launch ends with the slowest)
+
+and for the two weight-gradient GEMMs (one workgroup per tile, thread 0 stamps the shader clock at four points) the median
+cycles of a tile's prologue, main loop (per K step) and epilogue.
 """
 
 from __future__ import annotations
@@ -34,7 +37,7 @@ sys.path.insert(0, os.path.dirname(HERE))
 from xma.rocm.loader import SIGNATURES  # noqa: E402
 
 WORKLOADS = {"c3": (8192, 4096, 14336, 8, 2, 0.0), "c4": (16384, 2048, 1408, 64, 6, 1.5), "c5": (32768, 2048, 768, 128, 8, 0.0)}
-TILES, STAMPS, MAX_STEPS, STEP_TILE = 48, 8, 240, 3
+TILES, STAMPS, MAX_STEPS, STEP_TILE, DW_TILES = 48, 8, 240, 3, 8192
 
 
 def load(path=None):
@@ -46,7 +49,7 @@ def load(path=None):
         if hasattr(lib, name):
             f = getattr(lib, name)
             f.restype, f.argtypes = res, args
-    for name in ("xma_rocm_debug_pst_times", "xma_rocm_debug_pst_cycles", "xma_rocm_debug_pst_steps"):
+    for name in ("xma_rocm_debug_pst_times", "xma_rocm_debug_pst_cycles", "xma_rocm_debug_pst_steps", "xma_rocm_debug_dw_cycles"):
         getattr(lib, name).argtypes = [ctypes.c_void_p]
     return lib
 
@@ -71,7 +74,10 @@ def make_ops(lib, name):
     eo = torch.empty(Tk, H, device=dev, dtype=bf)
     st = torch.cuda.current_stream().cuda_stream
     P = lambda t: t.data_ptr()  # noqa: E731
-    keep = (x, w1, w2, ss, offs, z, h, dz, dy, rw, eo)
+    gdy = torch.randn(Tk, H, device=dev, generator=g).to(bf)
+    dw1 = torch.empty(E, 2 * I, H, device=dev, dtype=bf)
+    dw2 = torch.empty(E, H, I, device=dev, dtype=bf)
+    keep = (x, w1, w2, ss, offs, z, h, dz, dy, rw, eo, gdy, dw1, dw2)
 
     def s2s(*a):
         rc = lib.xma_rocm_scatter2scatter(*a, None, 0, st)
@@ -82,7 +88,29 @@ def make_ops(lib, name):
         "down-projection": (lambda: s2s(P(h), I, P(w2), H * I, I, 0, P(ss), P(offs), P(eo), H, None, 0, None, Tk, H, I, E, 1, 1, 0, 0, 0), I // 64),
         "dX2 + SwiGLU backward": (lambda: s2s(P(dy), H, P(w2), H * I, I, 1, P(ss), P(offs), P(dz), 2 * I, P(z), 2 * I, P(rw), Tk, I, H, E, k, 0, 1, 2, 0), H // 64),
         "dX1": (lambda: s2s(P(dz), 2 * I, P(w1), 2 * I * H, H, 1, P(ss), P(offs), P(eo), H, None, 0, None, Tk, H, 2 * I, E, 1, 1, 0, 0, 0), 2 * I // 64),
+    }, {
+        "dW2": lambda: lib.xma_rocm_group_bwd_W(P(gdy), H, 1, 1, None, P(h), I, 1, 1, P(ss), P(offs), P(dw2), H * I, I, H, I, E, 0, st),
+        "dW1": lambda: lib.xma_rocm_group_bwd_W(P(dz), 2 * I, 1, 1, None, P(x), H, 0, k, P(ss), P(offs), P(dw1), 2 * I * H, H, 2 * I, H, E, 0, st),
     }, keep
+
+
+def measure_dw(lib, op):
+    """one launch of a weight-gradient GEMM -> median cycles of the parts of its tiles that have at least 8 K steps"""
+    for _ in range(2):
+        assert op() == 0, lib.xma_rocm_last_error()
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    assert op() == 0
+    e.record()
+    torch.cuda.synchronize()
+    buf = np.zeros((DW_TILES, 6), dtype=np.uint64)
+    assert lib.xma_rocm_debug_dw_cycles(buf.ctypes.data) == 0
+    c = buf.astype(np.int64)
+    c = c[(c[:, 3] > 0) & (c[:, 4] >= 8)]
+    kt = c[:, 4]
+    return {"launch_us": s.elapsed_time(e) * 1e3, "tiles": len(c), "steps": float(kt.mean()), "prologue": float(np.median(c[:, 1] - c[:, 0])),
+            "per_step": float(np.median((c[:, 2] - c[:, 1]) / kt)), "epilogue": float(np.median(c[:, 3] - c[:, 2])), "tile": float(np.median(c[:, 3] - c[:, 0]))}
 
 
 def measure(lib, op, KT):
@@ -124,7 +152,7 @@ def measure(lib, op, KT):
 
 
 def run(lib, name):
-    ops, _keep = make_ops(lib, name)
+    ops, dw_ops, _keep = make_ops(lib, name)
     for what, (op, KT) in ops.items():
         r = measure(lib, op, KT)
         m = r["phases_us"]
@@ -137,6 +165,10 @@ def run(lib, name):
                   f"{' '.join(f'{v:.0f}' for v in s['next'])}; steady {s['steady']:.0f}; last two {' '.join(f'{v:.0f}' for v in s['last'])}")
         if r["ends_us"]:
             print(f"   workgroups end at (us from the first start): min {r['ends_us'][0]:.0f} median {r['ends_us'][1]:.0f} max {r['ends_us'][2]:.0f}")
+    for what, op in dw_ops.items():
+        r = measure_dw(lib, op)
+        print(f"{name} {what}: launch {r['launch_us']:.0f} us; {r['tiles']} tiles of {r['steps']:.1f} K steps (mean); cycles: prologue {r['prologue']:.0f}, "
+              f"loop {r['per_step']:.0f} per K step, epilogue {r['epilogue']:.0f}, whole tile {r['tile']:.0f}", flush=True)
 
 
 if __name__ == "__main__":

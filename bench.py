@@ -49,14 +49,14 @@ WORKLOADS = {
 # run; the roofline block carries the one of the kernel it names.
 MEASURED_TRAFFIC_BYTES = {
     "c3": {
-        "up_swiglu": 9.00e9,  # 7.59 GB fetched + 1.41 GB written (3.42 GB algorithmic)
-        "down": 3.69e9,  # three launches: whole tiles, K slices of the last round, their sum
-        "dx2_swiglu_bwd": 6.77e9,
+        "up_swiglu": 8.79e9,  # 7.38 GB fetched + 1.41 GB written (3.42 GB algorithmic)
+        "down": 3.74e9,  # three launches: whole tiles, K slices of the last round, their sum
+        "dx2_swiglu_bwd": 6.51e9,
         "dw2": 3.76e9,
-        "dw1": 7.52e9,
-        "dx1": 7.39e9,  # three launches
+        "dw1": 7.52e9,  # 5.64 GB fetched + 1.88 GB written (2.95 GB algorithmic)
+        "dx1": 7.59e9,  # three launches
     },
-    "c2": 92.2e6,  # route: unit histogram 18.9 MB + scan 0.6 MB + scatter 72.7 MB (36.1 MB fetched + 56.2 MB written)
+    "c2": 92.2e6,  # route: unit histogram 18.9 MB + scan 0.6 MB + scatter 72.7 MB (36.1 MB fetched + 56.1 MB written)
 }
 TRAFFIC_SOURCE = "profiles/hbm_traffic_c3_c2_pmc.md (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE; a constant, not measured in this run)"
 
