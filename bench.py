@@ -554,6 +554,8 @@ def run_small_t(args):
         set_seed(0)
         moe = MoE(E, k, H, I, swiglu_packed, True, add_bias=False, std=0.02).to(torch.bfloat16).cuda()
         for T in (7, 64):
+            if args.only not in f"E{E}_k{k}_H{H}_I{I}_T{T}":
+                continue
             x = torch.randn(T, H, device="cuda").to(torch.bfloat16).requires_grad_()
             lg = torch.randn(T, E, device="cuda").to(torch.bfloat16).requires_grad_()
             grad = torch.randn(T, H, device="cuda").to(torch.bfloat16)
@@ -589,6 +591,8 @@ def run_small_t(args):
             }
         del moe
         torch.cuda.empty_cache()
+    if not res:
+        sys.exit(f"small_t: no case name contains {args.only!r}")
     first = next(iter(res.values()))
     print(json.dumps({"metric": "moe_small_t_fwd_bwd_latency_ms", "value": first["graph_ms"], "unit": "ms", "n_gpus": 1,
                       "steps": args.steps, "warmup": args.warmup, "ms_per_step": first["graph_ms"], "higher_is_better": False,
@@ -688,6 +692,7 @@ def main():
     ap.add_argument("--cpu-fraction", type=int, default=1, help="CPU baseline runs on T / this many tokens")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true", help="c3 only: leave out the summary of c4, c5 and c2")
+    ap.add_argument("--only", default="", help="small_t only: run the cases whose name contains this text (e.g. E8_k2_H2048_I8192_T7)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build measures one GPU; --gpus N with N > 1 is not supported (no collectives in the path)")
