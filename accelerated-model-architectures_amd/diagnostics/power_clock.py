@@ -7,6 +7,9 @@ Each kernel is launched back to back for a few seconds while a thread samples th
 (/sys/class/drm/card*/device/hwmon/hwmon*/power1_input, microwatts) every 20 ms; the first third of the samples is
 dropped.  Printed per kernel: milliseconds per call, mean watts, joules per call, and the energy per FLOP.  A kernel
 that sits at the board's power limit runs as fast as its energy per FLOP allows, whatever its instruction stream does.
+The lines marked `zeros:` repeat a launch with every matrix operand cleared: the same instructions and the same memory
+traffic, but nothing toggles in the matrix pipes, so the launch shows how fast its instruction stream runs when power
+does not hold the clock down.
 """
 
 from __future__ import annotations
@@ -67,7 +70,7 @@ def measure(name, fn, flops, paths, secs=2.5):
     ms = s.elapsed_time(e) / max(n, 1)
     kept = samples[len(samples) // 3:]
     watts = sum(kept) / max(len(kept), 1)
-    line = f"{name:34s} {ms:8.3f} ms/call  {watts:7.0f} W  {watts * ms * 1e-3:6.3f} J/call"
+    line = f"{name:44s} {ms:8.3f} ms/call  {watts:7.0f} W  {watts * ms * 1e-3:6.3f} J/call"
     if flops:
         line += f"  {flops / ms / 1e9:7.0f} TFLOP/s  {watts * ms * 1e-3 / flops * 1e12:5.2f} pJ/FLOP"
     print(line, flush=True)
@@ -93,13 +96,20 @@ def main():
     rnd = (torch.rand(16 * 256 * 8, device="cuda") * 4 - 2).to(torch.bfloat16)
     for label, opnd in (("MFMA stream, random operands", rnd), ("MFMA stream, zero operands", torch.zeros_like(rnd))):
         measure(label, lambda: check(lib.xma_rocm_diag_mfma_stream(opnd.data_ptr(), iters, out.data_ptr(), cus, st), "diag"), stream_flops, paths)
-    ops, dw_ops, keep = tile_phases.make_ops(lib, "c3")
+    ops, dw_ops, keep = tile_phases.make_ops(lib, "c3", split_last_round=True)
     T, H, I, E, k, _ = tile_phases.WORKLOADS["c3"]
     f = 2.0 * T * k * H * I
     for (what, (op, _kt)), fl in zip(ops.items(), (2 * f, f, f, 2 * f)):
         measure("grouped " + what, op, fl, paths)
     for (what, op), fl in zip(dw_ops.items(), (f, 2 * f)):
         measure("grouped " + what, op, fl, paths)
+    del ops, dw_ops, keep
+    # the same launches on all-zero operands: same instructions, same memory traffic, but the matrix pipes toggle nothing
+    ops, dw_ops, keep = tile_phases.make_ops(lib, "c3", split_last_round=True, zero_operands=True)
+    for (what, (op, _kt)), fl in zip(ops.items(), (2 * f, f, f, 2 * f)):
+        measure("zeros: grouped " + what, op, fl, paths)
+    for (what, op), fl in zip(dw_ops.items(), (f, 2 * f)):
+        measure("zeros: grouped " + what, op, fl, paths)
     g = torch.Generator(device="cuda").manual_seed(0)
     Tk = T * k
     xg = torch.randn(Tk, H, device="cuda", generator=g).to(torch.bfloat16)
@@ -111,6 +121,9 @@ def main():
     dz = torch.randn(Tk, 2 * I, device="cuda", generator=g).to(torch.bfloat16)
     measure("stock dy @ W, dX1 size", lambda: dz @ w1, 2 * f, paths)
     measure("stock dy^T @ x, dW1 size", lambda: dz.t() @ xg, 2 * f, paths)
+    xg.zero_()
+    w1.zero_()
+    measure("zeros: stock x @ W^T, up-projection size", lambda: torch.nn.functional.linear(xg, w1), 2 * f, paths)
     del keep
 
 

@@ -54,8 +54,11 @@ def load(path=None):
     return lib
 
 
-def make_ops(lib, name):
-    """the four forward-type GEMMs of a workload as closures, with their K step counts"""
+def make_ops(lib, name, split_last_round=False, zero_operands=False):
+    """the four forward-type GEMMs of a workload as closures, with their K step counts, and the two weight-gradient GEMMs;
+    split_last_round passes the workspace that lets a launch cut the tiles of its last, partial round into K slices (what
+    the layer does), otherwise every tile is computed by one workgroup (what the stamps of this script describe);
+    zero_operands clears every matrix operand (same instruction stream, same addresses, nothing toggles in the matrix pipes)"""
     T, H, I, E, k, bias = WORKLOADS[name]
     dev, bf = "cuda", torch.bfloat16
     g = torch.Generator(device=dev).manual_seed(0)
@@ -78,9 +81,18 @@ def make_ops(lib, name):
     dw1 = torch.empty(E, 2 * I, H, device=dev, dtype=bf)
     dw2 = torch.empty(E, H, I, device=dev, dtype=bf)
     keep = (x, w1, w2, ss, offs, z, h, dz, dy, rw, eo, gdy, dw1, dw2)
+    if zero_operands:
+        for t in (x, w1, w2, h, dz, dy, gdy, z):
+            t.zero_()
+
+    ws = {}
 
     def s2s(*a):
-        rc = lib.xma_rocm_scatter2scatter(*a, None, 0, st)
+        M, N, K = a[13], a[14], a[15]
+        nbytes = lib.xma_rocm_scatter2scatter_workspace_bytes(M, N, K, E) if split_last_round else 0
+        if nbytes and (N, K) not in ws:
+            ws[(N, K)] = torch.empty(nbytes, dtype=torch.uint8, device=dev)
+        rc = lib.xma_rocm_scatter2scatter(*a, ws[(N, K)].data_ptr() if nbytes else None, nbytes, st)
         assert rc == 0, lib.xma_rocm_last_error()
 
     return {
