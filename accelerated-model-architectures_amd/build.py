@@ -16,7 +16,7 @@ CSRC = os.path.join(HERE, "csrc")
 INCLUDE = os.path.join(os.path.dirname(HERE), "include")
 OUT_DIR = os.path.join(HERE, "xma", "rocm")
 LIB = os.path.join(OUT_DIR, "libxma_rocm.so")
-SOURCES = ["api.hip", "routing.hip", "elementwise.hip", "grouped_gemm.hip", "grouped_gemm_staged.hip", "fp32.hip", "router.hip", "swiglu.hip", "bias.hip", "diagnostics.hip"]
+SOURCES = ["api.hip", "routing.hip", "elementwise.hip", "grouped_gemm.hip", "grouped_gemm_staged.hip", "fp32.hip", "router.hip", "swiglu.hip", "bias.hip", "few_rows.hip", "diagnostics.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [

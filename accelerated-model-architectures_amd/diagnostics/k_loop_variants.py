@@ -32,7 +32,7 @@ PKG = os.path.dirname(HERE)
 OUT = os.path.join(HERE, "variants")  # generated sources and libraries: not tracked, but they travel to the GPU box
 VARIANTS = ["base", "novm", "nowait", "nodma", "noreads", "lead2"]
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-OTHER_OBJECTS = ["api", "routing", "elementwise", "grouped_gemm_staged", "fp32", "router", "swiglu", "bias", "diagnostics"]
+OTHER_OBJECTS = ["api", "routing", "elementwise", "grouped_gemm_staged", "fp32", "router", "swiglu", "bias", "few_rows", "diagnostics"]
 
 
 def _sub(s: str, old: str, new: str) -> str:

@@ -82,6 +82,9 @@ def continuous_count_rocm(x: torch.Tensor, y: torch.Tensor, workspace: torch.Ten
 
 
 CONTINUOUS_COUNT_SET_MAX_BINS = 8192
+# Up to this many rows in total (tokens x experts per token) the grouped GEMMs take the entry points written for the
+# few-token regime, which stream the weights instead of tiling them for the matrix pipes.
+FEW_ROWS_MAX = 64
 
 
 @torch.library.custom_op("xma_rocm::continuous_count_set", mutates_args={"y"})
@@ -302,14 +305,17 @@ def group_bwd_W_rocm(
     if dy_scale is not None:
         assert dy_scale.dtype == DY.dtype and dy_scale.is_contiguous()
     lib = get_library()
+    # a handful of rows in total (the index has one entry per row): the launch is a stream of stores, not arithmetic
+    few = sorted_scattered_idxs.numel() <= FEW_ROWS_MAX and DW.dtype in (torch.bfloat16, torch.float16)
+    name = "xma_rocm_group_bwd_W_few_rows" if few else "xma_rocm_group_bwd_W"
     check(
-        lib.xma_rocm_group_bwd_W(
+        getattr(lib, name)(
             _ptr(DY), _rows(DY, "DY"), int(dy_fan_out == 0), max(dy_fan_out, 1), _ptr(dy_scale),
             _ptr(X), _rows(X, "X"), int(x_fan_out == 0), max(x_fan_out, 1),
             _ptr(sorted_scattered_idxs), _ptr(expert_offsets), _ptr(DW), DW.stride(0), DW.stride(2),
             N_out, K_in, E, _code(X), _stream(X),
         ),
-        "xma_rocm_group_bwd_W",
+        name,
     )
 
 

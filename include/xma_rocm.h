@@ -214,6 +214,20 @@ XMA_API int xma_rocm_group_bwd_W(const void *DY, int64_t lddy, int dy_grouped, i
                          int dtype, void *stream);
 
 /*
+ * xma_rocm_group_bwd_W for the few-token regime (same arguments, same result up to the order of the fp32 sums; bf16 /
+ * fp16 only; DY needs no 16-byte alignment and N_out no multiple of 8).  One workgroup per 8 rows of DW[e] streams its
+ * stores and adds one outer product per row of the expert with vector FMAs: with a handful of rows per expert the launch
+ * runs at the rate of a fill of DW, where the MFMA tiles of xma_rocm_group_bwd_W spend a prologue, one K step and an
+ * epilogue per 256 x 256 tile.  Correct for any number of rows, but its time grows with rows x |DW|: meant for launches
+ * of at most a few dozen rows in total.  No counterpart in the reference (its kernel is the same for every size).
+ */
+XMA_API int xma_rocm_group_bwd_W_few_rows(const void *DY, int64_t lddy, int dy_grouped, int32_t dy_fan_out,
+                                  const void *dy_scale, const void *X, int64_t ldx, int x_grouped, int32_t x_fan_out,
+                                  const int64_t *sorted_scattered_idxs, const int64_t *expert_offsets, void *DW,
+                                  int64_t dw_expert_stride, int64_t lddw, int32_t N_out, int32_t K_in,
+                                  int32_t num_experts, int dtype, void *stream);
+
+/*
  * Gather copy: out[n, :] = A[idx[n] / fan_out, :] * (coeff ? coeff[idx[n]] : 1), n < M.
  * Replaces group, xma/layers/moe/triton_implementation/group_kernel.py:69-100.
  */

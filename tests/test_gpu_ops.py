@@ -29,6 +29,30 @@ def _routing(T, E, k, seed, skew=0.0, empty=()):
     return sel, se, ss, offs
 
 
+class _few_rows_limit:
+    """the limit below which the ops take the few-token entry points, set for the length of a with block (0: never)"""
+
+    def __init__(self, limit):
+        self.limit = limit
+
+    def __enter__(self):
+        from xma.rocm import ops
+
+        self.saved, ops.FEW_ROWS_MAX = ops.FEW_ROWS_MAX, self.limit
+
+    def __exit__(self, *exc):
+        from xma.rocm import ops
+
+        ops.FEW_ROWS_MAX = self.saved
+
+
+def _limits(rows):
+    """both code paths where the number of rows would pick the few-token one, else the only one there is"""
+    from xma.rocm import ops
+
+    return (0, ops.FEW_ROWS_MAX) if rows <= ops.FEW_ROWS_MAX else (ops.FEW_ROWS_MAX,)
+
+
 CASES = [
     # T, E, k, K, N, skew, empty experts
     (7, 4, 2, 64, 64, 0.0, ()),
@@ -253,15 +277,17 @@ def test_group_bwd_W_expert_row_counts(dtype, case):
     x_grp = torch.randn(M, K, generator=g).to(dtype)
     for X, x_fan, want in [(x_grp, 0, oracle.group_bwd_W(dy_grp, x_grp, offs, E)),
                            (x_tok, k, oracle.group_bwd_W(dy_grp, oracle.group(x_tok, ss, None, k), offs, E))]:
-        DW = torch.full((E, N, K), float("nan"), dtype=dtype, device="cuda").permute(0, 2, 1)
-        ops.group_bwd_W_rocm(dy_grp.cuda(), X.cuda(), ss.cuda(), offs.cuda(), DW, None, 0, x_fan)
-        torch.cuda.synchronize()
-        assert torch.isfinite(DW).all()
-        for e in range(E):  # every expert's slice against its own magnitude
-            if counts[e] == 0:
-                assert (DW[e] == 0).all()
-            else:
-                assert nerr(DW[e], want[e]) <= _tol(dtype), e
+        for limit in _limits(M):
+            DW = torch.full((E, N, K), float("nan"), dtype=dtype, device="cuda").permute(0, 2, 1)
+            with _few_rows_limit(limit):
+                ops.group_bwd_W_rocm(dy_grp.cuda(), X.cuda(), ss.cuda(), offs.cuda(), DW, None, 0, x_fan)
+            torch.cuda.synchronize()
+            assert torch.isfinite(DW).all()
+            for e in range(E):  # every expert's slice against its own magnitude
+                if counts[e] == 0:
+                    assert (DW[e] == 0).all()
+                else:
+                    assert nerr(DW[e], want[e]) <= _tol(dtype), (e, limit)
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
@@ -288,17 +314,62 @@ def test_group_bwd_W(dtype, case):
         assert torch.isfinite(DW).all()
         return DW
 
-    # both grouped (the reference op), x gathered (dW1), dy gathered and scaled (dW2)
-    want = oracle.group_bwd_W(dy_grp, x_grp, offs, E)
-    assert nerr(run(dy_grp, x_grp, None, 0, 0), want) <= _tol(dtype)
-    want = oracle.group_bwd_W(dy_grp, oracle.group(x_tok, ss, None, k), offs, E)
-    assert nerr(run(dy_grp, x_tok, None, 0, k), want) <= _tol(dtype)
-    want = oracle.group_bwd_W(oracle.group(dy_tok, ss, scale, k), x_grp, offs, E)
-    assert nerr(run(dy_tok, x_grp, scale, k, 0), want) <= _tol(dtype)
-    # experts without rows get an all-zero slice
-    got = run(dy_grp, x_grp, None, 0, 0)
-    for e in empty:
-        assert (got[e] == 0).all()
+    for limit in _limits(M):
+        with _few_rows_limit(limit):
+            # both grouped (the reference op), x gathered (dW1), dy gathered and scaled (dW2)
+            want = oracle.group_bwd_W(dy_grp, x_grp, offs, E)
+            assert nerr(run(dy_grp, x_grp, None, 0, 0), want) <= _tol(dtype)
+            want = oracle.group_bwd_W(dy_grp, oracle.group(x_tok, ss, None, k), offs, E)
+            assert nerr(run(dy_grp, x_tok, None, 0, k), want) <= _tol(dtype)
+            want = oracle.group_bwd_W(oracle.group(dy_tok, ss, scale, k), x_grp, offs, E)
+            assert nerr(run(dy_tok, x_grp, scale, k, 0), want) <= _tol(dtype)
+            # experts without rows get an all-zero slice
+            got = run(dy_grp, x_grp, None, 0, 0)
+            for e in empty:
+                assert (got[e] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", [(7, 8, 2, 264, 136, ()), (3, 128, 8, 576, 512, ()), (16, 4, 4, 2048, 72, (2,)), (1, 8, 1, 64, 8, ()),
+                                  (9, 5, 3, 4104, 24, (0, 4))])
+def test_group_bwd_W_few_rows(dtype, case):
+    """The weight gradient written for a handful of rows (an outer product per row, streamed stores) against the oracle
+    and against the MFMA kernel on the same operands: every operand form of the layer, more than 2048 columns (two column blocks, the second partly filled), experts without rows (zeros), more experts than rows."""
+    from xma.rocm import ops
+
+    T, E, k, K, N, empty = case
+    print(f"case T={T} E={E} k={k} K={K} N={N} {dtype}", flush=True)
+    sel, se, ss, offs = _routing(T, E, k, 21, 0.0, empty)
+    M = T * k
+    assert M <= ops.FEW_ROWS_MAX
+    g = torch.Generator().manual_seed(22)
+    x_tok = torch.randn(T, K, generator=g).to(dtype)
+    dy_tok = torch.randn(T, N, generator=g).to(dtype)
+    dy_grp = torch.randn(M, N, generator=g).to(dtype)
+    x_grp = torch.randn(M, K, generator=g).to(dtype)
+    scale = torch.rand(M, generator=g).to(dtype)
+    forms = [(dy_grp, x_grp, None, 0, 0, oracle.group_bwd_W(dy_grp, x_grp, offs, E)),
+             (dy_grp, x_tok, None, 0, k, oracle.group_bwd_W(dy_grp, oracle.group(x_tok, ss, None, k), offs, E)),
+             (dy_tok, x_grp, scale, k, 0, oracle.group_bwd_W(oracle.group(dy_tok, ss, scale, k), x_grp, offs, E)),
+             (dy_tok, x_grp, None, k, 0, oracle.group_bwd_W(oracle.group(dy_tok, ss, None, k), x_grp, offs, E))]
+    counts = torch.bincount(se, minlength=E)
+    for DY, X, sc, dy_fan, x_fan, want in forms:
+        got = {}
+        for limit in (0, ops.FEW_ROWS_MAX):
+            DW = torch.full((E, N, K), float("nan"), dtype=dtype, device="cuda").permute(0, 2, 1)
+            with _few_rows_limit(limit):
+                ops.group_bwd_W_rocm(DY.cuda(), X.cuda(), ss.cuda(), offs.cuda(), DW, None if sc is None else sc.cuda(), dy_fan, x_fan)
+            torch.cuda.synchronize()
+            assert torch.isfinite(DW).all()
+            got[limit] = DW
+        few, mfma = got[ops.FEW_ROWS_MAX], got[0]
+        assert nerr(few, want) <= _tol(dtype)
+        assert nerr(few, mfma) <= _tol(dtype)
+        for e in range(E):
+            if counts[e] == 0:
+                assert (few[e] == 0).all()
+            else:
+                assert nerr(few[e], want[e]) <= _tol(dtype), e
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
