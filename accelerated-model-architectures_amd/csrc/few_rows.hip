@@ -11,6 +11,7 @@ namespace {
 constexpr int FR_THREADS = 256;
 constexpr int FR_NB = 8; // output rows (n) per workgroup of the weight gradient
 constexpr int FR_RC = 4; // rows of the expert per step
+constexpr int FR_GROUPS = 8; // sets of FR_NB rows n per workgroup, at most (rows of DW of 32 pieces of 16 bytes or more fill it)
 
 template <typename T> __device__ __forceinline__ float fr_scalar(const uint16_t *p, int64_t i) { return Elem<T>::lo(p[i]); }
 
@@ -20,15 +21,21 @@ template <typename T> __device__ __forceinline__ void fr_unpack(const u32x4 v, f
 }
 
 // DW[e][n][k] = sum over the rows r of expert e of DY[dsrc(r)][n] * scale[idx[r]] * X[xsrc(r)][k]: an outer product per
-// row.  Workgroup = (2048 columns k, FR_NB rows n, expert); a thread owns 8 consecutive k of every n: it loads its 16 bytes
+// row.  Workgroup = (2048 columns k, FR_NB rows n, expert), or several sets of FR_NB rows when a row of DW is shorter than
+// the workgroup; a thread owns 8 consecutive k of every n of its set: it loads its 16 bytes
 // of each X row once, takes the FR_NB values of DY from LDS, and leaves FR_NB stores of 16 bytes.  fp32 sums in row order.
 // Every element of DW is written exactly once, zeros for an expert without rows.
 template <typename T> __global__ __launch_bounds__(FR_THREADS) void dw_few_rows_kernel(const DwArgs a) {
-    __shared__ float s_dy[2][FR_RC][FR_NB];
+    __shared__ float s_dy[2][FR_GROUPS][FR_RC][FR_NB];
     const int e = blockIdx.z, tid = threadIdx.x;
-    const int n0 = blockIdx.y * FR_NB;
-    const int k0 = (blockIdx.x * FR_THREADS + tid) * 8;
-    const bool k_ok = k0 < a.K_in;
+    // a row of DW shorter than the workgroup: `groups` sets of FR_NB rows n side by side, `cpr` threads each
+    const int cpr = a.K_in >> 3;
+    int groups = (cpr < FR_THREADS) ? FR_THREADS / cpr : 1;
+    if (groups > FR_GROUPS) groups = FR_GROUPS;
+    const int grp = (groups > 1) ? tid / cpr : 0;
+    const int n0 = (blockIdx.y * groups + grp) * FR_NB;
+    const int k0 = (groups > 1) ? (tid - grp * cpr) * 8 : (blockIdx.x * FR_THREADS + tid) * 8;
+    const bool k_ok = k0 < a.K_in && grp < groups;
     const int64_t lo = e ? a.offs[e - 1] : 0, hi = a.offs[e];
     float acc[FR_NB][8];
 #pragma unroll
@@ -37,17 +44,18 @@ template <typename T> __global__ __launch_bounds__(FR_THREADS) void dw_few_rows_
         for (int i = 0; i < 8; ++i) acc[j][i] = 0.f;
     int buf = 0;
     for (int64_t r0 = lo; r0 < hi; r0 += FR_RC, buf ^= 1) {
-        if (tid < FR_RC * FR_NB) { // the step's FR_RC x FR_NB values of dY, scaled
-            const int u = tid / FR_NB, j = tid % FR_NB;
+        if (tid < groups * FR_RC * FR_NB) { // the step's FR_RC x FR_NB values of dY of every group, scaled
+            const int gq = tid / (FR_RC * FR_NB), u = (tid / FR_NB) % FR_RC, j = tid % FR_NB;
             const int64_t r = r0 + u;
+            const int n = (blockIdx.y * groups + gq) * FR_NB + j;
             float v = 0.f;
-            if (r < hi && n0 + j < a.N_out) {
+            if (r < hi && n < a.N_out) {
                 const int64_t s = a.idx ? a.idx[r] : r;
                 const int64_t src = a.dy_grouped ? r : (int64_t)fastdiv((uint32_t)s, a.dy_div);
-                v = fr_scalar<T>(a.DY, src * a.lddy + n0 + j);
+                v = fr_scalar<T>(a.DY, src * a.lddy + n);
                 if (a.scale) v *= fr_scalar<T>(a.scale, s);
             }
-            s_dy[buf][u][j] = v;
+            s_dy[buf][gq][u][j] = v;
         }
         u32x4 x[FR_RC];
 #pragma unroll
@@ -66,7 +74,7 @@ template <typename T> __global__ __launch_bounds__(FR_THREADS) void dw_few_rows_
             fr_unpack<T>(x[u], xf);
 #pragma unroll
             for (int j = 0; j < FR_NB; ++j) {
-                const float d = s_dy[buf][u][j];
+                const float d = s_dy[buf][grp < groups ? grp : 0][u][j];
 #pragma unroll
                 for (int i = 0; i < 8; ++i) acc[j][i] = __builtin_fmaf(d, xf[i], acc[j][i]);
             }
@@ -101,7 +109,10 @@ extern "C" int xma_rocm_group_bwd_W_few_rows(const void *DY, int64_t lddy, int d
                 XMA_ROCM_EINVAL, "group_bwd_W_few_rows: null or misaligned operand");
     XMA_REQUIRE(sorted_scattered_idxs || (dy_grouped && x_grouped && !dy_scale), XMA_ROCM_EINVAL,
                 "group_bwd_W_few_rows: sorted_scattered_idxs is required unless everything is grouped");
-    const int64_t rows_n = ((int64_t)N_out + FR_NB - 1) / FR_NB;
+    const int cpr = K_in / 8;
+    int groups = (cpr < FR_THREADS) ? FR_THREADS / cpr : 1;
+    if (groups > FR_GROUPS) groups = FR_GROUPS;
+    const int64_t rows_n = ((int64_t)N_out + FR_NB * groups - 1) / (FR_NB * groups);
     XMA_REQUIRE(rows_n <= 65535, XMA_ROCM_EUNSUPPORTED, "group_bwd_W_few_rows: N_out=%d exceeds %d", N_out, 65535 * FR_NB);
     DwArgs a;
     a.DY = (const uint16_t *)DY;
@@ -123,11 +134,364 @@ extern "C" int xma_rocm_group_bwd_W_few_rows(const void *DY, int64_t lddy, int d
     a.x_fan_out = x_fan_out;
     a.dy_div = make_fastdiv((uint32_t)dy_fan_out);
     a.x_div = make_fastdiv((uint32_t)x_fan_out);
-    const dim3 grid((K_in / 8 + FR_THREADS - 1) / FR_THREADS, (unsigned)rows_n, E);
+    const dim3 grid(groups > 1 ? 1 : (cpr + FR_THREADS - 1) / FR_THREADS, (unsigned)rows_n, E);
     hipStream_t st = (hipStream_t)stream;
     if (dtype == XMA_ROCM_BF16)
         dw_few_rows_kernel<__bf16><<<grid, FR_THREADS, 0, st>>>(a);
     else
         dw_few_rows_kernel<_Float16><<<grid, FR_THREADS, 0, st>>>(a);
     return xma_check_launch("dw_few_rows_kernel");
+}
+
+namespace {
+
+// ------------------------------------------------------------------------------------------------
+// Forward-type product for a handful of rows: acc[r][n] = sum_k X[src(r)][k] * B_e[k][n] in fp32, written to a workspace
+// part[S][M][N] as S partial sums over K ranges, then one small kernel that adds the parts in order and runs the epilogue.
+//   W[e] as (N, K), K contiguous (x @ W^T): a wave takes two rows of W at a time, its lanes split K in 16-byte pieces,
+//       the expert's rows of X wait in LDS, and the lanes' partial dot products meet in a butterfly.  S = 1.
+//   W[e] as (K, N), N contiguous (dy @ W): a thread owns 8 columns n and walks the rows k of its workgroup's K range;
+//       the X values of the range sit in LDS as floats.  S = K / range.
+// ------------------------------------------------------------------------------------------------
+constexpr int FR_NT_ROWS = 32;  // rows of W per workgroup (8 per wave, two at a time); 8 when the rows are short
+constexpr int FR_NT_KMAX = 8192; // the X rows of a step are staged whole: RC x K 16-bit values in LDS
+
+__device__ __forceinline__ int64_t fr_src_row(const FwdArgs &a, int64_t r) {
+    return a.x_grouped ? r : (int64_t)fastdiv((uint32_t)a.idx[r], a.fan_div);
+}
+
+template <typename T, int RC>
+__device__ __forceinline__ void fr_nt_rows(const FwdArgs &a, float *__restrict__ part, uint16_t *s_x, int e, int64_t lo,
+                                           int64_t hi, int n_first, int n_count) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int chunks = a.K >> 3; // 16-byte pieces of a row
+    for (int64_t r0 = lo; r0 < hi; r0 += RC) {
+        __syncthreads(); // the rows of the step before are no longer read
+        for (int i = tid; i < RC * chunks; i += FR_THREADS) {
+            const int u = i / chunks, c = i - u * chunks;
+            u32x4 v = {0u, 0u, 0u, 0u};
+            if (r0 + u < hi) v = *(const u32x4 *)(a.X + fr_src_row(a, r0 + u) * a.ldx + 8 * c);
+            *(u32x4 *)(s_x + ((int64_t)u * chunks + c) * 8) = v;
+        }
+        __syncthreads();
+        for (int p = wave * 2; p < n_count; p += 2 * (FR_THREADS / 64)) { // rows p, p + 1 of the workgroup's block
+            const int n_a = n_first + p, n_b = (p + 1 < n_count) ? n_a + 1 : n_a;
+            const uint16_t *w_a = a.W + (int64_t)e * a.w_es + (int64_t)n_a * a.ldw;
+            const uint16_t *w_b = a.W + (int64_t)e * a.w_es + (int64_t)n_b * a.ldw;
+            float s[RC][2];
+#pragma unroll
+            for (int u = 0; u < RC; ++u) s[u][0] = s[u][1] = 0.f;
+            for (int c0 = lane; c0 < chunks; c0 += 4 * 64) { // up to four pieces of either row in flight per lane
+                u32x4 wa[4], wb[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int c = c0 + 64 * q;
+                    wa[q] = wb[q] = u32x4{0u, 0u, 0u, 0u};
+                    if (c < chunks) {
+                        wa[q] = __builtin_nontemporal_load((const u32x4 *)(w_a + 8 * c));
+                        wb[q] = __builtin_nontemporal_load((const u32x4 *)(w_b + 8 * c));
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int c = c0 + 64 * q;
+                    if (c < chunks) {
+                        float fa[8], fb[8];
+                        fr_unpack<T>(wa[q], fa);
+                        fr_unpack<T>(wb[q], fb);
+#pragma unroll
+                        for (int u = 0; u < RC; ++u) {
+                            float fx[8];
+                            fr_unpack<T>(*(const u32x4 *)(s_x + ((int64_t)u * chunks + c) * 8), fx);
+#pragma unroll
+                            for (int i = 0; i < 8; ++i) {
+                                s[u][0] = __builtin_fmaf(fx[i], fa[i], s[u][0]);
+                                s[u][1] = __builtin_fmaf(fx[i], fb[i], s[u][1]);
+                            }
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < RC; ++u)
+#pragma unroll
+                for (int h = 0; h < 2; ++h)
+#pragma unroll
+                    for (int d = 32; d > 0; d >>= 1) s[u][h] += __shfl_xor(s[u][h], d);
+            if (lane == 0) {
+#pragma unroll
+                for (int u = 0; u < RC; ++u) {
+                    if (r0 + u < hi) {
+                        part[(r0 + u) * a.N + n_a] = s[u][0];
+                        if (p + 1 < n_count) part[(r0 + u) * a.N + n_b] = s[u][1];
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(FR_THREADS) void fr_nt_kernel(const FwdArgs a, float *__restrict__ part, int rows_per_wg) {
+    extern __shared__ __attribute__((aligned(16))) uint16_t s_x_nt[];
+    const int e = blockIdx.y;
+    const int64_t lo = e ? a.offs[e - 1] : 0, hi = a.offs[e];
+    if (lo >= hi) return; // uniform
+    const int n_first = blockIdx.x * rows_per_wg;
+    const int n_count = (a.N - n_first < rows_per_wg) ? a.N - n_first : rows_per_wg;
+    if (hi - lo <= 2)
+        fr_nt_rows<T, 2>(a, part, s_x_nt, e, lo, hi, n_first, n_count);
+    else
+        fr_nt_rows<T, 4>(a, part, s_x_nt, e, lo, hi, n_first, n_count);
+}
+
+constexpr int FR_NN_KC_MIN = 32;  // rows k of W per workgroup, at least (four rounds of eight loads per thread)
+constexpr int FR_NN_SPLITS = 64;  // K ranges, at most
+constexpr int FR_NN_KC_MAX = 1024; // 8 rows x range floats in LDS: 32 KB
+
+inline int fr_nn_range(int K) {
+    int kc = (K + FR_NN_SPLITS - 1) / FR_NN_SPLITS;
+    if (kc < FR_NN_KC_MIN) kc = FR_NN_KC_MIN;
+    return kc;
+}
+
+template <typename T, int RC>
+__device__ __forceinline__ void fr_nn_rows(const FwdArgs &a, float *__restrict__ part, float *s_x, int e, int64_t lo,
+                                           int64_t hi, int k_lo, int k_hi, int n_t, bool n_ok) {
+    const int tid = threadIdx.x;
+    const int kc = k_hi - k_lo;
+    const uint16_t *w = a.W + (int64_t)e * a.w_es + (int64_t)k_lo * a.ldw + n_t;
+    for (int64_t r0 = lo; r0 < hi; r0 += RC) {
+        __syncthreads();
+        for (int i = tid; i < RC * kc; i += FR_THREADS) {
+            const int u = i / kc, k = i - u * kc;
+            s_x[i] = (r0 + u < hi) ? fr_scalar<T>(a.X, fr_src_row(a, r0 + u) * a.ldx + k_lo + k) : 0.f;
+        }
+        __syncthreads();
+        float acc[RC][8];
+#pragma unroll
+        for (int u = 0; u < RC; ++u)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[u][i] = 0.f;
+        if (n_ok) {
+            for (int k0 = 0; k0 < kc; k0 += 8) { // eight rows of W in flight per thread
+                u32x4 wv[8];
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    wv[q] = u32x4{0u, 0u, 0u, 0u};
+                    if (k0 + q < kc) wv[q] = __builtin_nontemporal_load((const u32x4 *)(w + (int64_t)(k0 + q) * a.ldw));
+                }
+#pragma unroll
+                for (int q = 0; q < 8; ++q) {
+                    if (k0 + q < kc) {
+                        float fw[8];
+                        fr_unpack<T>(wv[q], fw);
+#pragma unroll
+                        for (int u = 0; u < RC; ++u) {
+                            const float xv = s_x[u * kc + k0 + q];
+#pragma unroll
+                            for (int i = 0; i < 8; ++i) acc[u][i] = __builtin_fmaf(xv, fw[i], acc[u][i]);
+                        }
+                    }
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < RC; ++u) {
+                if (r0 + u < hi) {
+                    float4 *o = (float4 *)(part + (r0 + u) * a.N + n_t);
+                    o[0] = make_float4(acc[u][0], acc[u][1], acc[u][2], acc[u][3]);
+                    o[1] = make_float4(acc[u][4], acc[u][5], acc[u][6], acc[u][7]);
+                }
+            }
+        }
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(FR_THREADS) void fr_nn_kernel(const FwdArgs a, float *__restrict__ part, int kc) {
+    extern __shared__ __attribute__((aligned(16))) float s_x_nn[];
+    const int e = blockIdx.z, split = blockIdx.y;
+    const int64_t lo = e ? a.offs[e - 1] : 0, hi = a.offs[e];
+    if (lo >= hi) return; // uniform
+    const int k_lo = split * kc, k_hi = (k_lo + kc < a.K) ? k_lo + kc : a.K;
+    const int n_t = (blockIdx.x * FR_THREADS + threadIdx.x) * 8;
+    float *mine = part + (int64_t)split * a.M * a.N;
+    if (hi - lo <= 2)
+        fr_nn_rows<T, 2>(a, mine, s_x_nn, e, lo, hi, k_lo, k_hi, n_t, n_t < a.N);
+    else if (hi - lo <= 4)
+        fr_nn_rows<T, 4>(a, mine, s_x_nn, e, lo, hi, k_lo, k_hi, n_t, n_t < a.N);
+    else
+        fr_nn_rows<T, 8>(a, mine, s_x_nn, e, lo, hi, k_lo, k_hi, n_t, n_t < a.N);
+}
+
+// One workgroup per row and 512 columns: the S parts are added in order, the bias joins, and the epilogue of the MFMA kernels is applied
+// with the same arithmetic (tile_epilogue in grouped_gemm.hip): STORE rounds acc * scale; SWIGLU rounds the
+// pre-activations and takes the activation from the rounded pair; SWIGLU_BWD turns d h = acc * scale and the stored
+// pre-activations into (d gate, d up) and, on request, the scaled activation.
+template <typename T, int EPI>
+__global__ __launch_bounds__(FR_THREADS) void fr_epilogue_kernel(const FwdArgs a, const float *__restrict__ part, int S) {
+    __shared__ int s_e;
+    const int64_t r = blockIdx.y;
+    if (threadIdx.x == 0) { // the expert of row r: first e with offs[e] > r
+        int lo = 0, hi = a.E - 1;
+        while (lo < hi) {
+            const int mid = (lo + hi) >> 1;
+            if (a.offs[mid] > r) hi = mid; else lo = mid + 1;
+        }
+        s_e = lo;
+    }
+    __syncthreads();
+    const int e = s_e;
+    const int64_t s_idx = a.idx ? a.idx[r] : r;
+    const float sc = a.scale ? fr_scalar<T>(a.scale, s_idx) : 1.f;
+    const int64_t dst = a.y_grouped ? r : s_idx;
+    const uint16_t *bias = a.bias ? a.bias + (int64_t)e * a.bias_es : nullptr;
+    const int n = 2 * (blockIdx.x * FR_THREADS + threadIdx.x); // N is even: a thread takes a pair of columns
+    if (n < a.N) {
+        float v0 = bias ? fr_scalar<T>(bias, n) : 0.f, v1 = bias ? fr_scalar<T>(bias, n + 1) : 0.f;
+        const float *p0 = part + r * a.N + n;
+        const int64_t step = a.M * a.N;
+        for (int s0 = 0; s0 < S; s0 += 8) { // eight parts in flight, added in order
+            float2 p[8];
+#pragma unroll
+            for (int q = 0; q < 8; ++q) p[q] = (s0 + q < S) ? *(const float2 *)(p0 + (s0 + q) * step) : make_float2(0.f, 0.f);
+#pragma unroll
+            for (int q = 0; q < 8; ++q) v0 += p[q].x, v1 += p[q].y;
+        }
+        if constexpr (EPI == XMA_ROCM_EPI_SWIGLU_BWD) {
+            // columns n, n + 1 of d h belong to the pairs (2n, 2n + 1) and (2n + 2, 2n + 3) of z and dz
+            const uint32_t z0 = *(const uint32_t *)(a.aux + r * a.ldaux + 2 * n), z1 = *(const uint32_t *)(a.aux + r * a.ldaux + 2 * n + 2);
+            uint32_t o[2];
+            float hv[2];
+            const uint32_t zz[2] = {z0, z1};
+            const float dh[2] = {v0 * sc, v1 * sc};
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const float gg = Elem<T>::lo(zz[q]), uu = Elem<T>::hi(zz[q]);
+                const float sg = sigmoidf_fast(gg), silu = gg * sg;
+                o[q] = Elem<T>::pack(dh[q] * uu * (sg + silu * (1.f - sg)), dh[q] * silu);
+                hv[q] = uu * silu * sc;
+            }
+            *(u32x2 *)(a.out + r * a.ldo + 2 * n) = u32x2{o[0], o[1]};
+            if (a.aux2) *(uint32_t *)(a.aux2 + r * a.ldaux2 + n) = Elem<T>::pack(hv[0], hv[1]);
+        } else {
+            const uint32_t z = Elem<T>::pack(v0 * sc, v1 * sc);
+            if (a.out) *(uint32_t *)(a.out + dst * a.ldo + n) = z;
+            if constexpr (EPI == XMA_ROCM_EPI_SWIGLU) {
+                const float g = Elem<T>::lo(z), u = Elem<T>::hi(z);
+                a.aux[dst * a.ldaux + (n >> 1)] = (uint16_t)(Elem<T>::pack(u * g * sigmoidf_fast(g), 0.f) & 0xffffu);
+            }
+        }
+    }
+}
+
+template <typename T> int fr_launch(const FwdArgs &a, int w_is_kn, int epilogue, float *part, hipStream_t st) {
+    int S = 1, rc;
+    if (w_is_kn) {
+        const int kc = fr_nn_range(a.K);
+        S = (a.K + kc - 1) / kc;
+        const dim3 grid((a.N / 8 + FR_THREADS - 1) / FR_THREADS, S, a.E);
+        fr_nn_kernel<T><<<grid, FR_THREADS, (size_t)8 * kc * sizeof(float), st>>>(a, part, kc);
+        if ((rc = xma_check_launch("fr_nn_kernel"))) return rc;
+    } else {
+        const int rows_per_wg = (a.K >= 2048) ? FR_NT_ROWS : 8; // short rows: one pair of rows per wave, more workgroups
+        const dim3 grid((a.N + rows_per_wg - 1) / rows_per_wg, a.E);
+        const size_t lds = (size_t)4 * a.K * sizeof(uint16_t);
+        if (lds > 48 * 1024 && (rc = xma_set_max_lds_once((const void *)fr_nt_kernel<T>, 4 * FR_NT_KMAX * (int)sizeof(uint16_t)))) return rc;
+        fr_nt_kernel<T><<<grid, FR_THREADS, lds, st>>>(a, part, rows_per_wg);
+        if ((rc = xma_check_launch("fr_nt_kernel"))) return rc;
+    }
+    const dim3 egrid((a.N / 2 + FR_THREADS - 1) / FR_THREADS, (unsigned)a.M);
+    if (epilogue == XMA_ROCM_EPI_STORE)
+        fr_epilogue_kernel<T, XMA_ROCM_EPI_STORE><<<egrid, FR_THREADS, 0, st>>>(a, part, S);
+    else if (epilogue == XMA_ROCM_EPI_SWIGLU)
+        fr_epilogue_kernel<T, XMA_ROCM_EPI_SWIGLU><<<egrid, FR_THREADS, 0, st>>>(a, part, S);
+    else
+        fr_epilogue_kernel<T, XMA_ROCM_EPI_SWIGLU_BWD><<<egrid, FR_THREADS, 0, st>>>(a, part, S);
+    return xma_check_launch("fr_epilogue_kernel");
+}
+
+} // namespace
+
+extern "C" size_t xma_rocm_scatter2scatter_few_rows_workspace_bytes(int64_t M, int32_t N, int32_t K, int w_is_kn) {
+    if (M <= 0 || N <= 0 || K <= 0) return 0;
+    int S = 1;
+    if (w_is_kn) {
+        const int kc = fr_nn_range(K);
+        S = (K + kc - 1) / kc;
+    }
+    return (size_t)S * (size_t)M * (size_t)N * sizeof(float);
+}
+
+extern "C" int xma_rocm_scatter2scatter_few_rows(const void *X, int64_t ldx, const void *W, int64_t w_expert_stride,
+                                                 int64_t ldw, int w_is_kn, const int64_t *sorted_scattered_idxs,
+                                                 const int64_t *expert_offsets, void *out, int64_t ldo, void *aux,
+                                                 int64_t ldaux, void *aux2, int64_t ldaux2, const void *row_scale,
+                                                 const void *bias, int64_t bias_expert_stride, int64_t M, int32_t N,
+                                                 int32_t K, int32_t E, int32_t fan_out, int x_grouped, int y_grouped,
+                                                 int epilogue, int dtype, void *workspace, size_t workspace_bytes,
+                                                 void *stream) {
+    XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED, "scatter2scatter_few_rows: dtype %d", dtype);
+    XMA_REQUIRE(epilogue >= XMA_ROCM_EPI_STORE && epilogue <= XMA_ROCM_EPI_SWIGLU_BWD, XMA_ROCM_EINVAL,
+                "scatter2scatter_few_rows: epilogue %d", epilogue);
+    XMA_REQUIRE(M >= 0 && M <= 65535 && N >= 8 && K >= 8 && E >= 1 && E <= 65535 && fan_out >= 1, XMA_ROCM_EINVAL,
+                "scatter2scatter_few_rows: M=%lld N=%d K=%d E=%d fan_out=%d (M and E at most 65535)", (long long)M, N, K, E, fan_out);
+    XMA_REQUIRE(N % 8 == 0 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldo % 8 == 0 && w_expert_stride % 8 == 0,
+                XMA_ROCM_EUNSUPPORTED, "scatter2scatter_few_rows: N=%d K=%d and the leading dimensions must be multiples of 8", N, K);
+    XMA_REQUIRE(w_is_kn || K <= FR_NT_KMAX, XMA_ROCM_EUNSUPPORTED, "scatter2scatter_few_rows: K=%d exceeds %d for W as (N, K)", K,
+                FR_NT_KMAX);
+    XMA_REQUIRE(!w_is_kn || fr_nn_range(K) <= FR_NN_KC_MAX, XMA_ROCM_EUNSUPPORTED,
+                "scatter2scatter_few_rows: K=%d exceeds %d for W as (K, N)", K, FR_NN_KC_MAX * FR_NN_SPLITS);
+    if (M == 0) return XMA_ROCM_OK;
+    auto al16 = [](const void *p) { return ((uintptr_t)p & 15) == 0; };
+    XMA_REQUIRE(X && W && expert_offsets && al16(X) && al16(W), XMA_ROCM_EINVAL, "scatter2scatter_few_rows: null or misaligned operand");
+    XMA_REQUIRE(sorted_scattered_idxs || (x_grouped && y_grouped && !row_scale), XMA_ROCM_EINVAL,
+                "scatter2scatter_few_rows: sorted_scattered_idxs is required unless everything is grouped");
+    if (epilogue == XMA_ROCM_EPI_STORE) {
+        XMA_REQUIRE(out && al16(out), XMA_ROCM_EINVAL, "scatter2scatter_few_rows: out is null or misaligned");
+    } else if (epilogue == XMA_ROCM_EPI_SWIGLU) {
+        XMA_REQUIRE(aux && al16(aux) && ldaux % 8 == 0 && N % 16 == 0 && (!out || al16(out)), XMA_ROCM_EINVAL,
+                    "scatter2scatter_few_rows: SWIGLU needs aux (M, N/2), ldaux %% 8 == 0, N %% 16 == 0");
+    } else {
+        XMA_REQUIRE(out && aux && al16(out) && al16(aux) && ldaux % 8 == 0 && y_grouped && !bias, XMA_ROCM_EINVAL,
+                    "scatter2scatter_few_rows: SWIGLU_BWD needs out, aux (z), y_grouped and no bias");
+    }
+    XMA_REQUIRE(!aux2 || (epilogue == XMA_ROCM_EPI_SWIGLU_BWD && al16(aux2) && ldaux2 % 8 == 0 && ldaux2 >= N), XMA_ROCM_EINVAL,
+                "scatter2scatter_few_rows: scaled activations go with SWIGLU_BWD, 16-byte aligned rows");
+    XMA_REQUIRE(!bias || (al16(bias) && bias_expert_stride % 8 == 0 && bias_expert_stride >= 0), XMA_ROCM_EINVAL,
+                "scatter2scatter_few_rows: bias (E, N) must be 16-byte aligned with an expert stride that is a multiple of 8");
+    const size_t need = xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, w_is_kn);
+    XMA_REQUIRE(workspace && workspace_bytes >= need && al16(workspace), XMA_ROCM_EWORKSPACE,
+                "scatter2scatter_few_rows: workspace of %zu bytes, %zu needed (16-byte aligned)", workspace ? workspace_bytes : (size_t)0, need);
+    FwdArgs a;
+    a.X = (const uint16_t *)X;
+    a.ldx = ldx;
+    a.W = (const uint16_t *)W;
+    a.w_es = w_expert_stride;
+    a.ldw = ldw;
+    a.idx = sorted_scattered_idxs;
+    a.offs = expert_offsets;
+    a.out = (uint16_t *)out;
+    a.ldo = ldo;
+    a.aux = (uint16_t *)aux;
+    a.ldaux = ldaux;
+    a.aux2 = (uint16_t *)aux2;
+    a.ldaux2 = ldaux2;
+    a.scale = (const uint16_t *)row_scale;
+    a.bias = (const uint16_t *)bias;
+    a.bias_es = bias_expert_stride;
+    a.M = M;
+    a.N = N;
+    a.K = K;
+    a.E = E;
+    a.fan_out = fan_out;
+    a.fan_div = make_fastdiv((uint32_t)fan_out);
+    a.x_grouped = x_grouped;
+    a.y_grouped = y_grouped;
+    a.partial = nullptr;
+    a.split_cus = 0;
+    a.grid_main = 0;
+    hipStream_t st = (hipStream_t)stream;
+    if (dtype == XMA_ROCM_BF16) return fr_launch<__bf16>(a, w_is_kn ? 1 : 0, epilogue, (float *)workspace, st);
+    return fr_launch<_Float16>(a, w_is_kn ? 1 : 0, epilogue, (float *)workspace, st);
 }

@@ -82,9 +82,12 @@ def continuous_count_rocm(x: torch.Tensor, y: torch.Tensor, workspace: torch.Ten
 
 
 CONTINUOUS_COUNT_SET_MAX_BINS = 8192
-# Up to this many rows in total (tokens x experts per token) the grouped GEMMs take the entry points written for the
-# few-token regime, which stream the weights instead of tiling them for the matrix pipes.
-FEW_ROWS_MAX = 64
+# The grouped GEMMs take the entry points written for the few-token regime, which stream the weights instead of tiling
+# them for the matrix pipes, up to FEW_ROWS_PER_EXPERT rows per expert on average (the expert's rows are walked 4 or 8 at a
+# time, each pass streaming its weights again: measured cross-over at 6 - 7 rows per expert) and FEW_ROWS_MAX rows in all.
+FEW_ROWS_MAX = 256
+FEW_ROWS_PER_EXPERT = 6
+FEW_ROWS_MAX_WORKSPACE = 256 << 20  # bytes of fp32 partial sums a forward-type launch may ask for
 
 
 @torch.library.custom_op("xma_rocm::continuous_count_set", mutates_args={"y"})
@@ -158,6 +161,38 @@ def scatter2scatter_workspace_bytes(M: int, N: int, K: int, E: int, device_index
     return _S2S_WORKSPACE_BYTES[key]
 
 
+FEW_ROWS_NT_MAX_K = 8192  # limits of the few-token entry point for the two weight layouts
+FEW_ROWS_NN_MAX_K = 65536
+
+
+def _few_rows(M: int, E: int, dtype: torch.dtype) -> bool:
+    """whether a grouped GEMM of M rows over E experts takes an entry point written for the few-token regime"""
+    return 0 < M <= min(FEW_ROWS_MAX, FEW_ROWS_PER_EXPERT * E) and dtype in (torch.bfloat16, torch.float16)
+
+
+def _few_rows_fwd(lib, M: int, N: int, K: int, E: int, w_is_kn: int, dtype: torch.dtype) -> bool:
+    """the same for a forward-type GEMM, whose few-token entry point has limits of its own"""
+    if not _few_rows(M, E, dtype) or K > (FEW_ROWS_NN_MAX_K if w_is_kn else FEW_ROWS_NT_MAX_K):
+        return False
+    return lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, w_is_kn) <= FEW_ROWS_MAX_WORKSPACE
+
+
+def _scatter2scatter_few_rows(lib, X, W, w_is_kn, w_es, ldw, idx, offs, out, aux, aux2, scale, bias, fan_out, x_grouped,
+                              y_grouped, epilogue, M, N, K):
+    ws_bytes = lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, w_is_kn)
+    workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=X.device)
+    check(
+        lib.xma_rocm_scatter2scatter_few_rows(
+            _ptr(X), _rows(X, "X"), _ptr(W), w_es, ldw, w_is_kn, _ptr(idx), _ptr(offs),
+            _ptr(out), 0 if out is None else _rows(out, "out"), _ptr(aux), 0 if aux is None else _rows(aux, "aux"),
+            _ptr(aux2), 0 if aux2 is None else _rows(aux2, "aux2"), _ptr(scale), _ptr(bias),
+            0 if bias is None else bias.stride(0), M, N, K, W.size(0), fan_out, int(x_grouped), int(y_grouped), epilogue,
+            _code(X), _ptr(workspace), ws_bytes, _stream(X),
+        ),
+        "xma_rocm_scatter2scatter_few_rows",
+    )
+
+
 def _scatter2scatter(X, W, idx, offs, out, aux, scale, fan_out, x_grouped, y_grouped, epilogue, M, N, K, bias=None):
     w_is_kn, w_es, ldw = _weight_layout(W)
     if bias is not None:  # (E, N): the experts' bias, the first term of every fp32 sum
@@ -170,6 +205,10 @@ def _scatter2scatter(X, W, idx, offs, out, aux, scale, fan_out, x_grouped, y_gro
     if scale is not None:
         assert scale.dtype == X.dtype and scale.is_contiguous()
     lib = get_library()
+    if _few_rows_fwd(lib, M, N, K, W.size(0), w_is_kn, X.dtype):
+        _scatter2scatter_few_rows(lib, X, W, w_is_kn, w_es, ldw, idx, offs, out, aux, None, scale, bias, fan_out, x_grouped,
+                                  y_grouped, epilogue, M, N, K)
+        return
     # scratch for the K slices of the tiles of a last, partial round (0 bytes for launches of many rounds); it comes from
     # torch's caching allocator like every other buffer of the op
     ws_bytes = scatter2scatter_workspace_bytes(M, N, K, W.size(0), X.device.index or 0)
@@ -271,6 +310,10 @@ def down_projection_dx_swiglu_scaled_act_rocm(
     w_is_kn, w_es, ldw = _weight_layout(W)
     assert w_is_kn == 1, "W should be the down-projection parameter as stored, (E, H, I) with I contiguous"
     lib = get_library()
+    if _few_rows_fwd(lib, M, N, K, E, 1, dY.dtype):
+        _scatter2scatter_few_rows(lib, dY, W, 1, w_es, ldw, sorted_scattered_idxs, expert_offsets, dz, z, scaled_act,
+                                  row_scale, None, FAN_OUT, False, True, EPI_SWIGLU_BWD, M, N, K)
+        return
     ws_bytes = scatter2scatter_workspace_bytes(M, N, K, E, dY.device.index or 0)
     workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=dY.device) if ws_bytes else None
     check(
@@ -305,8 +348,8 @@ def group_bwd_W_rocm(
     if dy_scale is not None:
         assert dy_scale.dtype == DY.dtype and dy_scale.is_contiguous()
     lib = get_library()
-    # a handful of rows in total (the index has one entry per row): the launch is a stream of stores, not arithmetic
-    few = sorted_scattered_idxs.numel() <= FEW_ROWS_MAX and DW.dtype in (torch.bfloat16, torch.float16)
+    # a handful of rows per expert (the index has one entry per row): the launch is a stream of stores, not arithmetic
+    few = _few_rows(sorted_scattered_idxs.numel(), E, DW.dtype)
     name = "xma_rocm_group_bwd_W_few_rows" if few else "xma_rocm_group_bwd_W"
     check(
         getattr(lib, name)(

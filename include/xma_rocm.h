@@ -196,6 +196,27 @@ XMA_API int xma_rocm_down_projection_dx_swiglu(const void *dY, int64_t lddy, con
                                                void *stream);
 
 /*
+ * xma_rocm_scatter2scatter_bias / xma_rocm_down_projection_dx_swiglu for the few-token regime: the same arguments
+ * (aux2 = the scaled activations of the latter, or NULL), the same results up to the order of the fp32 sums, bf16 / fp16
+ * only.  With a handful of rows per expert the product is a stream over the weights: rows of W[e] as (N, K) are read by a
+ * wave with its lanes along K, rows of W[e] as (K, N) by threads that own 8 columns each, with vector FMAs on fp32
+ * sums; the sums go through the workspace (required: xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K,
+ * w_is_kn) bytes) to a small kernel that applies the bias and the epilogue with the arithmetic of the MFMA kernels.
+ * Limits: M and E at most 65535, K at most 8192 for W as (N, K) and 65536 for W as (K, N).  Correct for any M, but the
+ * time grows with (rows per expert) x |W|: meant for launches of a few rows per expert (the torch ops of this package
+ * take it up to six on average).  No counterpart in the reference
+ * (its kernel is the same for every size).
+ */
+XMA_API size_t xma_rocm_scatter2scatter_few_rows_workspace_bytes(int64_t M, int32_t N, int32_t K, int w_is_kn);
+XMA_API int xma_rocm_scatter2scatter_few_rows(const void *X, int64_t ldx, const void *W, int64_t w_expert_stride, int64_t ldw,
+                                      int w_is_kn, const int64_t *sorted_scattered_idxs,
+                                      const int64_t *expert_offsets, void *out, int64_t ldo, void *aux, int64_t ldaux,
+                                      void *aux2, int64_t ldaux2, const void *row_scale, const void *bias,
+                                      int64_t bias_expert_stride, int64_t M, int32_t N, int32_t K, int32_t num_experts,
+                                      int32_t fan_out, int x_grouped, int y_grouped, int epilogue, int dtype,
+                                      void *workspace, size_t workspace_bytes, void *stream);
+
+/*
  * Weight gradient of a grouped linear: for every expert e
  *     DW[e] (N_out, K_in) = sum_{n in expert e} DY[dsrc(n), :N_out]^T  X[xsrc(n), :K_in]
  *     dsrc(n) = n if dy_grouped else sorted_scattered_idxs[n] / dy_fan_out   (then scaled by dy_scale[idx[n]] if given)
@@ -218,8 +239,8 @@ XMA_API int xma_rocm_group_bwd_W(const void *DY, int64_t lddy, int dy_grouped, i
  * fp16 only; DY needs no 16-byte alignment and N_out no multiple of 8).  One workgroup per 8 rows of DW[e] streams its
  * stores and adds one outer product per row of the expert with vector FMAs: with a handful of rows per expert the launch
  * runs at the rate of a fill of DW, where the MFMA tiles of xma_rocm_group_bwd_W spend a prologue, one K step and an
- * epilogue per 256 x 256 tile.  Correct for any number of rows, but its time grows with rows x |DW|: meant for launches
- * of at most a few dozen rows in total.  No counterpart in the reference (its kernel is the same for every size).
+ * epilogue per 256 x 256 tile.  Correct for any number of rows, but its time grows with (rows per expert) x |DW|: meant
+ * for launches of a few rows per expert.  No counterpart in the reference (its kernel is the same for every size).
  */
 XMA_API int xma_rocm_group_bwd_W_few_rows(const void *DY, int64_t lddy, int dy_grouped, int32_t dy_fan_out,
                                   const void *dy_scale, const void *X, int64_t ldx, int x_grouped, int32_t x_fan_out,

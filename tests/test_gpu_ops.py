@@ -30,7 +30,8 @@ def _routing(T, E, k, seed, skew=0.0, empty=()):
 
 
 class _few_rows_limit:
-    """the limit below which the ops take the few-token entry points, set for the length of a with block (0: never)"""
+    """the number of rows up to which the ops take the few-token entry points, whatever the number of experts, set for the
+    length of a with block (0: never)"""
 
     def __init__(self, limit):
         self.limit = limit
@@ -38,12 +39,13 @@ class _few_rows_limit:
     def __enter__(self):
         from xma.rocm import ops
 
-        self.saved, ops.FEW_ROWS_MAX = ops.FEW_ROWS_MAX, self.limit
+        self.saved = (ops.FEW_ROWS_MAX, ops.FEW_ROWS_PER_EXPERT)
+        ops.FEW_ROWS_MAX, ops.FEW_ROWS_PER_EXPERT = self.limit, 1 << 30
 
     def __exit__(self, *exc):
         from xma.rocm import ops
 
-        ops.FEW_ROWS_MAX = self.saved
+        ops.FEW_ROWS_MAX, ops.FEW_ROWS_PER_EXPERT = self.saved
 
 
 def _limits(rows):
@@ -88,12 +90,14 @@ def test_scatter2scatter(dtype, case, w_kn, x_grouped, y_grouped):
     for rs in (None, scale):
         want = oracle.scatter2scatter(X, W, se, ss, k, x_grouped, y_grouped, rs)
         Wd = W.cuda() if w_kn else W.permute(0, 2, 1).contiguous().cuda().permute(0, 2, 1)
-        out = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
-        R.scatter2scatter(X.cuda(), Wd, se.cuda(), ss.cuda(), out, k, x_grouped, y_grouped, offs.cuda(),
-                          None if rs is None else rs.cuda())
-        torch.cuda.synchronize()
-        assert torch.isfinite(out).all()
-        assert nerr(out, want) <= _tol(dtype)
+        for limit in _limits(M):
+            out = torch.full((M, N), float("nan"), dtype=dtype, device="cuda")
+            with _few_rows_limit(limit):
+                R.scatter2scatter(X.cuda(), Wd, se.cuda(), ss.cuda(), out, k, x_grouped, y_grouped, offs.cuda(),
+                                  None if rs is None else rs.cuda())
+            torch.cuda.synchronize()
+            assert torch.isfinite(out).all()
+            assert nerr(out, want) <= _tol(dtype), limit
 
 
 def test_scatter2scatter_launches_outside_the_persistent_kernel():
@@ -327,6 +331,125 @@ def test_group_bwd_W(dtype, case):
             got = run(dy_grp, x_grp, None, 0, 0)
             for e in empty:
                 assert (got[e] == 0).all()
+
+
+FEW_ROWS_CASES = [
+    # T, E, k, H, I, empty experts
+    (7, 8, 2, 264, 136, ()),
+    (3, 128, 8, 576, 256, ()),  # more experts than rows
+    (16, 4, 4, 2048, 72, (2,)),  # about twenty rows per expert: several passes of 4 or 8 rows over the weights
+    (1, 8, 1, 64, 8, ()),
+    (9, 5, 3, 4104, 24, (0, 4)),  # a row of W as (N, K) is 513 pieces of 16 bytes: two passes of a wave and one lane more
+    (7, 8, 2, 512, 8192, ()),  # K = 8192 for the down-projection (64 KB of LDS), 128 K ranges of 128 for dX1
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", FEW_ROWS_CASES)
+def test_forward_type_gemms_few_rows(dtype, case):
+    """The six operand forms of the layer's forward-type GEMMs through the kernels written for a handful of rows (weights
+    streamed once, vector FMAs, sums through a workspace, one small epilogue kernel), each against the oracle and against
+    the MFMA kernels on the same operands: up-projection + SwiGLU with a bias (z and h), up-projection with a plain store,
+    down-projection with a bias, a row scale and scattered rows, dX1 (dz @ W1, scattered), dX2 + SwiGLU backward with and
+    without the scaled activations."""
+    from xma.rocm import ops
+
+    T, E, k, H, I, empty = case
+    print(f"case T={T} E={E} k={k} H={H} I={I} {dtype}", flush=True)
+    sel, se, ss, offs = _routing(T, E, k, 41, 0.0, empty)
+    M = T * k
+    assert M <= ops.FEW_ROWS_MAX
+    g = torch.Generator().manual_seed(42)
+    x = torch.randn(T, H, generator=g).to(dtype)
+    W1 = (torch.randn(E, 2 * I, H, generator=g) * 0.05).to(dtype)  # c_fc.weight (E, out, in)
+    W2 = (torch.randn(E, H, I, generator=g) * 0.05).to(dtype)  # c_proj.weight
+    b1 = torch.randn(E, 2 * I, generator=g).to(dtype)
+    b2 = torch.randn(E, H, generator=g).to(dtype)
+    w = torch.rand(M, generator=g).to(dtype)
+    dy = torch.randn(T, H, generator=g).to(dtype)
+    dzg = torch.randn(M, 2 * I, generator=g).to(dtype)
+    xd, W1d, W2d, b1d, b2d, wd, dyd, dzd, ssd, offsd = (t.cuda() for t in (x, W1, W2, b1, b2, w, dy, dzg, ss, offs))
+    tol = _tol(dtype)
+
+    def both(fn):
+        """fn() -> tuple of device outputs; run with the MFMA kernels and with the few-row kernels"""
+        res = {}
+        for limit in (0, ops.FEW_ROWS_MAX):
+            with _few_rows_limit(limit):
+                res[limit] = fn()
+            torch.cuda.synchronize()
+        return res[ops.FEW_ROWS_MAX], res[0]
+
+    def new(*shape):
+        return torch.full(shape, float("nan"), dtype=dtype, device="cuda")
+
+    # up-projection + SwiGLU, bias
+    def up():
+        z, h = new(M, 2 * I), new(M, I)
+        ops.up_projection_swiglu_rocm(xd, W1d.permute(0, 2, 1), ssd, offsd, z, h, k, b1d)
+        return z, h
+
+    want_z = oracle.scatter2scatter(x, W1.permute(0, 2, 1), se, ss, k, False, True, None, bias=b1)
+    (z_f, h_f), (z_m, h_m) = both(up)
+    assert torch.isfinite(z_f).all() and torch.isfinite(h_f).all()
+    assert nerr(z_f, want_z) <= tol and nerr(z_f, z_m) <= tol
+    assert nerr(h_f, oracle.swiglu_packed(want_z)) <= tol and nerr(h_f, h_m) <= tol
+
+    # up-projection, plain store, no bias
+    def up_store():
+        z = new(M, 2 * I)
+        ops.scatter2scatter_rocm(xd, W1d.permute(0, 2, 1), ssd, offsd, z, None, k, False, True)
+        return (z,)
+
+    (z_f,), (z_m,) = both(up_store)
+    assert nerr(z_f, oracle.scatter2scatter(x, W1.permute(0, 2, 1), se, ss, k, False, True, None)) <= tol and nerr(z_f, z_m) <= tol
+
+    # down-projection: grouped rows in, scattered rows out, bias and row scale
+    hg = torch.randn(M, I, generator=g).to(dtype)
+    hgd = hg.cuda()
+
+    def down():
+        out = new(M, H)
+        ops.scatter2scatter_rocm(hgd, W2d.permute(0, 2, 1), ssd, offsd, out, wd, 1, True, False, b2d)
+        return (out,)
+
+    (o_f,), (o_m,) = both(down)
+    want = oracle.scatter2scatter(hg, W2.permute(0, 2, 1), se, ss, 1, True, False, w, bias=b2)
+    assert torch.isfinite(o_f).all() and nerr(o_f, want) <= tol and nerr(o_f, o_m) <= tol
+
+    # dX1: dz @ W1 (W as (K, N) = the parameter as stored), scattered rows out
+    def dx1():
+        out = new(M, H)
+        ops.scatter2scatter_rocm(dzd, W1d, ssd, offsd, out, None, 1, True, False)
+        return (out,)
+
+    (o_f,), (o_m,) = both(dx1)
+    want = oracle.scatter2scatter(dzg, W1, se, ss, 1, True, False, None)
+    assert torch.isfinite(o_f).all() and nerr(o_f, want) <= tol and nerr(o_f, o_m) <= tol
+
+    # dX2 + SwiGLU backward, without and with the scaled activations
+    zg = torch.randn(M, 2 * I, generator=g).to(dtype)
+    zgd = zg.cuda()
+
+    def dx2():
+        dz = new(M, 2 * I)
+        ops.down_projection_dx_swiglu_rocm(dyd, W2d, ssd, offsd, zgd, dz, wd, k)
+        return (dz,)
+
+    def dx2_act():
+        dz, act = new(M, 2 * I), new(M, I)
+        ops.down_projection_dx_swiglu_scaled_act_rocm(dyd, W2d, ssd, offsd, zgd, dz, act, wd, k)
+        return dz, act
+
+    z32 = zg.float().requires_grad_()
+    h32 = oracle.swiglu_packed(z32)
+    dh = torch.stack([(dy.float()[ss[n] // k] * w.float()[ss[n]]) @ W2.float()[se[n]] for n in range(M)])
+    h32.backward(dh)
+    (dz_f,), (dz_m,) = both(dx2)
+    assert torch.isfinite(dz_f).all() and nerr(dz_f, z32.grad) <= tol and nerr(dz_f, dz_m) <= tol
+    (dz_a, act_f), (_, act_m) = both(dx2_act)
+    assert torch.equal(dz_a, dz_f)
+    assert nerr(act_f, h32.detach() * w.float()[ss][:, None]) <= tol and nerr(act_f, act_m) <= tol
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
