@@ -149,7 +149,8 @@ namespace {
 // Forward-type product for a handful of rows: acc[r][n] = sum_k X[src(r)][k] * B_e[k][n] in fp32, written to a workspace
 // part[S][M][N] as S partial sums over K ranges, then one small kernel that adds the parts in order and runs the epilogue.
 //   W[e] as (N, K), K contiguous (x @ W^T): a wave takes two rows of W at a time, its lanes split K in 16-byte pieces,
-//       the expert's rows of X wait in LDS, and the lanes' partial dot products meet in a butterfly.  S = 1.
+//       the expert's rows of X wait in LDS, and the lanes' partial dot products meet in a butterfly.  S = 1, and for the
+//       STORE and SWIGLU epilogues the wave finishes the job itself: no workspace, no second kernel.
 //   W[e] as (K, N), N contiguous (dy @ W): a thread owns 8 columns n and walks the rows k of its workgroup's K range;
 //       the X values of the range sit in LDS as floats.  S = K / range.
 // ------------------------------------------------------------------------------------------------
@@ -160,7 +161,7 @@ __device__ __forceinline__ int64_t fr_src_row(const FwdArgs &a, int64_t r) {
     return a.x_grouped ? r : (int64_t)fastdiv((uint32_t)a.idx[r], a.fan_div);
 }
 
-template <typename T, int RC>
+template <typename T, int RC, int EPI>
 __device__ __forceinline__ void fr_nt_rows(const FwdArgs &a, float *__restrict__ part, uint16_t *s_x, int e, int64_t lo,
                                            int64_t hi, int n_first, int n_count) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -221,9 +222,23 @@ __device__ __forceinline__ void fr_nt_rows(const FwdArgs &a, float *__restrict__
             if (lane == 0) {
 #pragma unroll
                 for (int u = 0; u < RC; ++u) {
-                    if (r0 + u < hi) {
-                        part[(r0 + u) * a.N + n_a] = s[u][0];
-                        if (p + 1 < n_count) part[(r0 + u) * a.N + n_b] = s[u][1];
+                    const int64_t r = r0 + u;
+                    if (r >= hi) continue;
+                    if constexpr (EPI < 0) { // the sums go to the workspace, the epilogue kernel follows
+                        part[r * a.N + n_a] = s[u][0];
+                        if (p + 1 < n_count) part[r * a.N + n_b] = s[u][1];
+                    } else { // the only part there is: bias, scale and the epilogue right here (n_a is even, n_b = n_a + 1)
+                        const int64_t s_idx = a.idx ? a.idx[r] : r;
+                        const float sc = a.scale ? fr_scalar<T>(a.scale, s_idx) : 1.f;
+                        const int64_t dst = a.y_grouped ? r : s_idx;
+                        float v0 = s[u][0], v1 = s[u][1];
+                        if (a.bias) v0 += fr_scalar<T>(a.bias, (int64_t)e * a.bias_es + n_a), v1 += fr_scalar<T>(a.bias, (int64_t)e * a.bias_es + n_b);
+                        const uint32_t z = Elem<T>::pack(v0 * sc, v1 * sc);
+                        if (a.out) *(uint32_t *)(a.out + dst * a.ldo + n_a) = z;
+                        if constexpr (EPI == XMA_ROCM_EPI_SWIGLU) {
+                            const float g = Elem<T>::lo(z), up = Elem<T>::hi(z);
+                            a.aux[dst * a.ldaux + (n_a >> 1)] = (uint16_t)(Elem<T>::pack(up * g * sigmoidf_fast(g), 0.f) & 0xffffu);
+                        }
                     }
                 }
             }
@@ -231,7 +246,9 @@ __device__ __forceinline__ void fr_nt_rows(const FwdArgs &a, float *__restrict__
     }
 }
 
-template <typename T>
+// EPI = XMA_ROCM_EPI_STORE or _SWIGLU: the wave that holds a pair of sums applies bias, scale and epilogue itself (the
+// columns of a pair are (gate, up)); EPI = -1: the sums go to the workspace for fr_epilogue_kernel.
+template <typename T, int EPI>
 __global__ __launch_bounds__(FR_THREADS) void fr_nt_kernel(const FwdArgs a, float *__restrict__ part, int rows_per_wg) {
     extern __shared__ __attribute__((aligned(16))) uint16_t s_x_nt[];
     const int e = blockIdx.y;
@@ -240,9 +257,9 @@ __global__ __launch_bounds__(FR_THREADS) void fr_nt_kernel(const FwdArgs a, floa
     const int n_first = blockIdx.x * rows_per_wg;
     const int n_count = (a.N - n_first < rows_per_wg) ? a.N - n_first : rows_per_wg;
     if (hi - lo <= 2)
-        fr_nt_rows<T, 2>(a, part, s_x_nt, e, lo, hi, n_first, n_count);
+        fr_nt_rows<T, 2, EPI>(a, part, s_x_nt, e, lo, hi, n_first, n_count);
     else
-        fr_nt_rows<T, 4>(a, part, s_x_nt, e, lo, hi, n_first, n_count);
+        fr_nt_rows<T, 4, EPI>(a, part, s_x_nt, e, lo, hi, n_first, n_count);
 }
 
 constexpr int FR_NN_KC_MIN = 32;  // rows k of W per workgroup, at least (four rounds of eight loads per thread)
@@ -397,8 +414,19 @@ template <typename T> int fr_launch(const FwdArgs &a, int w_is_kn, int epilogue,
         const int rows_per_wg = (a.K >= 2048) ? FR_NT_ROWS : 8; // short rows: one pair of rows per wave, more workgroups
         const dim3 grid((a.N + rows_per_wg - 1) / rows_per_wg, a.E);
         const size_t lds = (size_t)4 * a.K * sizeof(uint16_t);
-        if (lds > 48 * 1024 && (rc = xma_set_max_lds_once((const void *)fr_nt_kernel<T>, 4 * FR_NT_KMAX * (int)sizeof(uint16_t)))) return rc;
-        fr_nt_kernel<T><<<grid, FR_THREADS, lds, st>>>(a, part, rows_per_wg);
+        const int max_lds = 4 * FR_NT_KMAX * (int)sizeof(uint16_t);
+        if (epilogue == XMA_ROCM_EPI_STORE) {
+            if (lds > 48 * 1024 && (rc = xma_set_max_lds_once((const void *)fr_nt_kernel<T, XMA_ROCM_EPI_STORE>, max_lds))) return rc;
+            fr_nt_kernel<T, XMA_ROCM_EPI_STORE><<<grid, FR_THREADS, lds, st>>>(a, part, rows_per_wg);
+            return xma_check_launch("fr_nt_kernel");
+        }
+        if (epilogue == XMA_ROCM_EPI_SWIGLU) {
+            if (lds > 48 * 1024 && (rc = xma_set_max_lds_once((const void *)fr_nt_kernel<T, XMA_ROCM_EPI_SWIGLU>, max_lds))) return rc;
+            fr_nt_kernel<T, XMA_ROCM_EPI_SWIGLU><<<grid, FR_THREADS, lds, st>>>(a, part, rows_per_wg);
+            return xma_check_launch("fr_nt_kernel");
+        }
+        if (lds > 48 * 1024 && (rc = xma_set_max_lds_once((const void *)fr_nt_kernel<T, -1>, max_lds))) return rc;
+        fr_nt_kernel<T, -1><<<grid, FR_THREADS, lds, st>>>(a, part, rows_per_wg);
         if ((rc = xma_check_launch("fr_nt_kernel"))) return rc;
     }
     const dim3 egrid((a.N / 2 + FR_THREADS - 1) / FR_THREADS, (unsigned)a.M);
@@ -460,8 +488,9 @@ extern "C" int xma_rocm_scatter2scatter_few_rows(const void *X, int64_t ldx, con
                 "scatter2scatter_few_rows: scaled activations go with SWIGLU_BWD, 16-byte aligned rows");
     XMA_REQUIRE(!bias || (al16(bias) && bias_expert_stride % 8 == 0 && bias_expert_stride >= 0), XMA_ROCM_EINVAL,
                 "scatter2scatter_few_rows: bias (E, N) must be 16-byte aligned with an expert stride that is a multiple of 8");
-    const size_t need = xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, w_is_kn);
-    XMA_REQUIRE(workspace && workspace_bytes >= need && al16(workspace), XMA_ROCM_EWORKSPACE,
+    // W as (N, K) with the STORE or SWIGLU epilogue finishes in one kernel and needs no workspace
+    const size_t need = (w_is_kn || epilogue == XMA_ROCM_EPI_SWIGLU_BWD) ? xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, w_is_kn) : 0;
+    XMA_REQUIRE(need == 0 || (workspace && workspace_bytes >= need && al16(workspace)), XMA_ROCM_EWORKSPACE,
                 "scatter2scatter_few_rows: workspace of %zu bytes, %zu needed (16-byte aligned)", workspace ? workspace_bytes : (size_t)0, need);
     FwdArgs a;
     a.X = (const uint16_t *)X;

@@ -179,8 +179,10 @@ def _few_rows_fwd(lib, M: int, N: int, K: int, E: int, w_is_kn: int, dtype: torc
 
 def _scatter2scatter_few_rows(lib, X, W, w_is_kn, w_es, ldw, idx, offs, out, aux, aux2, scale, bias, fan_out, x_grouped,
                               y_grouped, epilogue, M, N, K):
-    ws_bytes = lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, w_is_kn)
-    workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=X.device)
+    # W as (N, K) with the STORE or SWIGLU epilogue finishes in one kernel; everything else sums through a workspace
+    needs_ws = bool(w_is_kn) or epilogue == EPI_SWIGLU_BWD
+    ws_bytes = lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, w_is_kn) if needs_ws else 0
+    workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=X.device) if ws_bytes else None
     check(
         lib.xma_rocm_scatter2scatter_few_rows(
             _ptr(X), _rows(X, "X"), _ptr(W), w_es, ldw, w_is_kn, _ptr(idx), _ptr(offs),

@@ -548,6 +548,7 @@ def run_small_t(args):
     from xma.functional import swiglu_packed
     from xma.layers import MoE
     from xma.layers.moe import rocm_implementation as R
+    from xma.rocm import ops as _ops
 
     res = {}
     for E, k, H, I in ((8, 2, 2048, 8192), (128, 8, 576, 256)):
@@ -586,6 +587,7 @@ def run_small_t(args):
             stream_bytes = 2 * touched * wbytes + E * wbytes  # forward and dX read the touched experts, dW writes all
             res[f"E{E}_k{k}_H{H}_I{I}_T{T}"] = {
                 "eager_ms": round(eager_ms, 4), "graph_ms": round(graph_ms, 4), "experts_touched": touched,
+                "gemm_kernels": "few_rows (weights streamed, vector FMAs)" if _ops._few_rows(T * k, E, torch.bfloat16) else "mfma tiles",
                 "weight_stream_ms_at_8TBs": round(stream_bytes / PEAK_HBM_GBS / 1e6, 4),
                 "graph_over_stream": round(graph_ms / (stream_bytes / PEAK_HBM_GBS / 1e6), 2),
             }

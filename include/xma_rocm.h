@@ -200,8 +200,10 @@ XMA_API int xma_rocm_down_projection_dx_swiglu(const void *dY, int64_t lddy, con
  * (aux2 = the scaled activations of the latter, or NULL), the same results up to the order of the fp32 sums, bf16 / fp16
  * only.  With a handful of rows per expert the product is a stream over the weights: rows of W[e] as (N, K) are read by a
  * wave with its lanes along K, rows of W[e] as (K, N) by threads that own 8 columns each, with vector FMAs on fp32
- * sums; the sums go through the workspace (required: xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K,
- * w_is_kn) bytes) to a small kernel that applies the bias and the epilogue with the arithmetic of the MFMA kernels.
+ * sums.  For W as (K, N), and for SWIGLU_BWD, the sums go through the workspace (required then:
+ * xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, w_is_kn) bytes) to a small kernel that applies the bias and
+ * the epilogue with the arithmetic of the MFMA kernels; W as (N, K) with STORE or SWIGLU finishes in one kernel and takes
+ * no workspace (NULL, 0).
  * Limits: M and E at most 65535, K at most 8192 for W as (N, K) and 65536 for W as (K, N).  Correct for any M, but the
  * time grows with (rows per expert) x |W|: meant for launches of a few rows per expert (the torch ops of this package
  * take it up to six on average).  No counterpart in the reference
