@@ -54,10 +54,13 @@ class _RouterTopK(torch.autograd.Function):
         ops.router_topk_rocm(router_logits, weights, ids)
         ctx.save_for_backward(router_logits, ids)
         ctx.mark_non_differentiable(ids)
+        ctx.set_materialize_grads(False)  # no zero fill for the gradient of the ids, which nothing reads
         return weights, ids
 
     @staticmethod
-    def backward(ctx, d_weights: torch.Tensor, _d_ids):
+    def backward(ctx, d_weights: torch.Tensor | None, _d_ids):
+        if d_weights is None:  # nothing downstream depends on the router weights
+            return None, None, None
         router_logits, ids = ctx.saved_tensors
         d_logits = torch.empty_like(router_logits, memory_format=torch.contiguous_format)
         ops.router_topk_bwd_rocm(router_logits, ids, d_weights.contiguous(), d_logits)
