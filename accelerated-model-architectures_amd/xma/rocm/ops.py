@@ -557,3 +557,26 @@ def router_topk_bwd_rocm(logits: torch.Tensor, ids: torch.Tensor, d_weights: tor
                                      _rows(d_logits, "d_logits"), _stream(logits)),
         "xma_rocm_router_topk_bwd",
     )
+
+
+# ------------------------------------------------------------------------------------------------ eager fast path
+def _eager_fast_path(op):
+    """The registered op when a compiler is tracing (the graph gets its node), its Python body directly otherwise: the
+    dispatcher's way to the same body costs 7 us per call on the host (measured: 14.5 against 7.2 us for `combine`), which
+    is most of an eager step of a handful of tokens.  The ops return nothing and write tensors that their callers have
+    just allocated, so nothing that autograd does for a registered op (version counters of mutated arguments) is missed."""
+    body = op._init_fn
+
+    def call(*args, **kwargs):
+        if torch.compiler.is_compiling():
+            return op(*args, **kwargs)
+        return body(*args, **kwargs)
+
+    call.__name__, call.__doc__, call.registered_op = body.__name__, body.__doc__, op
+    return call
+
+
+for _name, _obj in list(globals().items()):
+    if isinstance(_obj, torch._library.custom_ops.CustomOpDef):
+        globals()[_name] = _eager_fast_path(_obj)
+del _name, _obj
