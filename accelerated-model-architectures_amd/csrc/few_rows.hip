@@ -149,13 +149,14 @@ namespace {
 // Forward-type product for a handful of rows: acc[r][n] = sum_k X[src(r)][k] * B_e[k][n] in fp32, written to a workspace
 // part[S][M][N] as S partial sums over K ranges, then one small kernel that adds the parts in order and runs the epilogue.
 //   W[e] as (N, K), K contiguous (x @ W^T): a wave takes two rows of W at a time, its lanes split K in 16-byte pieces,
-//       the expert's rows of X wait in LDS, and the lanes' partial dot products meet in a butterfly.  S = 1, and for the
+//       the expert's rows of X wait in LDS (2048 columns at a time), and the lanes' partial dot products meet in a butterfly.  S = 1, and for the
 //       STORE and SWIGLU epilogues the wave finishes the job itself: no workspace, no second kernel.
 //   W[e] as (K, N), N contiguous (dy @ W): a thread owns 8 columns n and walks the rows k of its workgroup's K range;
 //       the X values of the range sit in LDS as floats.  S = K / range.
 // ------------------------------------------------------------------------------------------------
 constexpr int FR_NT_ROWS = 32;  // rows of W per workgroup (8 per wave, two at a time); 8 when the rows are short
-constexpr int FR_NT_KMAX = 8192; // the X rows of a step are staged whole: RC x K 16-bit values in LDS
+constexpr int FR_NT_PIECE = 2048; // elements of K whose X values are staged in LDS at a time (4 rows: 16 KB)
+constexpr int FR_NT_PAIRS = FR_NT_ROWS / 8; // pairs of rows of W per wave
 
 __device__ __forceinline__ int64_t fr_src_row(const FwdArgs &a, int64_t r) {
     return a.x_grouped ? r : (int64_t)fastdiv((uint32_t)a.idx[r], a.fan_div);
@@ -165,73 +166,85 @@ template <typename T, int RC, int EPI>
 __device__ __forceinline__ void fr_nt_rows(const FwdArgs &a, float *__restrict__ part, uint16_t *s_x, int e, int64_t lo,
                                            int64_t hi, int n_first, int n_count) {
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    const int chunks = a.K >> 3; // 16-byte pieces of a row
     for (int64_t r0 = lo; r0 < hi; r0 += RC) {
-        __syncthreads(); // the rows of the step before are no longer read
-        for (int i = tid; i < RC * chunks; i += FR_THREADS) {
-            const int u = i / chunks, c = i - u * chunks;
-            u32x4 v = {0u, 0u, 0u, 0u};
-            if (r0 + u < hi) v = *(const u32x4 *)(a.X + fr_src_row(a, r0 + u) * a.ldx + 8 * c);
-            *(u32x4 *)(s_x + ((int64_t)u * chunks + c) * 8) = v;
-        }
-        __syncthreads();
-        for (int p = wave * 2; p < n_count; p += 2 * (FR_THREADS / 64)) { // rows p, p + 1 of the workgroup's block
-            const int n_a = n_first + p, n_b = (p + 1 < n_count) ? n_a + 1 : n_a;
-            const uint16_t *w_a = a.W + (int64_t)e * a.w_es + (int64_t)n_a * a.ldw;
-            const uint16_t *w_b = a.W + (int64_t)e * a.w_es + (int64_t)n_b * a.ldw;
-            float s[RC][2];
+        // pair j of this wave = rows wave * 2 + 8 j (+ 1) of the workgroup's block; n_count is even
+        float s[FR_NT_PAIRS][RC][2];
 #pragma unroll
-            for (int u = 0; u < RC; ++u) s[u][0] = s[u][1] = 0.f;
-            for (int c0 = lane; c0 < chunks; c0 += 4 * 64) { // up to four pieces of either row in flight per lane
-                u32x4 wa[4], wb[4];
+        for (int j = 0; j < FR_NT_PAIRS; ++j)
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int c = c0 + 64 * q;
-                    wa[q] = wb[q] = u32x4{0u, 0u, 0u, 0u};
-                    if (c < chunks) {
-                        wa[q] = __builtin_nontemporal_load((const u32x4 *)(w_a + 8 * c));
-                        wb[q] = __builtin_nontemporal_load((const u32x4 *)(w_b + 8 * c));
+            for (int u = 0; u < RC; ++u) s[j][u][0] = s[j][u][1] = 0.f;
+        for (int kp = 0; kp < a.K; kp += FR_NT_PIECE) { // K in pieces of 2048: RC x 4 KB of X in LDS at a time
+            const int pc = ((a.K - kp < FR_NT_PIECE) ? a.K - kp : FR_NT_PIECE) >> 3; // 16-byte pieces of this step, <= 256
+            __syncthreads(); // the piece before is no longer read
+            for (int i = tid; i < RC * pc; i += FR_THREADS) {
+                const int u = i / pc, c = i - u * pc;
+                u32x4 v = {0u, 0u, 0u, 0u};
+                if (r0 + u < hi) v = *(const u32x4 *)(a.X + fr_src_row(a, r0 + u) * a.ldx + kp + 8 * c);
+                *(u32x4 *)(s_x + (u * (FR_NT_PIECE / 8) + c) * 8) = v;
+            }
+            __syncthreads();
+#pragma unroll
+            for (int j = 0; j < FR_NT_PAIRS; ++j) {
+                const int p = wave * 2 + 8 * j;
+                if (p < n_count) { // wave-uniform
+                    const uint16_t *w_a = a.W + (int64_t)e * a.w_es + (int64_t)(n_first + p) * a.ldw + kp;
+                    const uint16_t *w_b = w_a + a.ldw;
+                    u32x4 wa[4], wb[4]; // this lane's pieces lane, lane + 64, ... of either row, all in flight
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int c = lane + 64 * q;
+                        wa[q] = wb[q] = u32x4{0u, 0u, 0u, 0u};
+                        if (c < pc) {
+                            wa[q] = __builtin_nontemporal_load((const u32x4 *)(w_a + 8 * c));
+                            wb[q] = __builtin_nontemporal_load((const u32x4 *)(w_b + 8 * c));
+                        }
                     }
-                }
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int c = c0 + 64 * q;
-                    if (c < chunks) {
-                        float fa[8], fb[8];
-                        fr_unpack<T>(wa[q], fa);
-                        fr_unpack<T>(wb[q], fb);
+                    for (int q = 0; q < 4; ++q) {
+                        const int c = lane + 64 * q;
+                        if (c < pc) {
+                            float fa[8], fb[8];
+                            fr_unpack<T>(wa[q], fa);
+                            fr_unpack<T>(wb[q], fb);
 #pragma unroll
-                        for (int u = 0; u < RC; ++u) {
-                            float fx[8];
-                            fr_unpack<T>(*(const u32x4 *)(s_x + ((int64_t)u * chunks + c) * 8), fx);
+                            for (int u = 0; u < RC; ++u) {
+                                float fx[8];
+                                fr_unpack<T>(*(const u32x4 *)(s_x + (u * (FR_NT_PIECE / 8) + c) * 8), fx);
 #pragma unroll
-                            for (int i = 0; i < 8; ++i) {
-                                s[u][0] = __builtin_fmaf(fx[i], fa[i], s[u][0]);
-                                s[u][1] = __builtin_fmaf(fx[i], fb[i], s[u][1]);
+                                for (int i = 0; i < 8; ++i) {
+                                    s[j][u][0] = __builtin_fmaf(fx[i], fa[i], s[j][u][0]);
+                                    s[j][u][1] = __builtin_fmaf(fx[i], fb[i], s[j][u][1]);
+                                }
                             }
                         }
                     }
                 }
             }
+        }
+#pragma unroll
+        for (int j = 0; j < FR_NT_PAIRS; ++j) {
+            const int p = wave * 2 + 8 * j;
+            if (p >= n_count) break; // wave-uniform
+            const int n_a = n_first + p, n_b = n_a + 1;
 #pragma unroll
             for (int u = 0; u < RC; ++u)
 #pragma unroll
                 for (int h = 0; h < 2; ++h)
 #pragma unroll
-                    for (int d = 32; d > 0; d >>= 1) s[u][h] += __shfl_xor(s[u][h], d);
+                    for (int d = 32; d > 0; d >>= 1) s[j][u][h] += __shfl_xor(s[j][u][h], d);
             if (lane == 0) {
 #pragma unroll
                 for (int u = 0; u < RC; ++u) {
                     const int64_t r = r0 + u;
                     if (r >= hi) continue;
                     if constexpr (EPI < 0) { // the sums go to the workspace, the epilogue kernel follows
-                        part[r * a.N + n_a] = s[u][0];
-                        if (p + 1 < n_count) part[r * a.N + n_b] = s[u][1];
-                    } else { // the only part there is: bias, scale and the epilogue right here (n_a is even, n_b = n_a + 1)
+                        part[r * a.N + n_a] = s[j][u][0];
+                        part[r * a.N + n_b] = s[j][u][1];
+                    } else { // the only part there is: bias, scale and the epilogue right here (n_a is even)
                         const int64_t s_idx = a.idx ? a.idx[r] : r;
                         const float sc = a.scale ? fr_scalar<T>(a.scale, s_idx) : 1.f;
                         const int64_t dst = a.y_grouped ? r : s_idx;
-                        float v0 = s[u][0], v1 = s[u][1];
+                        float v0 = s[j][u][0], v1 = s[j][u][1];
                         if (a.bias) v0 += fr_scalar<T>(a.bias, (int64_t)e * a.bias_es + n_a), v1 += fr_scalar<T>(a.bias, (int64_t)e * a.bias_es + n_b);
                         const uint32_t z = Elem<T>::pack(v0 * sc, v1 * sc);
                         if (a.out) *(uint32_t *)(a.out + dst * a.ldo + n_a) = z;
@@ -249,8 +262,8 @@ __device__ __forceinline__ void fr_nt_rows(const FwdArgs &a, float *__restrict__
 // EPI = XMA_ROCM_EPI_STORE or _SWIGLU: the wave that holds a pair of sums applies bias, scale and epilogue itself (the
 // columns of a pair are (gate, up)); EPI = -1: the sums go to the workspace for fr_epilogue_kernel.
 template <typename T, int EPI>
-__global__ __launch_bounds__(FR_THREADS) void fr_nt_kernel(const FwdArgs a, float *__restrict__ part, int rows_per_wg) {
-    extern __shared__ __attribute__((aligned(16))) uint16_t s_x_nt[];
+__global__ __launch_bounds__(FR_THREADS, 4) void fr_nt_kernel(const FwdArgs a, float *__restrict__ part, int rows_per_wg) {
+    __shared__ __attribute__((aligned(16))) uint16_t s_x_nt[4 * FR_NT_PIECE];
     const int e = blockIdx.y;
     const int64_t lo = e ? a.offs[e - 1] : 0, hi = a.offs[e];
     if (lo >= hi) return; // uniform
@@ -411,22 +424,18 @@ template <typename T> int fr_launch(const FwdArgs &a, int w_is_kn, int epilogue,
         fr_nn_kernel<T><<<grid, FR_THREADS, (size_t)8 * kc * sizeof(float), st>>>(a, part, kc);
         if ((rc = xma_check_launch("fr_nn_kernel"))) return rc;
     } else {
-        const int rows_per_wg = (a.K >= 2048) ? FR_NT_ROWS : 8; // short rows: one pair of rows per wave, more workgroups
+        // one pair of rows per wave instead of four where the rows are short or the launch would have few workgroups
+        const int rows_per_wg = (a.K >= 2048 && (int64_t)(a.N / FR_NT_ROWS) * a.E >= 2048) ? FR_NT_ROWS : 8;
         const dim3 grid((a.N + rows_per_wg - 1) / rows_per_wg, a.E);
-        const size_t lds = (size_t)4 * a.K * sizeof(uint16_t);
-        const int max_lds = 4 * FR_NT_KMAX * (int)sizeof(uint16_t);
         if (epilogue == XMA_ROCM_EPI_STORE) {
-            if (lds > 48 * 1024 && (rc = xma_set_max_lds_once((const void *)fr_nt_kernel<T, XMA_ROCM_EPI_STORE>, max_lds))) return rc;
-            fr_nt_kernel<T, XMA_ROCM_EPI_STORE><<<grid, FR_THREADS, lds, st>>>(a, part, rows_per_wg);
+            fr_nt_kernel<T, XMA_ROCM_EPI_STORE><<<grid, FR_THREADS, 0, st>>>(a, part, rows_per_wg);
             return xma_check_launch("fr_nt_kernel");
         }
         if (epilogue == XMA_ROCM_EPI_SWIGLU) {
-            if (lds > 48 * 1024 && (rc = xma_set_max_lds_once((const void *)fr_nt_kernel<T, XMA_ROCM_EPI_SWIGLU>, max_lds))) return rc;
-            fr_nt_kernel<T, XMA_ROCM_EPI_SWIGLU><<<grid, FR_THREADS, lds, st>>>(a, part, rows_per_wg);
+            fr_nt_kernel<T, XMA_ROCM_EPI_SWIGLU><<<grid, FR_THREADS, 0, st>>>(a, part, rows_per_wg);
             return xma_check_launch("fr_nt_kernel");
         }
-        if (lds > 48 * 1024 && (rc = xma_set_max_lds_once((const void *)fr_nt_kernel<T, -1>, max_lds))) return rc;
-        fr_nt_kernel<T, -1><<<grid, FR_THREADS, lds, st>>>(a, part, rows_per_wg);
+        fr_nt_kernel<T, -1><<<grid, FR_THREADS, 0, st>>>(a, part, rows_per_wg);
         if ((rc = xma_check_launch("fr_nt_kernel"))) return rc;
     }
     const dim3 egrid((a.N / 2 + FR_THREADS - 1) / FR_THREADS, (unsigned)a.M);
@@ -466,8 +475,6 @@ extern "C" int xma_rocm_scatter2scatter_few_rows(const void *X, int64_t ldx, con
                 "scatter2scatter_few_rows: M=%lld N=%d K=%d E=%d fan_out=%d (M and E at most 65535)", (long long)M, N, K, E, fan_out);
     XMA_REQUIRE(N % 8 == 0 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldo % 8 == 0 && w_expert_stride % 8 == 0,
                 XMA_ROCM_EUNSUPPORTED, "scatter2scatter_few_rows: N=%d K=%d and the leading dimensions must be multiples of 8", N, K);
-    XMA_REQUIRE(w_is_kn || K <= FR_NT_KMAX, XMA_ROCM_EUNSUPPORTED, "scatter2scatter_few_rows: K=%d exceeds %d for W as (N, K)", K,
-                FR_NT_KMAX);
     XMA_REQUIRE(!w_is_kn || fr_nn_range(K) <= FR_NN_KC_MAX, XMA_ROCM_EUNSUPPORTED,
                 "scatter2scatter_few_rows: K=%d exceeds %d for W as (K, N)", K, FR_NN_KC_MAX * FR_NN_SPLITS);
     if (M == 0) return XMA_ROCM_OK;

@@ -161,8 +161,7 @@ def scatter2scatter_workspace_bytes(M: int, N: int, K: int, E: int, device_index
     return _S2S_WORKSPACE_BYTES[key]
 
 
-FEW_ROWS_NT_MAX_K = 8192  # limits of the few-token entry point for the two weight layouts
-FEW_ROWS_NN_MAX_K = 65536
+FEW_ROWS_NN_MAX_K = 65536  # limit of the few-token entry point for W as (K, N)
 
 
 def _few_rows(M: int, E: int, dtype: torch.dtype) -> bool:
@@ -172,7 +171,7 @@ def _few_rows(M: int, E: int, dtype: torch.dtype) -> bool:
 
 def _few_rows_fwd(lib, M: int, N: int, K: int, E: int, w_is_kn: int, dtype: torch.dtype) -> bool:
     """the same for a forward-type GEMM, whose few-token entry point has limits of its own"""
-    if not _few_rows(M, E, dtype) or K > (FEW_ROWS_NN_MAX_K if w_is_kn else FEW_ROWS_NT_MAX_K):
+    if not _few_rows(M, E, dtype) or (w_is_kn and K > FEW_ROWS_NN_MAX_K):
         return False
     return lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, w_is_kn) <= FEW_ROWS_MAX_WORKSPACE
 

@@ -204,7 +204,7 @@ XMA_API int xma_rocm_down_projection_dx_swiglu(const void *dY, int64_t lddy, con
  * xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, w_is_kn) bytes) to a small kernel that applies the bias and
  * the epilogue with the arithmetic of the MFMA kernels; W as (N, K) with STORE or SWIGLU finishes in one kernel and takes
  * no workspace (NULL, 0).
- * Limits: M and E at most 65535, K at most 8192 for W as (N, K) and 65536 for W as (K, N).  Correct for any M, but the
+ * Limits: M and E at most 65535, K at most 65536 for W as (K, N).  Correct for any M, but the
  * time grows with (rows per expert) x |W|: meant for launches of a few rows per expert (the torch ops of this package
  * take it up to six on average).  No counterpart in the reference
  * (its kernel is the same for every size).
