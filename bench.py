@@ -543,7 +543,8 @@ def run_small_t(args):
     """Latency of one forward + backward of the expert computation with a handful of tokens, the case the reference's
     own test runs (7 tokens, tests/layers/moe_test.py:107) at its two size points (moe_test.py:26-53), and with 64
     tokens: eager, and replayed from a HIP graph (no host launch overhead), beside the time the weights touched by the
-    step need to stream through HBM once per use at 8 TB/s (forward, dX and the dW store: three uses)."""
+    step need to stream through HBM once per use at 8 TB/s (forward, dX and the dW store: three uses); and the forward
+    alone (router, routing, both projections, combine) from a graph, the step of a decoding loop."""
     from xma import KernelBackend, set_seed
     from xma.functional import swiglu_packed
     from xma.layers import MoE
@@ -581,6 +582,17 @@ def run_small_t(args):
             with torch.cuda.graph(g_):
                 step()
             graph_ms = _time_gpu(g_.replay, max(args.steps, 20), warmup=5)
+            def forward_only():
+                with torch.no_grad():
+                    w, ids = R.router_topk(lg, k, ids_dtype=torch.int32)
+                    return moe._compute_experts(x, w, ids, kernel_backend=KernelBackend.rocm)
+
+            forward_only()
+            torch.cuda.synchronize()
+            gf = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gf):
+                forward_only()
+            fwd_graph_ms = _time_gpu(gf.replay, max(args.steps, 20), warmup=5)
             _, sel = R.router_topk(lg.detach(), k)
             touched = int(torch.unique(sel).numel())
             wbytes = (2 * I * H + H * I) * 2  # both matrices of one expert
@@ -588,6 +600,8 @@ def run_small_t(args):
             res[f"E{E}_k{k}_H{H}_I{I}_T{T}"] = {
                 "eager_ms": round(eager_ms, 4), "graph_ms": round(graph_ms, 4), "experts_touched": touched,
                 "gemm_kernels": "few_rows (weights streamed, vector FMAs)" if _ops._few_rows(T * k, E, torch.bfloat16) else "mfma tiles",
+                "forward_only_graph_ms": round(fwd_graph_ms, 4),
+                "forward_only_weight_stream_ms_at_8TBs": round(touched * wbytes / PEAK_HBM_GBS / 1e6, 4),
                 "weight_stream_ms_at_8TBs": round(stream_bytes / PEAK_HBM_GBS / 1e6, 4),
                 "graph_over_stream": round(graph_ms / (stream_bytes / PEAK_HBM_GBS / 1e6), 2),
             }
