@@ -24,16 +24,17 @@ def _make(T=300, E=8, k=2, H=256, I=512, dtype=torch.bfloat16, seed=0):
     return moe, x
 
 
+@pytest.mark.parametrize("T", [300, 7])  # 7 tokens: the grouped GEMMs take the kernels of the few-token regime
 @pytest.mark.parametrize("k", [2, 4])  # 4: the backward that takes dW2 from the scaled activations of the dX2 epilogue
 @pytest.mark.parametrize("backend", ["aot_eager", "inductor"])
-def test_compiled_module_matches_eager(backend, k):
+def test_compiled_module_matches_eager(backend, k, T):
     """torch.compile(fullgraph=True) of the module, with the tracing-only backend and with the default one the
     reference's test uses (tests/layers/moe_test.py:104-105 passes no backend, i.e. inductor): the custom ops mutate
     caller-allocated outputs, so functionalisation has to carry them through unchanged."""
     from xma import KernelBackend
 
     torch._dynamo.reset()
-    moe, x = _make(k=k)
+    moe, x = _make(T=T, k=k)
     print("compile: eager run", flush=True)
     xe = x.clone().requires_grad_()
     ye, _ = moe(xe, kernel_backend=KernelBackend.rocm)
@@ -117,15 +118,16 @@ def test_compiled_functionals_match_eager(backend):
         raise
 
 
+@pytest.mark.parametrize("T", [300, 7])  # 7 tokens: the kernels of the few-token regime, whose passes depend on the routing
 @pytest.mark.parametrize("k", [2, 4])
-def test_graph_capture_and_replay(k):
+def test_graph_capture_and_replay(k, T):
     """fwd + bwd of the router (behind the gate) and of the expert computation captured once and replayed on new
     inputs (new routing included); every replay is checked against an eager run, with eager work and synchronisations
     in between."""
     from xma import KernelBackend
 
     E = 8
-    moe, x = _make(E=E, k=k)
+    moe, x = _make(T=T, E=E, k=k)
     T, H = x.shape
     g = torch.Generator(device="cuda").manual_seed(1)
 
