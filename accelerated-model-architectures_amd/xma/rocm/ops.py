@@ -83,10 +83,12 @@ def continuous_count_rocm(x: torch.Tensor, y: torch.Tensor, workspace: torch.Ten
 
 CONTINUOUS_COUNT_SET_MAX_BINS = 8192
 # The grouped GEMMs take the entry points written for the few-token regime, which stream the weights instead of tiling
-# them for the matrix pipes, up to FEW_ROWS_PER_EXPERT rows per expert on average (the expert's rows are walked 4 or 8 at a
-# time, each pass streaming its weights again: measured cross-over at 6 - 7 rows per expert) and FEW_ROWS_MAX rows in all.
-FEW_ROWS_MAX = 256
-FEW_ROWS_PER_EXPERT = 6
+# them for the matrix pipes, up to FEW_ROWS_PER_EXPERT rows per expert on average and FEW_ROWS_MAX rows in all.  The limits
+# are the measured cross-overs (8 experts, H = 2048, I = 8192): an expert's rows are walked 4 at a time by the x @ W^T
+# kernel and 8 at a time by the dy @ W kernel, each pass streaming the weights again; the weight gradient grows slowly
+# with the rows.
+FEW_ROWS_MAX = 256  # beyond that the per-row work of these kernels shows where the experts are small (128 experts of 0.4 MB)
+FEW_ROWS_PER_EXPERT = {"x @ W^T": 4, "dy @ W": 8, "dW": 16}
 FEW_ROWS_MAX_WORKSPACE = 256 << 20  # bytes of fp32 partial sums a forward-type launch may ask for
 
 
@@ -164,14 +166,14 @@ def scatter2scatter_workspace_bytes(M: int, N: int, K: int, E: int, device_index
 FEW_ROWS_NN_MAX_K = 65536  # limit of the few-token entry point for W as (K, N)
 
 
-def _few_rows(M: int, E: int, dtype: torch.dtype) -> bool:
+def _few_rows(M: int, E: int, dtype: torch.dtype, form: str) -> bool:
     """whether a grouped GEMM of M rows over E experts takes an entry point written for the few-token regime"""
-    return 0 < M <= min(FEW_ROWS_MAX, FEW_ROWS_PER_EXPERT * E) and dtype in (torch.bfloat16, torch.float16)
+    return 0 < M <= min(FEW_ROWS_MAX, FEW_ROWS_PER_EXPERT[form] * E) and dtype in (torch.bfloat16, torch.float16)
 
 
 def _few_rows_fwd(lib, M: int, N: int, K: int, E: int, w_is_kn: int, dtype: torch.dtype) -> bool:
     """the same for a forward-type GEMM, whose few-token entry point has limits of its own"""
-    if not _few_rows(M, E, dtype) or (w_is_kn and K > FEW_ROWS_NN_MAX_K):
+    if not _few_rows(M, E, dtype, "dy @ W" if w_is_kn else "x @ W^T") or (w_is_kn and K > FEW_ROWS_NN_MAX_K):
         return False
     return lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, w_is_kn) <= FEW_ROWS_MAX_WORKSPACE
 
@@ -350,7 +352,7 @@ def group_bwd_W_rocm(
         assert dy_scale.dtype == DY.dtype and dy_scale.is_contiguous()
     lib = get_library()
     # a handful of rows per expert (the index has one entry per row): the launch is a stream of stores, not arithmetic
-    few = _few_rows(sorted_scattered_idxs.numel(), E, DW.dtype)
+    few = _few_rows(sorted_scattered_idxs.numel(), E, DW.dtype, "dW")
     name = "xma_rocm_group_bwd_W_few_rows" if few else "xma_rocm_group_bwd_W"
     check(
         getattr(lib, name)(

@@ -599,7 +599,7 @@ def run_small_t(args):
             stream_bytes = 2 * touched * wbytes + E * wbytes  # forward and dX read the touched experts, dW writes all
             res[f"E{E}_k{k}_H{H}_I{I}_T{T}"] = {
                 "eager_ms": round(eager_ms, 4), "graph_ms": round(graph_ms, 4), "experts_touched": touched,
-                "gemm_kernels": "few_rows (weights streamed, vector FMAs)" if _ops._few_rows(T * k, E, torch.bfloat16) else "mfma tiles",
+                "gemm_kernels": {form: ("few_rows" if _ops._few_rows(T * k, E, torch.bfloat16, form) else "mfma tiles") for form in _ops.FEW_ROWS_PER_EXPERT},
                 "forward_only_graph_ms": round(fwd_graph_ms, 4),
                 "forward_only_weight_stream_ms_at_8TBs": round(touched * wbytes / PEAK_HBM_GBS / 1e6, 4),
                 "weight_stream_ms_at_8TBs": round(stream_bytes / PEAK_HBM_GBS / 1e6, 4),

@@ -40,7 +40,7 @@ class _few_rows_limit:
         from xma.rocm import ops
 
         self.saved = (ops.FEW_ROWS_MAX, ops.FEW_ROWS_PER_EXPERT)
-        ops.FEW_ROWS_MAX, ops.FEW_ROWS_PER_EXPERT = self.limit, 1 << 30
+        ops.FEW_ROWS_MAX, ops.FEW_ROWS_PER_EXPERT = self.limit, dict.fromkeys(ops.FEW_ROWS_PER_EXPERT, 1 << 30)
 
     def __exit__(self, *exc):
         from xma.rocm import ops
