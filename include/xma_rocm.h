@@ -206,7 +206,7 @@ XMA_API int xma_rocm_down_projection_dx_swiglu(const void *dY, int64_t lddy, con
  * no workspace (NULL, 0).
  * Limits: M and E at most 65535, K at most 65536 for W as (K, N).  Correct for any M, but the
  * time grows with (rows per expert) x |W|: meant for launches of a few rows per expert (the torch ops of this package
- * take it up to six on average).  No counterpart in the reference
+ * take it up to 4 on average for W as (N, K) and 8 for W as (K, N)).  No counterpart in the reference
  * (its kernel is the same for every size).
  */
 XMA_API size_t xma_rocm_scatter2scatter_few_rows_workspace_bytes(int64_t M, int32_t N, int32_t K, int w_is_kn);
@@ -242,7 +242,7 @@ XMA_API int xma_rocm_group_bwd_W(const void *DY, int64_t lddy, int dy_grouped, i
  * stores and adds one outer product per row of the expert with vector FMAs: with a handful of rows per expert the launch
  * runs at the rate of a fill of DW, where the MFMA tiles of xma_rocm_group_bwd_W spend a prologue, one K step and an
  * epilogue per 256 x 256 tile.  Correct for any number of rows, but its time grows with (rows per expert) x |DW|: meant
- * for launches of a few rows per expert.  No counterpart in the reference (its kernel is the same for every size).
+ * for launches of a few rows per expert (the torch ops take it up to 16 on average).  No counterpart in the reference (its kernel is the same for every size).
  */
 XMA_API int xma_rocm_group_bwd_W_few_rows(const void *DY, int64_t lddy, int dy_grouped, int32_t dy_fan_out,
                                   const void *dy_scale, const void *X, int64_t ldx, int x_grouped, int32_t x_fan_out,
