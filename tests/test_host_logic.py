@@ -66,9 +66,41 @@ def test_argument_errors_are_reported_before_any_launch():
     assert lib.xma_rocm_router_topk(None, 8, 4, 8, 2, 0, None, None, 1, None) == -1  # null pointers with T > 0
     assert lib.xma_rocm_router_topk_bwd(None, 8, 4, 8, 2, 0, None, 1, None, None, 4, None) == -1  # ldd < E
     assert lib.xma_rocm_router_topk(None, 8, 0, 8, 2, 0, None, None, 1, None) == 0
+    # the few-token entry points: dtype (no fp32), M beyond the epilogue's grid, a missing workspace where sums go through
+    # one (W as (K, N)), none needed for W as (N, K) with a plain store (fails later, on the null operands), dW shapes
+    p = ctypes.c_void_p(256)
+    few = lib.xma_rocm_scatter2scatter_few_rows
+    assert few(p, 64, p, 64 * 64, 64, 0, p, p, p, 64, None, 0, None, 0, None, None, 0, 4, 64, 64, 2, 1, 1, 1, 0, 2, None, 0, None) == -2
+    assert few(p, 64, p, 64 * 64, 64, 0, p, p, p, 64, None, 0, None, 0, None, None, 0, 70000, 64, 64, 2, 1, 1, 1, 0, 0, None, 0, None) == -1
+    assert few(p, 64, p, 64 * 64, 64, 1, p, p, p, 64, None, 0, None, 0, None, None, 0, 4, 64, 64, 2, 1, 1, 1, 0, 0, None, 0, None) == -3
+    assert b"workspace" in lib.xma_rocm_last_error()
+    assert few(None, 64, None, 64 * 64, 64, 0, p, p, p, 64, None, 0, None, 0, None, None, 0, 4, 64, 64, 2, 1, 1, 1, 0, 0, None, 0, None) == -1
+    assert b"null or misaligned" in lib.xma_rocm_last_error()
+    assert lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes(4, 64, 64, 0) == 4 * 64 * 4
+    assert lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes(4, 64, 16384, 1) == 64 * 4 * 64 * 4  # 64 ranges of K
+    assert lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes(0, 64, 64, 1) == 0
+    dw = lib.xma_rocm_group_bwd_W_few_rows
+    assert dw(p, 64, 1, 1, None, p, 64, 1, 1, p, p, p, 64 * 64, 64, 64, 64, 2, 2, None) == -2  # fp32
+    assert dw(p, 64, 1, 1, None, p, 60, 1, 1, p, p, p, 64 * 64, 64, 64, 64, 2, 0, None) == -2  # ldx % 8
+    assert dw(None, 64, 1, 1, None, p, 64, 1, 1, p, p, p, 64 * 64, 64, 64, 64, 2, 0, None) == -1
     # empty problems are accepted without touching a pointer
+    assert few(None, 64, None, 64 * 64, 64, 0, None, None, None, 64, None, 0, None, 0, None, None, 0, 0, 64, 64, 2, 1, 1, 1, 0, 0, None, 0, None) == 0
     assert lib.xma_rocm_combine(None, 8, None, None, 8, 0, 2, 16, 0, None) == 0
     assert lib.xma_rocm_continuous_count(None, 0, 0, ctypes.c_void_p(16), 4, None, 0, None) == 0
+
+
+def test_few_token_dispatch_rule():
+    """which grouped GEMM forms take the kernels of the few-token regime: by rows per expert on average, per form, with a
+    cap on the rows in all; fp32 never"""
+    from xma.rocm import ops
+
+    bf = torch.bfloat16
+    assert ops._few_rows(14, 8, bf, "x @ W^T") and ops._few_rows(32, 8, bf, "x @ W^T") and not ops._few_rows(33, 8, bf, "x @ W^T")
+    assert ops._few_rows(64, 8, bf, "dy @ W") and not ops._few_rows(65, 8, bf, "dy @ W")
+    assert ops._few_rows(128, 8, bf, "dW") and not ops._few_rows(129, 8, bf, "dW")
+    assert ops._few_rows(256, 128, bf, "x @ W^T") and not ops._few_rows(257, 128, bf, "dW")  # the cap on the rows in all
+    assert not ops._few_rows(0, 8, bf, "dW") and not ops._few_rows(14, 8, torch.float32, "dW")
+    assert ops._few_rows(14, 8, torch.float16, "dy @ W")
 
 
 def test_fused_router_shape_rule_matches_the_library():
