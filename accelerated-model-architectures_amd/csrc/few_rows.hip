@@ -155,6 +155,8 @@ namespace {
 //       the X values of the range sit in LDS as floats.  S = K / range.
 // ------------------------------------------------------------------------------------------------
 constexpr int FR_NT_ROWS = 32;  // rows of W per workgroup (8 per wave, two at a time); 8 when the rows are short
+constexpr int FR_NT_VALU_ROWS_PER_EXPERT = 4; // on average; beyond that x @ W^T takes the small MFMA tile,
+constexpr int FR_NT_VALU_ROWS = 256;            // and beyond this many rows in all (the vector kernel's work per row)
 constexpr int FR_NT_PIECE = 2048; // elements of K whose X values are staged in LDS at a time (4 rows: 16 KB)
 constexpr int FR_NT_PAIRS = FR_NT_ROWS / 8; // pairs of rows of W per wave
 
@@ -415,6 +417,126 @@ __global__ __launch_bounds__(FR_THREADS) void fr_epilogue_kernel(const FwdArgs a
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// x @ W^T for 5 to 32 rows per expert: too many for vector FMAs (one pass over the weights per 4 rows), too few for the
+// 256 x 256 tiles (one 32 KB stage of weights in flight per compute unit).  A small MFMA tile instead: 32 rows of the
+// expert x 128 rows of W[e], K in steps of 64, operands through registers into two LDS stages of 20 KB, so that four
+// workgroups share a compute unit and keep 80 KB of loads in flight.  One v_mfma_f32_32x32x16 block per wave; lane l holds
+// 16 sums of row l % 32 in quads of 4 consecutive columns, so bias, row scale and the STORE / SWIGLU epilogue are
+// lane-local, with the arithmetic of tile_epilogue in grouped_gemm.hip.  An expert's rows are taken 32 at a time.
+// ------------------------------------------------------------------------------------------------
+constexpr int ST_M = 32, ST_N = 128, ST_K = 64;
+constexpr int ST_W_BYTES = ST_N * ST_K * 2, ST_X_BYTES = ST_M * ST_K * 2, ST_STAGE = ST_W_BYTES + ST_X_BYTES;
+
+// 16-byte slot of (row, chunk) in a tile of 128-byte rows: chunk ^ (row & 7) keeps 8 consecutive rows off each other's banks
+__device__ __forceinline__ int st_slot(int row, int chunk) { return row * 128 + ((chunk ^ (row & 7)) << 4); }
+
+// EPI = -1: the launch is cut along K (blockIdx.z takes `steps_per` steps) because N alone gives too few workgroups; the
+// fp32 sums go to part[blockIdx.z][M][N] and fr_epilogue_kernel finishes.
+template <typename T, int EPI>
+__global__ __launch_bounds__(FR_THREADS) void fr_nt_tile_kernel(const FwdArgs a, float *__restrict__ part, int steps_per) {
+    __shared__ __attribute__((aligned(16))) unsigned char s_t[2 * ST_STAGE];
+    const int e = blockIdx.y;
+    const int64_t lo = e ? a.offs[e - 1] : 0, hi = a.offs[e];
+    if (lo >= hi) return; // uniform
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
+    const int n0 = blockIdx.x * ST_N;
+    const int steps_all = (a.K + ST_K - 1) / ST_K;
+    const int s_begin = (EPI < 0) ? blockIdx.z * steps_per : 0;
+    const int s_end = (EPI < 0 && s_begin + steps_per < steps_all) ? s_begin + steps_per : steps_all;
+    // loader: thread = (row tid / 8 (+ 32 i), chunk tid % 8)
+    const int ld_row = tid >> 3, ld_chunk = tid & 7;
+    const uint16_t *w_src[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int n = n0 + ld_row + 32 * i;
+        if (n >= a.N) n = a.N - 1; // clamped: computed, never stored
+        w_src[i] = a.W + (int64_t)e * a.w_es + (int64_t)n * a.ldw + 8 * ld_chunk;
+    }
+    for (int64_t r0 = lo; r0 < hi; r0 += ST_M) {
+        int64_t xr = r0 + ld_row;
+        if (xr >= hi) xr = hi - 1;
+        const uint16_t *x_src = a.X + fr_src_row(a, xr) * a.ldx + 8 * ld_chunk;
+        u32x4 wv[4], xv;
+        auto fetch = [&](int s) {
+            const bool ok = s * ST_K + 8 * ld_chunk < a.K; // chunks past K are zeros
+#pragma unroll
+            for (int i = 0; i < 4; ++i) wv[i] = ok ? __builtin_nontemporal_load((const u32x4 *)(w_src[i] + s * ST_K)) : u32x4{0u, 0u, 0u, 0u};
+            xv = ok ? *(const u32x4 *)(x_src + s * ST_K) : u32x4{0u, 0u, 0u, 0u};
+        };
+        auto stash = [&](int stage) {
+            unsigned char *base = s_t + stage * ST_STAGE;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) *(u32x4 *)(base + st_slot(ld_row + 32 * i, ld_chunk)) = wv[i];
+            *(u32x4 *)(base + ST_W_BYTES + st_slot(ld_row, ld_chunk)) = xv;
+        };
+        f32x16 acc;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+        __syncthreads(); // the pass before no longer reads the stages
+        fetch(s_begin);
+        stash(s_begin & 1);
+        __syncthreads();
+        for (int s = s_begin; s < s_end; ++s) {
+            if (s + 1 < s_end) fetch(s + 1); // in flight while this step computes
+            const unsigned char *base = s_t + (s & 1) * ST_STAGE;
+#pragma unroll
+            for (int kk = 0; kk < 4; ++kk) {
+                const u32x4 wa = *(const u32x4 *)(base + st_slot(wave * 32 + l32, 2 * kk + half));
+                const u32x4 xb = *(const u32x4 *)(base + ST_W_BYTES + st_slot(l32, 2 * kk + half));
+                acc = Elem<T>::mfma(wa, xb, acc);
+            }
+            if (s + 1 < s_end) stash((s + 1) & 1); // that stage was last read in step s - 1, behind a barrier
+            __syncthreads();
+        }
+        const int64_t r = r0 + l32;
+        if (r >= hi) continue;
+        if constexpr (EPI < 0) {
+            float *mine = part + ((int64_t)blockIdx.z * a.M + r) * a.N;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = n0 + wave * 32 + 8 * g + 4 * half;
+                if (n < a.N) *(float4 *)(mine + n) = make_float4(acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]);
+            }
+            continue;
+        }
+        const int64_t s_idx = a.idx ? a.idx[r] : r;
+        const float sc = a.scale ? fr_scalar<T>(a.scale, s_idx) : 1.f;
+        const int64_t dst = a.y_grouped ? r : s_idx;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int n = n0 + wave * 32 + 8 * g + 4 * half; // acc[4 g + q] is column n + q of row r
+            if (n >= a.N) continue;
+            float v[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                v[q] = acc[4 * g + q];
+                if (a.bias) v[q] += fr_scalar<T>(a.bias, (int64_t)e * a.bias_es + n + q);
+                v[q] *= sc;
+            }
+            const uint32_t z0 = Elem<T>::pack(v[0], v[1]), z1 = Elem<T>::pack(v[2], v[3]);
+            if (a.out) *(u32x2 *)(a.out + dst * a.ldo + n) = u32x2{z0, z1};
+            if constexpr (EPI == XMA_ROCM_EPI_SWIGLU) {
+                const float g0 = Elem<T>::lo(z0), u0 = Elem<T>::hi(z0), g1 = Elem<T>::lo(z1), u1 = Elem<T>::hi(z1);
+                *(uint32_t *)(a.aux + dst * a.ldaux + (n >> 1)) = Elem<T>::pack(u0 * g0 * sigmoidf_fast(g0), u1 * g1 * sigmoidf_fast(g1));
+            }
+        }
+    }
+}
+
+// x @ W^T: more than a pass or two of the vector kernel per expert -> the small MFMA tile
+inline bool fr_nt_takes_tile(int64_t M, int E) { return M > (int64_t)FR_NT_VALU_ROWS_PER_EXPERT * E || M > FR_NT_VALU_ROWS; }
+
+// K ranges of the small MFMA tile: enough workgroups for four per compute unit (twice as many measured slower: the
+// partial sums and their kernel cost more than the extra parallelism brings), ranges of at least 8 steps
+inline int fr_tile_splits(int N, int K, int E) {
+    const int64_t wgs = (int64_t)((N + ST_N - 1) / ST_N) * E;
+    const int steps = (K + ST_K - 1) / ST_K;
+    int S = (int)((1024 + wgs - 1) / wgs);
+    if (S > steps / 8) S = steps / 8;
+    return S < 1 ? 1 : S;
+}
+
 template <typename T> int fr_launch(const FwdArgs &a, int w_is_kn, int epilogue, float *part, hipStream_t st) {
     int S = 1, rc;
     if (w_is_kn) {
@@ -424,6 +546,28 @@ template <typename T> int fr_launch(const FwdArgs &a, int w_is_kn, int epilogue,
         fr_nn_kernel<T><<<grid, FR_THREADS, (size_t)8 * kc * sizeof(float), st>>>(a, part, kc);
         if ((rc = xma_check_launch("fr_nn_kernel"))) return rc;
     } else {
+        if (epilogue != XMA_ROCM_EPI_SWIGLU_BWD && fr_nt_takes_tile(a.M, a.E)) {
+            // more than a pass or two of the vector kernel per expert: the small MFMA tile
+            const int S = fr_tile_splits(a.N, a.K, a.E);
+            const int steps_all = (a.K + ST_K - 1) / ST_K, steps_per = (steps_all + S - 1) / S;
+            const dim3 grid((a.N + ST_N - 1) / ST_N, a.E, S);
+            if (S == 1) {
+                if (epilogue == XMA_ROCM_EPI_STORE)
+                    fr_nt_tile_kernel<T, XMA_ROCM_EPI_STORE><<<grid, FR_THREADS, 0, st>>>(a, nullptr, steps_all);
+                else
+                    fr_nt_tile_kernel<T, XMA_ROCM_EPI_SWIGLU><<<grid, FR_THREADS, 0, st>>>(a, nullptr, steps_all);
+                return xma_check_launch("fr_nt_tile_kernel");
+            }
+            fr_nt_tile_kernel<T, -1><<<grid, FR_THREADS, 0, st>>>(a, part, steps_per);
+            if ((rc = xma_check_launch("fr_nt_tile_kernel"))) return rc;
+            const dim3 egrid((a.N / 2 + FR_THREADS - 1) / FR_THREADS, (unsigned)a.M);
+            const int parts = (steps_all + steps_per - 1) / steps_per;
+            if (epilogue == XMA_ROCM_EPI_STORE)
+                fr_epilogue_kernel<T, XMA_ROCM_EPI_STORE><<<egrid, FR_THREADS, 0, st>>>(a, part, parts);
+            else
+                fr_epilogue_kernel<T, XMA_ROCM_EPI_SWIGLU><<<egrid, FR_THREADS, 0, st>>>(a, part, parts);
+            return xma_check_launch("fr_epilogue_kernel");
+        }
         // one pair of rows per wave instead of four where the rows are short or the launch would have few workgroups
         const int rows_per_wg = (a.K >= 2048 && (int64_t)(a.N / FR_NT_ROWS) * a.E >= 2048) ? FR_NT_ROWS : 8;
         const dim3 grid((a.N + rows_per_wg - 1) / rows_per_wg, a.E);
@@ -450,12 +594,20 @@ template <typename T> int fr_launch(const FwdArgs &a, int w_is_kn, int epilogue,
 
 } // namespace
 
-extern "C" size_t xma_rocm_scatter2scatter_few_rows_workspace_bytes(int64_t M, int32_t N, int32_t K, int w_is_kn) {
-    if (M <= 0 || N <= 0 || K <= 0) return 0;
-    int S = 1;
-    if (w_is_kn) {
+extern "C" size_t xma_rocm_scatter2scatter_few_rows_workspace_bytes(int64_t M, int32_t N, int32_t K, int32_t E, int w_is_kn,
+                                                                    int epilogue) {
+    if (M <= 0 || N <= 0 || K <= 0 || E <= 0) return 0;
+    int S;
+    if (w_is_kn) { // partial sums of the K ranges
         const int kc = fr_nn_range(K);
         S = (K + kc - 1) / kc;
+    } else if (epilogue == XMA_ROCM_EPI_SWIGLU_BWD) {
+        S = 1; // the vector kernel's sums go to the epilogue kernel
+    } else if (fr_nt_takes_tile(M, E)) {
+        S = fr_tile_splits(N, K, E);
+        if (S == 1) return 0;
+    } else {
+        return 0; // the vector kernel finishes the job itself
     }
     return (size_t)S * (size_t)M * (size_t)N * sizeof(float);
 }
@@ -495,8 +647,7 @@ extern "C" int xma_rocm_scatter2scatter_few_rows(const void *X, int64_t ldx, con
                 "scatter2scatter_few_rows: scaled activations go with SWIGLU_BWD, 16-byte aligned rows");
     XMA_REQUIRE(!bias || (al16(bias) && bias_expert_stride % 8 == 0 && bias_expert_stride >= 0), XMA_ROCM_EINVAL,
                 "scatter2scatter_few_rows: bias (E, N) must be 16-byte aligned with an expert stride that is a multiple of 8");
-    // W as (N, K) with the STORE or SWIGLU epilogue finishes in one kernel and needs no workspace
-    const size_t need = (w_is_kn || epilogue == XMA_ROCM_EPI_SWIGLU_BWD) ? xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, w_is_kn) : 0;
+    const size_t need = xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, E, w_is_kn, epilogue);
     XMA_REQUIRE(need == 0 || (workspace && workspace_bytes >= need && al16(workspace)), XMA_ROCM_EWORKSPACE,
                 "scatter2scatter_few_rows: workspace of %zu bytes, %zu needed (16-byte aligned)", workspace ? workspace_bytes : (size_t)0, need);
     FwdArgs a;

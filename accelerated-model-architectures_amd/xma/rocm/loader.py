@@ -59,7 +59,7 @@ SIGNATURES = {
         _int,
         [_p, _i64, _int, _i32, _p, _p, _i64, _int, _i32, _p, _p, _p, _i64, _i64, _i32, _i32, _i32, _int, _p],
     ),
-    "xma_rocm_scatter2scatter_few_rows_workspace_bytes": (_sz, [_i64, _i32, _i32, _int]),
+    "xma_rocm_scatter2scatter_few_rows_workspace_bytes": (_sz, [_i64, _i32, _i32, _i32, _int, _int]),
     "xma_rocm_scatter2scatter_few_rows": (
         _int,
         [_p, _i64, _p, _i64, _i64, _int, _p, _p, _p, _i64, _p, _i64, _p, _i64, _p, _p, _i64, _i64, _i32, _i32, _i32, _i32,

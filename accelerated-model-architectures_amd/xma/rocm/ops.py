@@ -87,8 +87,10 @@ CONTINUOUS_COUNT_SET_MAX_BINS = 8192
 # are the measured cross-overs (8 experts, H = 2048, I = 8192): an expert's rows are walked 4 at a time by the x @ W^T
 # kernel and 8 at a time by the dy @ W kernel, each pass streaming the weights again; the weight gradient grows slowly
 # with the rows.
-FEW_ROWS_MAX = 256  # beyond that the per-row work of these kernels shows where the experts are small (128 experts of 0.4 MB)
-FEW_ROWS_PER_EXPERT = {"x @ W^T": 4, "dy @ W": 8, "dW": 16}
+FEW_ROWS_MAX = 256  # beyond that the per-row work of the vector kernels shows where the experts are small (128 experts of 0.4 MB)
+FEW_ROWS_PER_EXPERT = {"x @ W^T": 32, "dy @ W": 8, "dW": 16}
+FEW_ROWS_MAX_MFMA = 512  # x @ W^T beyond 4 rows per expert or 256 rows takes a small MFMA tile (32 rows x 128 columns); 1024
+# rows over 128 experts of 0.4 MB measured slower than the 256 x 256 tiles (0.205 against 0.180 ms per step), 512 faster
 FEW_ROWS_MAX_WORKSPACE = 256 << 20  # bytes of fp32 partial sums a forward-type launch may ask for
 
 
@@ -168,21 +170,21 @@ FEW_ROWS_NN_MAX_K = 65536  # limit of the few-token entry point for W as (K, N)
 
 def _few_rows(M: int, E: int, dtype: torch.dtype, form: str) -> bool:
     """whether a grouped GEMM of M rows over E experts takes an entry point written for the few-token regime"""
-    return 0 < M <= min(FEW_ROWS_MAX, FEW_ROWS_PER_EXPERT[form] * E) and dtype in (torch.bfloat16, torch.float16)
+    cap = FEW_ROWS_MAX_MFMA if form == "x @ W^T" and FEW_ROWS_MAX > 0 else FEW_ROWS_MAX
+    return 0 < M <= min(cap, FEW_ROWS_PER_EXPERT[form] * E) and dtype in (torch.bfloat16, torch.float16)
 
 
-def _few_rows_fwd(lib, M: int, N: int, K: int, E: int, w_is_kn: int, dtype: torch.dtype) -> bool:
+def _few_rows_fwd(lib, M: int, N: int, K: int, E: int, w_is_kn: int, dtype: torch.dtype, epilogue: int) -> bool:
     """the same for a forward-type GEMM, whose few-token entry point has limits of its own"""
     if not _few_rows(M, E, dtype, "dy @ W" if w_is_kn else "x @ W^T") or (w_is_kn and K > FEW_ROWS_NN_MAX_K):
         return False
-    return lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, w_is_kn) <= FEW_ROWS_MAX_WORKSPACE
+    return lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, E, w_is_kn, epilogue) <= FEW_ROWS_MAX_WORKSPACE
 
 
 def _scatter2scatter_few_rows(lib, X, W, w_is_kn, w_es, ldw, idx, offs, out, aux, aux2, scale, bias, fan_out, x_grouped,
                               y_grouped, epilogue, M, N, K):
-    # W as (N, K) with the STORE or SWIGLU epilogue finishes in one kernel; everything else sums through a workspace
-    needs_ws = bool(w_is_kn) or epilogue == EPI_SWIGLU_BWD
-    ws_bytes = lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, w_is_kn) if needs_ws else 0
+    # whatever does not finish in one kernel sums through a workspace (0 bytes: none needed)
+    ws_bytes = lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, W.size(0), w_is_kn, epilogue)
     workspace = torch.empty(ws_bytes // 4, dtype=torch.float32, device=X.device) if ws_bytes else None
     check(
         lib.xma_rocm_scatter2scatter_few_rows(
@@ -208,7 +210,7 @@ def _scatter2scatter(X, W, idx, offs, out, aux, scale, fan_out, x_grouped, y_gro
     if scale is not None:
         assert scale.dtype == X.dtype and scale.is_contiguous()
     lib = get_library()
-    if _few_rows_fwd(lib, M, N, K, W.size(0), w_is_kn, X.dtype):
+    if _few_rows_fwd(lib, M, N, K, W.size(0), w_is_kn, X.dtype, epilogue):
         _scatter2scatter_few_rows(lib, X, W, w_is_kn, w_es, ldw, idx, offs, out, aux, None, scale, bias, fan_out, x_grouped,
                                   y_grouped, epilogue, M, N, K)
         return
@@ -313,7 +315,7 @@ def down_projection_dx_swiglu_scaled_act_rocm(
     w_is_kn, w_es, ldw = _weight_layout(W)
     assert w_is_kn == 1, "W should be the down-projection parameter as stored, (E, H, I) with I contiguous"
     lib = get_library()
-    if _few_rows_fwd(lib, M, N, K, E, 1, dY.dtype):
+    if _few_rows_fwd(lib, M, N, K, E, 1, dY.dtype, EPI_SWIGLU_BWD):
         _scatter2scatter_few_rows(lib, dY, W, 1, w_es, ldw, sorted_scattered_idxs, expert_offsets, dz, z, scaled_act,
                                   row_scale, None, FAN_OUT, False, True, EPI_SWIGLU_BWD, M, N, K)
         return

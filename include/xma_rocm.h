@@ -198,18 +198,20 @@ XMA_API int xma_rocm_down_projection_dx_swiglu(const void *dY, int64_t lddy, con
 /*
  * xma_rocm_scatter2scatter_bias / xma_rocm_down_projection_dx_swiglu for the few-token regime: the same arguments
  * (aux2 = the scaled activations of the latter, or NULL), the same results up to the order of the fp32 sums, bf16 / fp16
- * only.  With a handful of rows per expert the product is a stream over the weights: rows of W[e] as (N, K) are read by a
- * wave with its lanes along K, rows of W[e] as (K, N) by threads that own 8 columns each, with vector FMAs on fp32
- * sums.  For W as (K, N), and for SWIGLU_BWD, the sums go through the workspace (required then:
- * xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, w_is_kn) bytes) to a small kernel that applies the bias and
- * the epilogue with the arithmetic of the MFMA kernels; W as (N, K) with STORE or SWIGLU finishes in one kernel and takes
- * no workspace (NULL, 0).
- * Limits: M and E at most 65535, K at most 65536 for W as (K, N).  Correct for any M, but the
- * time grows with (rows per expert) x |W|: meant for launches of a few rows per expert (the torch ops of this package
- * take it up to 4 on average for W as (N, K) and 8 for W as (K, N)).  No counterpart in the reference
- * (its kernel is the same for every size).
+ * only.  With a handful of rows per expert the product is a stream over the weights.  W[e] as (N, K): up to 4 rows per
+ * expert on average (and 256 in all) a wave reads two rows of W with its lanes along K and vector FMAs do the rest;
+ * beyond that a small MFMA tile (32 rows of the expert x 128 rows of W, four workgroups per compute unit) takes over,
+ * cut along K where N alone gives too few workgroups.  W[e] as (K, N): threads own 8 columns each and walk a K range.
+ * Whatever does not finish in one kernel sums through the workspace (xma_rocm_scatter2scatter_few_rows_workspace_bytes
+ * bytes for the same M, N, K, num_experts, w_is_kn and epilogue; 0 = none needed, pass NULL) to a small kernel that
+ * applies the bias and the epilogue with the arithmetic of the MFMA kernels.  Limits: M and E at most 65535, K at most
+ * 65536 for W as (K, N).  Correct for any M, but an expert's rows are walked 4 (vector kernel), 8 (W as (K, N)) or 32 (small
+ * tile) at a time, each pass streaming its weights again: meant for launches of a few rows per expert (the torch ops of
+ * this package take it up to 32 on average for W as (N, K) and 8 for W as (K, N)).  No counterpart in the reference (its
+ * kernel is the same for every size).
  */
-XMA_API size_t xma_rocm_scatter2scatter_few_rows_workspace_bytes(int64_t M, int32_t N, int32_t K, int w_is_kn);
+XMA_API size_t xma_rocm_scatter2scatter_few_rows_workspace_bytes(int64_t M, int32_t N, int32_t K, int32_t num_experts,
+                                                         int w_is_kn, int epilogue);
 XMA_API int xma_rocm_scatter2scatter_few_rows(const void *X, int64_t ldx, const void *W, int64_t w_expert_stride, int64_t ldw,
                                       int w_is_kn, const int64_t *sorted_scattered_idxs,
                                       const int64_t *expert_offsets, void *out, int64_t ldo, void *aux, int64_t ldaux,
