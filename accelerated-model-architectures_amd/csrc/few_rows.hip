@@ -155,8 +155,8 @@ namespace {
 //       the X values of the range sit in LDS as floats.  S = K / range.
 // ------------------------------------------------------------------------------------------------
 constexpr int FR_NT_ROWS = 32;  // rows of W per workgroup (8 per wave, two at a time); 8 when the rows are short
-constexpr int FR_NT_VALU_ROWS_PER_EXPERT = 4; // on average; beyond that x @ W^T takes the small MFMA tile,
-constexpr int FR_NT_VALU_ROWS = 256;            // and beyond this many rows in all (the vector kernel's work per row)
+constexpr int FR_NT_VALU_ROWS_PER_EXPERT = 2; // on average; beyond that x @ W^T takes the small MFMA tile,
+constexpr int FR_NT_VALU_ROWS = 64;             // and beyond this many rows in all (the vector kernels' work per row)
 constexpr int FR_NT_PIECE = 2048; // elements of K whose X values are staged in LDS at a time (4 rows: 16 KB)
 constexpr int FR_NT_PAIRS = FR_NT_ROWS / 8; // pairs of rows of W per wave
 
@@ -418,24 +418,31 @@ __global__ __launch_bounds__(FR_THREADS) void fr_epilogue_kernel(const FwdArgs a
 }
 
 // ------------------------------------------------------------------------------------------------
-// x @ W^T for 5 to 32 rows per expert: too many for vector FMAs (one pass over the weights per 4 rows), too few for the
+// 5 to 32 rows per expert: too many for vector FMAs (one pass over the weights per 4 or 8 rows), too few for the
 // 256 x 256 tiles (one 32 KB stage of weights in flight per compute unit).  A small MFMA tile instead: 32 rows of the
-// expert x 128 rows of W[e], K in steps of 64, operands through registers into two LDS stages of 20 KB, so that four
+// expert x 128 output columns, K in steps of 64, operands through registers into two LDS stages of 20 KB, so that four
 // workgroups share a compute unit and keep 80 KB of loads in flight.  One v_mfma_f32_32x32x16 block per wave; lane l holds
-// 16 sums of row l % 32 in quads of 4 consecutive columns, so bias, row scale and the STORE / SWIGLU epilogue are
-// lane-local, with the arithmetic of tile_epilogue in grouped_gemm.hip.  An expert's rows are taken 32 at a time.
+// 16 sums of row l % 32 in quads of 4 consecutive columns, so bias, row scale and the epilogues are lane-local, with the
+// arithmetic of tile_epilogue in grouped_gemm.hip.  An expert's rows are taken 32 at a time.
+//   WT = 0, W[e] as (N, K): the W tile is [128 n][64 k], read back with ds_read_b128 like the X tile.
+//   WT = 1, W[e] as (K, N): the W tile is [64 k][128 n] as it lies in memory; ds_read_b64_tr_b16 hands a lane 4
+//       consecutive k of one column (groups of 16 lanes: lane p addresses 4 columns of k-row p / 4 and receives column p).
 // ------------------------------------------------------------------------------------------------
 constexpr int ST_M = 32, ST_N = 128, ST_K = 64;
 constexpr int ST_W_BYTES = ST_N * ST_K * 2, ST_X_BYTES = ST_M * ST_K * 2, ST_STAGE = ST_W_BYTES + ST_X_BYTES;
 
 // 16-byte slot of (row, chunk) in a tile of 128-byte rows: chunk ^ (row & 7) keeps 8 consecutive rows off each other's banks
 __device__ __forceinline__ int st_slot(int row, int chunk) { return row * 128 + ((chunk ^ (row & 7)) << 4); }
+// the same for the [64 k][128 n] tile of 256-byte rows: 16-byte chunk c of k-row kr sits at c ^ ((kr & 3) << 2)
+__device__ __forceinline__ int st_slot_kn(int kr, int chunk) { return kr * 256 + ((chunk ^ ((kr & 3) << 2)) << 4); }
 
 // EPI = -1: the launch is cut along K (blockIdx.z takes `steps_per` steps) because N alone gives too few workgroups; the
 // fp32 sums go to part[blockIdx.z][M][N] and fr_epilogue_kernel finishes.
-template <typename T, int EPI>
-__global__ __launch_bounds__(FR_THREADS) void fr_nt_tile_kernel(const FwdArgs a, float *__restrict__ part, int steps_per) {
+template <typename T, int WT, int EPI>
+__global__ __launch_bounds__(FR_THREADS) void fr_tile_kernel(const FwdArgs a, float *__restrict__ part, int steps_per) {
     __shared__ __attribute__((aligned(16))) unsigned char s_t[2 * ST_STAGE];
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) v4s *lds_v4s;
     const int e = blockIdx.y;
     const int64_t lo = e ? a.offs[e - 1] : 0, hi = a.offs[e];
     if (lo >= hi) return; // uniform
@@ -444,14 +451,30 @@ __global__ __launch_bounds__(FR_THREADS) void fr_nt_tile_kernel(const FwdArgs a,
     const int steps_all = (a.K + ST_K - 1) / ST_K;
     const int s_begin = (EPI < 0) ? blockIdx.z * steps_per : 0;
     const int s_end = (EPI < 0 && s_begin + steps_per < steps_all) ? s_begin + steps_per : steps_all;
-    // loader: thread = (row tid / 8 (+ 32 i), chunk tid % 8)
+    // X loader: thread = (row tid / 8, chunk tid % 8); W loader, WT = 0: the same with rows + 32 i; WT = 1: (k-row
+    // tid / 16 + 16 i, 16-byte chunk tid % 16 of the 128 columns)
     const int ld_row = tid >> 3, ld_chunk = tid & 7;
+    const int kn_row = tid >> 4, kn_chunk = tid & 15;
+    const bool kn_ok = n0 + 8 * kn_chunk < a.N; // N % 8 == 0: a chunk is inside or outside
     const uint16_t *w_src[4];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-        int n = n0 + ld_row + 32 * i;
-        if (n >= a.N) n = a.N - 1; // clamped: computed, never stored
-        w_src[i] = a.W + (int64_t)e * a.w_es + (int64_t)n * a.ldw + 8 * ld_chunk;
+        if constexpr (WT == 0) {
+            int n = n0 + ld_row + 32 * i;
+            if (n >= a.N) n = a.N - 1; // clamped: computed, never stored
+            w_src[i] = a.W + (int64_t)e * a.w_es + (int64_t)n * a.ldw + 8 * ld_chunk;
+        } else {
+            w_src[i] = a.W + (int64_t)e * a.w_es + (int64_t)(kn_row + 16 * i) * a.ldw + n0 + 8 * kn_chunk;
+        }
+    }
+    // this lane's fragment of the W tile (byte offset inside a stage, k slice 0)
+    int w_frag;
+    if constexpr (WT == 0) {
+        w_frag = 0; // st_slot depends on kk: computed in the loop
+    } else {
+        const int p = lane & 15, G = lane >> 4;
+        const int m = wave * 32 + ((G & 1) << 4) + ((p & 3) << 2), kr = ((G >> 1) << 3) + (p >> 2);
+        w_frag = kr * 256 + ((((m >> 3) ^ ((kr & 3) << 2))) << 4) + ((m & 7) << 1);
     }
     for (int64_t r0 = lo; r0 < hi; r0 += ST_M) {
         int64_t xr = r0 + ld_row;
@@ -459,15 +482,28 @@ __global__ __launch_bounds__(FR_THREADS) void fr_nt_tile_kernel(const FwdArgs a,
         const uint16_t *x_src = a.X + fr_src_row(a, xr) * a.ldx + 8 * ld_chunk;
         u32x4 wv[4], xv;
         auto fetch = [&](int s) {
-            const bool ok = s * ST_K + 8 * ld_chunk < a.K; // chunks past K are zeros
+            const u32x4 zero = {0u, 0u, 0u, 0u};
+            const bool x_ok = s * ST_K + 8 * ld_chunk < a.K; // chunks past K are zeros
+            xv = x_ok ? *(const u32x4 *)(x_src + s * ST_K) : zero;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) wv[i] = ok ? __builtin_nontemporal_load((const u32x4 *)(w_src[i] + s * ST_K)) : u32x4{0u, 0u, 0u, 0u};
-            xv = ok ? *(const u32x4 *)(x_src + s * ST_K) : u32x4{0u, 0u, 0u, 0u};
+            for (int i = 0; i < 4; ++i) {
+                if constexpr (WT == 0) {
+                    wv[i] = x_ok ? __builtin_nontemporal_load((const u32x4 *)(w_src[i] + s * ST_K)) : zero;
+                } else {
+                    const bool ok = kn_ok && s * ST_K + kn_row + 16 * i < a.K;
+                    wv[i] = ok ? __builtin_nontemporal_load((const u32x4 *)(w_src[i] + (int64_t)s * ST_K * a.ldw)) : zero;
+                }
+            }
         };
         auto stash = [&](int stage) {
             unsigned char *base = s_t + stage * ST_STAGE;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) *(u32x4 *)(base + st_slot(ld_row + 32 * i, ld_chunk)) = wv[i];
+            for (int i = 0; i < 4; ++i) {
+                if constexpr (WT == 0)
+                    *(u32x4 *)(base + st_slot(ld_row + 32 * i, ld_chunk)) = wv[i];
+                else
+                    *(u32x4 *)(base + st_slot_kn(kn_row + 16 * i, kn_chunk)) = wv[i];
+            }
             *(u32x4 *)(base + ST_W_BYTES + st_slot(ld_row, ld_chunk)) = xv;
         };
         f32x16 acc;
@@ -479,10 +515,18 @@ __global__ __launch_bounds__(FR_THREADS) void fr_nt_tile_kernel(const FwdArgs a,
         __syncthreads();
         for (int s = s_begin; s < s_end; ++s) {
             if (s + 1 < s_end) fetch(s + 1); // in flight while this step computes
-            const unsigned char *base = s_t + (s & 1) * ST_STAGE;
+            unsigned char *base = s_t + (s & 1) * ST_STAGE;
 #pragma unroll
             for (int kk = 0; kk < 4; ++kk) {
-                const u32x4 wa = *(const u32x4 *)(base + st_slot(wave * 32 + l32, 2 * kk + half));
+                u32x4 wa;
+                if constexpr (WT == 0) {
+                    wa = *(const u32x4 *)(base + st_slot(wave * 32 + l32, 2 * kk + half));
+                } else { // k-rows 16 kk + ..: the swizzle depends on kr & 3 only, so kk adds 16 rows = 4096 bytes
+                    const v4s k03 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(base + w_frag + kk * 4096));
+                    const v4s k47 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(base + w_frag + kk * 4096 + 1024));
+                    const u32x2 a01 = __builtin_bit_cast(u32x2, k03), a23 = __builtin_bit_cast(u32x2, k47);
+                    wa = u32x4{a01[0], a01[1], a23[0], a23[1]};
+                }
                 const u32x4 xb = *(const u32x4 *)(base + ST_W_BYTES + st_slot(l32, 2 * kk + half));
                 acc = Elem<T>::mfma(wa, xb, acc);
             }
@@ -507,25 +551,45 @@ __global__ __launch_bounds__(FR_THREADS) void fr_nt_tile_kernel(const FwdArgs a,
         for (int g = 0; g < 4; ++g) {
             const int n = n0 + wave * 32 + 8 * g + 4 * half; // acc[4 g + q] is column n + q of row r
             if (n >= a.N) continue;
-            float v[4];
+            if constexpr (EPI == XMA_ROCM_EPI_SWIGLU_BWD) {
+                // d h of 4 columns -> (d gate, d up) of their 4 pairs; rows are grouped on both sides
+                const u32x4 z = *(const u32x4 *)(a.aux + r * a.ldaux + 2 * n);
+                u32x4 o;
+                float hv[4];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                v[q] = acc[4 * g + q];
-                if (a.bias) v[q] += fr_scalar<T>(a.bias, (int64_t)e * a.bias_es + n + q);
-                v[q] *= sc;
-            }
-            const uint32_t z0 = Elem<T>::pack(v[0], v[1]), z1 = Elem<T>::pack(v[2], v[3]);
-            if (a.out) *(u32x2 *)(a.out + dst * a.ldo + n) = u32x2{z0, z1};
-            if constexpr (EPI == XMA_ROCM_EPI_SWIGLU) {
-                const float g0 = Elem<T>::lo(z0), u0 = Elem<T>::hi(z0), g1 = Elem<T>::lo(z1), u1 = Elem<T>::hi(z1);
-                *(uint32_t *)(a.aux + dst * a.ldaux + (n >> 1)) = Elem<T>::pack(u0 * g0 * sigmoidf_fast(g0), u1 * g1 * sigmoidf_fast(g1));
+                for (int q = 0; q < 4; ++q) {
+                    const float dh = acc[4 * g + q] * sc;
+                    const float gg = Elem<T>::lo(z[q]), uu = Elem<T>::hi(z[q]);
+                    const float sg = sigmoidf_fast(gg), silu = gg * sg;
+                    o[q] = Elem<T>::pack(dh * uu * (sg + silu * (1.f - sg)), dh * silu);
+                    hv[q] = uu * silu * sc;
+                }
+                *(u32x4 *)(a.out + r * a.ldo + 2 * n) = o;
+                if (a.aux2) *(u32x2 *)(a.aux2 + r * a.ldaux2 + n) = u32x2{Elem<T>::pack(hv[0], hv[1]), Elem<T>::pack(hv[2], hv[3])};
+            } else {
+                float v[4];
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    v[q] = acc[4 * g + q];
+                    if (a.bias) v[q] += fr_scalar<T>(a.bias, (int64_t)e * a.bias_es + n + q);
+                    v[q] *= sc;
+                }
+                const uint32_t z0 = Elem<T>::pack(v[0], v[1]), z1 = Elem<T>::pack(v[2], v[3]);
+                if (a.out) *(u32x2 *)(a.out + dst * a.ldo + n) = u32x2{z0, z1};
+                if constexpr (EPI == XMA_ROCM_EPI_SWIGLU) {
+                    const float g0 = Elem<T>::lo(z0), u0 = Elem<T>::hi(z0), g1 = Elem<T>::lo(z1), u1 = Elem<T>::hi(z1);
+                    *(uint32_t *)(a.aux + dst * a.ldaux + (n >> 1)) = Elem<T>::pack(u0 * g0 * sigmoidf_fast(g0), u1 * g1 * sigmoidf_fast(g1));
+                }
             }
         }
     }
 }
 
-// x @ W^T: more than a pass or two of the vector kernel per expert -> the small MFMA tile
-inline bool fr_nt_takes_tile(int64_t M, int E) { return M > (int64_t)FR_NT_VALU_ROWS_PER_EXPERT * E || M > FR_NT_VALU_ROWS; }
+// more than a pass or two of the vector kernels per expert -> the small MFMA tile
+constexpr int FR_NN_VALU_ROWS_PER_EXPERT = 2;
+inline bool fr_takes_tile(int64_t M, int E, int w_is_kn) {
+    return M > (int64_t)(w_is_kn ? FR_NN_VALU_ROWS_PER_EXPERT : FR_NT_VALU_ROWS_PER_EXPERT) * E || M > FR_NT_VALU_ROWS;
+}
 
 // K ranges of the small MFMA tile: enough workgroups for four per compute unit (twice as many measured slower: the
 // partial sums and their kernel cost more than the extra parallelism brings), ranges of at least 8 steps
@@ -537,59 +601,53 @@ inline int fr_tile_splits(int N, int K, int E) {
     return S < 1 ? 1 : S;
 }
 
-template <typename T> int fr_launch(const FwdArgs &a, int w_is_kn, int epilogue, float *part, hipStream_t st) {
-    int S = 1, rc;
+template <typename T, int EPI> int fr_launch_epilogue(const FwdArgs &a, const float *part, int S, hipStream_t st) {
+    const dim3 egrid((a.N / 2 + FR_THREADS - 1) / FR_THREADS, (unsigned)a.M);
+    fr_epilogue_kernel<T, EPI><<<egrid, FR_THREADS, 0, st>>>(a, part, S);
+    return xma_check_launch("fr_epilogue_kernel");
+}
+
+template <typename T, int WT, int EPI> int fr_launch_tile(const FwdArgs &a, float *part, hipStream_t st) {
+    const int S = fr_tile_splits(a.N, a.K, a.E);
+    const int steps_all = (a.K + ST_K - 1) / ST_K, steps_per = (steps_all + S - 1) / S;
+    const dim3 grid((a.N + ST_N - 1) / ST_N, a.E, S);
+    if (S == 1) {
+        fr_tile_kernel<T, WT, EPI><<<grid, FR_THREADS, 0, st>>>(a, nullptr, steps_all);
+        return xma_check_launch("fr_tile_kernel");
+    }
+    fr_tile_kernel<T, WT, -1><<<grid, FR_THREADS, 0, st>>>(a, part, steps_per);
+    int rc = xma_check_launch("fr_tile_kernel");
+    if (rc) return rc;
+    return fr_launch_epilogue<T, EPI>(a, part, (steps_all + steps_per - 1) / steps_per, st);
+}
+
+template <typename T, int EPI> int fr_launch_epi(const FwdArgs &a, int w_is_kn, float *part, hipStream_t st) {
+    int rc;
+    if (fr_takes_tile(a.M, a.E, w_is_kn)) return w_is_kn ? fr_launch_tile<T, 1, EPI>(a, part, st) : fr_launch_tile<T, 0, EPI>(a, part, st);
     if (w_is_kn) {
-        const int kc = fr_nn_range(a.K);
-        S = (a.K + kc - 1) / kc;
+        const int kc = fr_nn_range(a.K), S = (a.K + kc - 1) / kc;
         const dim3 grid((a.N / 8 + FR_THREADS - 1) / FR_THREADS, S, a.E);
         fr_nn_kernel<T><<<grid, FR_THREADS, (size_t)8 * kc * sizeof(float), st>>>(a, part, kc);
         if ((rc = xma_check_launch("fr_nn_kernel"))) return rc;
-    } else {
-        if (epilogue != XMA_ROCM_EPI_SWIGLU_BWD && fr_nt_takes_tile(a.M, a.E)) {
-            // more than a pass or two of the vector kernel per expert: the small MFMA tile
-            const int S = fr_tile_splits(a.N, a.K, a.E);
-            const int steps_all = (a.K + ST_K - 1) / ST_K, steps_per = (steps_all + S - 1) / S;
-            const dim3 grid((a.N + ST_N - 1) / ST_N, a.E, S);
-            if (S == 1) {
-                if (epilogue == XMA_ROCM_EPI_STORE)
-                    fr_nt_tile_kernel<T, XMA_ROCM_EPI_STORE><<<grid, FR_THREADS, 0, st>>>(a, nullptr, steps_all);
-                else
-                    fr_nt_tile_kernel<T, XMA_ROCM_EPI_SWIGLU><<<grid, FR_THREADS, 0, st>>>(a, nullptr, steps_all);
-                return xma_check_launch("fr_nt_tile_kernel");
-            }
-            fr_nt_tile_kernel<T, -1><<<grid, FR_THREADS, 0, st>>>(a, part, steps_per);
-            if ((rc = xma_check_launch("fr_nt_tile_kernel"))) return rc;
-            const dim3 egrid((a.N / 2 + FR_THREADS - 1) / FR_THREADS, (unsigned)a.M);
-            const int parts = (steps_all + steps_per - 1) / steps_per;
-            if (epilogue == XMA_ROCM_EPI_STORE)
-                fr_epilogue_kernel<T, XMA_ROCM_EPI_STORE><<<egrid, FR_THREADS, 0, st>>>(a, part, parts);
-            else
-                fr_epilogue_kernel<T, XMA_ROCM_EPI_SWIGLU><<<egrid, FR_THREADS, 0, st>>>(a, part, parts);
-            return xma_check_launch("fr_epilogue_kernel");
-        }
-        // one pair of rows per wave instead of four where the rows are short or the launch would have few workgroups
-        const int rows_per_wg = (a.K >= 2048 && (int64_t)(a.N / FR_NT_ROWS) * a.E >= 2048) ? FR_NT_ROWS : 8;
-        const dim3 grid((a.N + rows_per_wg - 1) / rows_per_wg, a.E);
-        if (epilogue == XMA_ROCM_EPI_STORE) {
-            fr_nt_kernel<T, XMA_ROCM_EPI_STORE><<<grid, FR_THREADS, 0, st>>>(a, part, rows_per_wg);
-            return xma_check_launch("fr_nt_kernel");
-        }
-        if (epilogue == XMA_ROCM_EPI_SWIGLU) {
-            fr_nt_kernel<T, XMA_ROCM_EPI_SWIGLU><<<grid, FR_THREADS, 0, st>>>(a, part, rows_per_wg);
-            return xma_check_launch("fr_nt_kernel");
-        }
+        return fr_launch_epilogue<T, EPI>(a, part, S, st);
+    }
+    // one pair of rows per wave instead of four where the rows are short or the launch would have few workgroups
+    const int rows_per_wg = (a.K >= 2048 && (int64_t)(a.N / FR_NT_ROWS) * a.E >= 2048) ? FR_NT_ROWS : 8;
+    const dim3 grid((a.N + rows_per_wg - 1) / rows_per_wg, a.E);
+    if constexpr (EPI == XMA_ROCM_EPI_SWIGLU_BWD) {
         fr_nt_kernel<T, -1><<<grid, FR_THREADS, 0, st>>>(a, part, rows_per_wg);
         if ((rc = xma_check_launch("fr_nt_kernel"))) return rc;
+        return fr_launch_epilogue<T, EPI>(a, part, 1, st);
+    } else {
+        fr_nt_kernel<T, EPI><<<grid, FR_THREADS, 0, st>>>(a, part, rows_per_wg);
+        return xma_check_launch("fr_nt_kernel");
     }
-    const dim3 egrid((a.N / 2 + FR_THREADS - 1) / FR_THREADS, (unsigned)a.M);
-    if (epilogue == XMA_ROCM_EPI_STORE)
-        fr_epilogue_kernel<T, XMA_ROCM_EPI_STORE><<<egrid, FR_THREADS, 0, st>>>(a, part, S);
-    else if (epilogue == XMA_ROCM_EPI_SWIGLU)
-        fr_epilogue_kernel<T, XMA_ROCM_EPI_SWIGLU><<<egrid, FR_THREADS, 0, st>>>(a, part, S);
-    else
-        fr_epilogue_kernel<T, XMA_ROCM_EPI_SWIGLU_BWD><<<egrid, FR_THREADS, 0, st>>>(a, part, S);
-    return xma_check_launch("fr_epilogue_kernel");
+}
+
+template <typename T> int fr_launch(const FwdArgs &a, int w_is_kn, int epilogue, float *part, hipStream_t st) {
+    if (epilogue == XMA_ROCM_EPI_STORE) return fr_launch_epi<T, XMA_ROCM_EPI_STORE>(a, w_is_kn, part, st);
+    if (epilogue == XMA_ROCM_EPI_SWIGLU) return fr_launch_epi<T, XMA_ROCM_EPI_SWIGLU>(a, w_is_kn, part, st);
+    return fr_launch_epi<T, XMA_ROCM_EPI_SWIGLU_BWD>(a, w_is_kn, part, st);
 }
 
 } // namespace
@@ -598,14 +656,14 @@ extern "C" size_t xma_rocm_scatter2scatter_few_rows_workspace_bytes(int64_t M, i
                                                                     int epilogue) {
     if (M <= 0 || N <= 0 || K <= 0 || E <= 0) return 0;
     int S;
-    if (w_is_kn) { // partial sums of the K ranges
+    if (fr_takes_tile(M, E, w_is_kn)) { // the small MFMA tile, cut along K or not
+        S = fr_tile_splits(N, K, E);
+        if (S == 1) return 0;
+    } else if (w_is_kn) { // partial sums of the K ranges
         const int kc = fr_nn_range(K);
         S = (K + kc - 1) / kc;
     } else if (epilogue == XMA_ROCM_EPI_SWIGLU_BWD) {
         S = 1; // the vector kernel's sums go to the epilogue kernel
-    } else if (fr_nt_takes_tile(M, E)) {
-        S = fr_tile_splits(N, K, E);
-        if (S == 1) return 0;
     } else {
         return 0; // the vector kernel finishes the job itself
     }

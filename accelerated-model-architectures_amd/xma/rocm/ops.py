@@ -83,14 +83,14 @@ def continuous_count_rocm(x: torch.Tensor, y: torch.Tensor, workspace: torch.Ten
 
 CONTINUOUS_COUNT_SET_MAX_BINS = 8192
 # The grouped GEMMs take the entry points written for the few-token regime, which stream the weights instead of tiling
-# them for the matrix pipes, up to FEW_ROWS_PER_EXPERT rows per expert on average and FEW_ROWS_MAX rows in all.  The limits
-# are the measured cross-overs (8 experts, H = 2048, I = 8192): an expert's rows are walked 4 at a time by the x @ W^T
-# kernel and 8 at a time by the dy @ W kernel, each pass streaming the weights again; the weight gradient grows slowly
-# with the rows.
-FEW_ROWS_MAX = 256  # beyond that the per-row work of the vector kernels shows where the experts are small (128 experts of 0.4 MB)
-FEW_ROWS_PER_EXPERT = {"x @ W^T": 32, "dy @ W": 8, "dW": 16}
-FEW_ROWS_MAX_MFMA = 512  # x @ W^T beyond 4 rows per expert or 256 rows takes a small MFMA tile (32 rows x 128 columns); 1024
-# rows over 128 experts of 0.4 MB measured slower than the 256 x 256 tiles (0.205 against 0.180 ms per step), 512 faster
+# them 256 x 256 for the matrix pipes, up to FEW_ROWS_PER_EXPERT rows per expert on average.  The limits are measured
+# cross-overs (8 experts of H = 2048, I = 8192; 64 of H = 2048, I = 1408; 128 of H = 576, I = 256): the forward-type GEMMs
+# walk an expert's rows 32 at a time (small MFMA tile; vector FMAs up to 2 rows per expert and 64 rows in all, the library
+# decides), each pass streaming the weights again, so they lead while most experts need one pass; the weight gradient is
+# vector FMAs throughout and grows with the rows.
+FEW_ROWS_PER_EXPERT = {"x @ W^T": 24, "dy @ W": 24, "dW": 16}
+FEW_ROWS_MAX = 256  # weight gradient: beyond that its per-row work shows where the experts are small
+FEW_ROWS_MAX_MFMA = 4096  # forward-type GEMMs
 FEW_ROWS_MAX_WORKSPACE = 256 << 20  # bytes of fp32 partial sums a forward-type launch may ask for
 
 
@@ -170,7 +170,7 @@ FEW_ROWS_NN_MAX_K = 65536  # limit of the few-token entry point for W as (K, N)
 
 def _few_rows(M: int, E: int, dtype: torch.dtype, form: str) -> bool:
     """whether a grouped GEMM of M rows over E experts takes an entry point written for the few-token regime"""
-    cap = FEW_ROWS_MAX_MFMA if form == "x @ W^T" and FEW_ROWS_MAX > 0 else FEW_ROWS_MAX
+    cap = FEW_ROWS_MAX_MFMA if form != "dW" and FEW_ROWS_MAX > 0 else FEW_ROWS_MAX
     return 0 < M <= min(cap, FEW_ROWS_PER_EXPERT[form] * E) and dtype in (torch.bfloat16, torch.float16)
 
 

@@ -77,9 +77,10 @@ def test_argument_errors_are_reported_before_any_launch():
     assert few(None, 64, None, 64 * 64, 64, 0, p, p, p, 64, None, 0, None, 0, None, None, 0, 4, 64, 64, 2, 1, 1, 1, 0, 0, None, 0, None) == -1
     assert b"null or misaligned" in lib.xma_rocm_last_error()
     ws = lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes  # (M, N, K, E, w_is_kn, epilogue)
-    assert ws(4, 64, 64, 2, 0, 0) == 0 and ws(4, 64, 64, 2, 0, 1) == 0  # the vector kernel finishes the job itself
+    assert ws(4, 64, 64, 2, 0, 0) == 0 and ws(4, 64, 64, 2, 0, 1) == 0  # the vector kernel finishes the job itself (2 rows per expert)
     assert ws(4, 64, 64, 2, 0, 2) == 4 * 64 * 4  # SwiGLU backward: through the epilogue kernel
     assert ws(4, 64, 16384, 2, 1, 0) == 64 * 4 * 64 * 4  # W as (K, N): 64 ranges of K
+    assert ws(64, 2048, 16384, 8, 1, 0) == 8 * 64 * 2048 * 4 and ws(64, 8192, 2048, 8, 1, 2) == 2 * 64 * 8192 * 4  # small tile
     assert ws(64, 16384, 2048, 8, 0, 1) == 0  # small MFMA tile, enough workgroups from N alone
     assert ws(64, 2048, 8192, 8, 0, 0) == 8 * 64 * 2048 * 4  # small MFMA tile cut into 8 ranges of K
     assert ws(0, 64, 64, 2, 1, 0) == 0
@@ -99,11 +100,11 @@ def test_few_token_dispatch_rule():
     from xma.rocm import ops
 
     bf = torch.bfloat16
-    assert ops._few_rows(14, 8, bf, "x @ W^T") and ops._few_rows(256, 8, bf, "x @ W^T") and not ops._few_rows(257, 8, bf, "x @ W^T")
-    assert ops._few_rows(512, 128, bf, "x @ W^T") and not ops._few_rows(513, 128, bf, "x @ W^T")  # its own cap on the rows
-    assert ops._few_rows(64, 8, bf, "dy @ W") and not ops._few_rows(65, 8, bf, "dy @ W")
+    assert ops._few_rows(14, 8, bf, "x @ W^T") and ops._few_rows(192, 8, bf, "x @ W^T") and not ops._few_rows(193, 8, bf, "x @ W^T")
+    assert ops._few_rows(3072, 128, bf, "dy @ W") and not ops._few_rows(4097, 256, bf, "x @ W^T")  # their cap on the rows
+    assert ops._few_rows(192, 8, bf, "dy @ W") and not ops._few_rows(193, 8, bf, "dy @ W")
     assert ops._few_rows(128, 8, bf, "dW") and not ops._few_rows(129, 8, bf, "dW")
-    assert ops._few_rows(256, 128, bf, "dy @ W") and not ops._few_rows(257, 128, bf, "dW")  # the cap on the rows in all
+    assert ops._few_rows(256, 128, bf, "dW") and not ops._few_rows(257, 128, bf, "dW")  # the weight gradient's cap
     assert not ops._few_rows(0, 8, bf, "dW") and not ops._few_rows(14, 8, torch.float32, "dW")
     assert ops._few_rows(14, 8, torch.float16, "dy @ W")
 
