@@ -1,17 +1,15 @@
 // Kernels for the few-token regime: every expert has a handful of rows, so a grouped GEMM is a stream over the weights
 // (or, for the weight gradient, a stream of stores) with next to no arithmetic.  The 256 x 256 MFMA tiles of
 // grouped_gemm.hip are built for arithmetic: with one K step per tile, or one stage of weights in flight per compute unit,
-// they move 3.3-3.8 TB/s.  Here the work is laid out for bandwidth: 16 bytes per lane, many short workgroups per compute
-// unit, vector FMAs on fp32 accumulators.  Correct for any number of rows, but the cost grows with rows x weights: the
-// caller picks these entry points by the total number of rows.
+// they move 3.3-3.8 TB/s.  Here the work is laid out for bandwidth: 16 bytes per lane, 256 contiguous bytes per row and
+// load instruction, many short workgroups per compute unit; vector FMAs for one or two rows per expert, small MFMA tiles
+// beyond.  Correct for any number of rows, but the forward-type kernels stream the weights once per 32 rows of an expert:
+// the caller picks these entry points by the number of rows per expert.
 #include "gemm_common.hpp"
 
 namespace {
 
 constexpr int FR_THREADS = 256;
-constexpr int FR_NB = 8; // output rows (n) per workgroup of the weight gradient
-constexpr int FR_RC = 4; // rows of the expert per step
-constexpr int FR_GROUPS = 8; // sets of FR_NB rows n per workgroup, at most (rows of DW of 32 pieces of 16 bytes or more fill it)
 
 template <typename T> __device__ __forceinline__ float fr_scalar(const uint16_t *p, int64_t i) { return Elem<T>::lo(p[i]); }
 
@@ -20,75 +18,102 @@ template <typename T> __device__ __forceinline__ void fr_unpack(const u32x4 v, f
     for (int q = 0; q < 4; ++q) f[2 * q] = Elem<T>::lo(v[q]), f[2 * q + 1] = Elem<T>::hi(v[q]);
 }
 
-// DW[e][n][k] = sum over the rows r of expert e of DY[dsrc(r)][n] * scale[idx[r]] * X[xsrc(r)][k]: an outer product per
-// row.  Workgroup = (2048 columns k, FR_NB rows n, expert), or several sets of FR_NB rows when a row of DW is shorter than
-// the workgroup; a thread owns 8 consecutive k of every n of its set: it loads its 16 bytes
-// of each X row once, takes the FR_NB values of DY from LDS, and leaves FR_NB stores of 16 bytes.  fp32 sums in row order.
-// Every element of DW is written exactly once, zeros for an expert without rows.
-template <typename T> __global__ __launch_bounds__(FR_THREADS) void dw_few_rows_kernel(const DwArgs a) {
-    __shared__ float s_dy[2][FR_GROUPS][FR_RC][FR_NB];
-    const int e = blockIdx.z, tid = threadIdx.x;
-    // a row of DW shorter than the workgroup: `groups` sets of FR_NB rows n side by side, `cpr` threads each
-    const int cpr = a.K_in >> 3;
-    int groups = (cpr < FR_THREADS) ? FR_THREADS / cpr : 1;
-    if (groups > FR_GROUPS) groups = FR_GROUPS;
-    const int grp = (groups > 1) ? tid / cpr : 0;
-    const int n0 = (blockIdx.y * groups + grp) * FR_NB;
-    const int k0 = (groups > 1) ? (tid - grp * cpr) * 8 : (blockIdx.x * FR_THREADS + tid) * 8;
-    const bool k_ok = k0 < a.K_in && grp < groups;
+// DW[e][n][k] = sum over the rows r of expert e of DY[dsrc(r)][n] * scale[idx[r]] * X[xsrc(r)][k]: MFMAs whose K dimension is
+// the expert's rows, 32 at a time, zeros beyond the last.  With few rows the launch is its stores (a vector-FMA version, a
+// thread owning 8 k of 8 rows n, was as fast up to 8 rows per expert and three times slower at 32).  Workgroup = a 128 x 128 tile of DW[e] (32 KB of stores) for (k block, n block, expert); both operand tiles are [32 rows][128
+// columns] as they lie in memory, and ds_read_b64_tr_b16 hands a lane 4 consecutive rows of one column (st_slot_kn and the
+// fragment offsets of fr_tile_kernel below).  Wave w owns the 32 rows n of block w and all 128 columns k: 4 accumulator blocks,
+// where lane l holds row n = l % 32 and quads of 4 consecutive k.  The tile leaves through LDS as whole 256-byte rows,
+// 16 bytes per lane.  Any number of rows (more passes), every element written exactly once, zeros for an expert without rows.
+constexpr int DT_TILE = 128, DT_ROWS = 32, DT_OPERAND = DT_ROWS * DT_TILE * 2;
+// 16-byte slot of (k-row, chunk) in a tile of 256-byte rows that is read down its columns: chunk c of k-row kr sits at
+// c ^ ((kr & 3) << 2)
+__device__ __forceinline__ int st_slot_kn(int kr, int chunk) { return kr * 256 + ((chunk ^ ((kr & 3) << 2)) << 4); }
+
+template <typename T> __global__ __launch_bounds__(FR_THREADS, 4) void dw_tile_kernel(const DwArgs a) {
+    __shared__ __attribute__((aligned(16))) unsigned char s_t[DT_TILE * DT_TILE * 2]; // the operand tiles (2 x 8 KB), then the output tile
+    typedef short v4s __attribute__((ext_vector_type(4)));
+    typedef __attribute__((address_space(3))) v4s *lds_v4s;
+    const int e = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
+    const int k0 = blockIdx.x * DT_TILE, n0 = blockIdx.y * DT_TILE;
     const int64_t lo = e ? a.offs[e - 1] : 0, hi = a.offs[e];
-    float acc[FR_NB][8];
+    // loader and storer: thread = (row tid / 16 + 16 i, 16-byte chunk tid % 16 of the 128 columns)
+    const int ld_row = tid >> 4, ld_chunk = tid & 15;
+    const bool dy_ok = n0 + 8 * ld_chunk < a.N_out, x_ok = k0 + 8 * ld_chunk < a.K_in; // multiples of 8: a chunk is inside or outside
+    // this lane's fragment of column block `blk` of an operand tile, rows 0-3 of its 8 (the other 4: + 1024, rows + 16: + 4096)
+    const int p = lane & 15, G = lane >> 4, kr = ((G >> 1) << 3) + (p >> 2), m_in = ((G & 1) << 4) + ((p & 3) << 2);
+    auto frag_off = [&](int blk) {
+        const int m = blk * 32 + m_in;
+        return kr * 256 + (((m >> 3) ^ ((kr & 3) << 2)) << 4) + ((m & 7) << 1);
+    };
+    auto frag = [&](const unsigned char *at) {
+        const v4s r03 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)at);
+        const v4s r47 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(at + 1024));
+        const u32x2 a01 = __builtin_bit_cast(u32x2, r03), a23 = __builtin_bit_cast(u32x2, r47);
+        return u32x4{a01[0], a01[1], a23[0], a23[1]};
+    };
+    f32x16 acc[4];
 #pragma unroll
-    for (int j = 0; j < FR_NB; ++j)
+    for (int j = 0; j < 4; ++j)
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[j][i] = 0.f;
-    int buf = 0;
-    for (int64_t r0 = lo; r0 < hi; r0 += FR_RC, buf ^= 1) {
-        if (tid < groups * FR_RC * FR_NB) { // the step's FR_RC x FR_NB values of dY of every group, scaled
-            const int gq = tid / (FR_RC * FR_NB), u = (tid / FR_NB) % FR_RC, j = tid % FR_NB;
-            const int64_t r = r0 + u;
-            const int n = (blockIdx.y * groups + gq) * FR_NB + j;
-            float v = 0.f;
-            if (r < hi && n < a.N_out) {
+        for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
+    for (int64_t r0 = lo; r0 < hi; r0 += DT_ROWS) {
+        u32x4 dyv[2], xv[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int64_t r = r0 + ld_row + 16 * i;
+            dyv[i] = xv[i] = u32x4{0u, 0u, 0u, 0u}; // rows past the expert's last add nothing
+            if (r < hi) {
                 const int64_t s = a.idx ? a.idx[r] : r;
-                const int64_t src = a.dy_grouped ? r : (int64_t)fastdiv((uint32_t)s, a.dy_div);
-                v = fr_scalar<T>(a.DY, src * a.lddy + n);
-                if (a.scale) v *= fr_scalar<T>(a.scale, s);
+                if (dy_ok) {
+                    const int64_t src = a.dy_grouped ? r : (int64_t)fastdiv((uint32_t)s, a.dy_div);
+                    dyv[i] = *(const u32x4 *)(a.DY + src * a.lddy + n0 + 8 * ld_chunk);
+                    if (a.scale) { // the scaled row rounded to the operand type, as a scaled grouped copy of dY would hold it
+                        const float sc = fr_scalar<T>(a.scale, s);
+                        float f[8];
+                        fr_unpack<T>(dyv[i], f);
+#pragma unroll
+                        for (int q = 0; q < 4; ++q) dyv[i][q] = Elem<T>::pack(f[2 * q] * sc, f[2 * q + 1] * sc);
+                    }
+                }
+                if (x_ok) {
+                    const int64_t src = a.x_grouped ? r : (int64_t)fastdiv((uint32_t)s, a.x_div);
+                    xv[i] = *(const u32x4 *)(a.X + src * a.ldx + k0 + 8 * ld_chunk);
+                }
             }
-            s_dy[buf][gq][u][j] = v;
         }
-        u32x4 x[FR_RC];
+        __syncthreads(); // the pass before no longer reads the tiles
 #pragma unroll
-        for (int u = 0; u < FR_RC; ++u) {
-            const int64_t r = r0 + u;
-            x[u] = u32x4{0u, 0u, 0u, 0u};
-            if (r < hi && k_ok) {
-                const int64_t src = a.x_grouped ? r : (int64_t)fastdiv((uint32_t)a.idx[r], a.x_div);
-                x[u] = *(const u32x4 *)(a.X + src * a.ldx + k0);
-            }
+        for (int i = 0; i < 2; ++i) {
+            *(u32x4 *)(s_t + st_slot_kn(ld_row + 16 * i, ld_chunk)) = dyv[i];
+            *(u32x4 *)(s_t + DT_OPERAND + st_slot_kn(ld_row + 16 * i, ld_chunk)) = xv[i];
         }
-        __syncthreads(); // two buffers: the next step's values are written while a slow wave still reads this step's
+        __syncthreads();
 #pragma unroll
-        for (int u = 0; u < FR_RC; ++u) {
-            float xf[8];
-            fr_unpack<T>(x[u], xf);
+        for (int kk = 0; kk < 2; ++kk) {
+            const u32x4 dy_f = frag(s_t + frag_off(wave) + kk * 4096);
 #pragma unroll
-            for (int j = 0; j < FR_NB; ++j) {
-                const float d = s_dy[buf][grp < groups ? grp : 0][u][j];
-#pragma unroll
-                for (int i = 0; i < 8; ++i) acc[j][i] = __builtin_fmaf(d, xf[i], acc[j][i]);
-            }
+            for (int j = 0; j < 4; ++j) acc[j] = Elem<T>::mfma(frag(s_t + DT_OPERAND + frag_off(j) + kk * 4096), dy_f, acc[j]);
         }
     }
-    if (!k_ok) return;
-    uint16_t *out = a.DW + (int64_t)e * a.dw_es + k0;
+    __syncthreads(); // the operand tiles are done with: the output tile takes their place
+    // acc[j][4 g + q] = DW[n0 + 32 wave + l32][k0 + 32 j + 8 g + 4 half + q]; the 16-byte chunk c of row n sits at c ^ (n % 16)
+    const int n_l = wave * 32 + l32;
 #pragma unroll
-    for (int j = 0; j < FR_NB; ++j) {
-        if (n0 + j < a.N_out) {
-            const u32x4 v = {Elem<T>::pack(acc[j][0], acc[j][1]), Elem<T>::pack(acc[j][2], acc[j][3]),
-                             Elem<T>::pack(acc[j][4], acc[j][5]), Elem<T>::pack(acc[j][6], acc[j][7])};
-            __builtin_nontemporal_store(v, (u32x4 *)(out + (int64_t)(n0 + j) * a.lddw));
-        }
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+            *(u32x2 *)(s_t + n_l * 256 + (((4 * j + g) ^ (n_l & 15)) << 4) + 8 * half) =
+                u32x2{Elem<T>::pack(acc[j][4 * g], acc[j][4 * g + 1]), Elem<T>::pack(acc[j][4 * g + 2], acc[j][4 * g + 3])};
+    __syncthreads();
+    if (!x_ok) return;
+    uint16_t *out = a.DW + (int64_t)e * a.dw_es + k0 + 8 * ld_chunk;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const int row = ld_row + 16 * i;
+        if (n0 + row < a.N_out)
+            __builtin_nontemporal_store(*(const u32x4 *)(s_t + row * 256 + ((ld_chunk ^ (row & 15)) << 4)),
+                                        (u32x4 *)(out + (int64_t)(n0 + row) * a.lddw));
     }
 }
 
@@ -100,20 +125,18 @@ extern "C" int xma_rocm_group_bwd_W_few_rows(const void *DY, int64_t lddy, int d
                                              const int64_t *expert_offsets, void *DW, int64_t dw_expert_stride, int64_t lddw,
                                              int32_t N_out, int32_t K_in, int32_t E, int dtype, void *stream) {
     XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED, "group_bwd_W_few_rows: dtype %d", dtype);
-    XMA_REQUIRE(N_out >= 1 && K_in >= 8 && E >= 1 && E <= 65535 && dy_fan_out >= 1 && x_fan_out >= 1, XMA_ROCM_EINVAL,
+    XMA_REQUIRE(N_out >= 8 && K_in >= 8 && E >= 1 && E <= 65535 && dy_fan_out >= 1 && x_fan_out >= 1, XMA_ROCM_EINVAL,
                 "group_bwd_W_few_rows: N_out=%d K_in=%d E=%d", N_out, K_in, E);
-    XMA_REQUIRE(K_in % 8 == 0 && ldx % 8 == 0 && lddw % 8 == 0 && dw_expert_stride % 8 == 0, XMA_ROCM_EUNSUPPORTED,
-                "group_bwd_W_few_rows: K_in=%d, ldx, lddw and the expert stride must be multiples of 8", K_in);
-    XMA_REQUIRE(DY && X && DW && expert_offsets && ((uintptr_t)X & 15) == 0 && ((uintptr_t)DW & 15) == 0 &&
-                    ((uintptr_t)DY & 1) == 0,
-                XMA_ROCM_EINVAL, "group_bwd_W_few_rows: null or misaligned operand");
+    XMA_REQUIRE(N_out % 8 == 0 && K_in % 8 == 0 && lddy % 8 == 0 && ldx % 8 == 0 && lddw % 8 == 0 && dw_expert_stride % 8 == 0,
+                XMA_ROCM_EUNSUPPORTED, "group_bwd_W_few_rows: N_out=%d K_in=%d and the leading dimensions must be multiples of 8",
+                N_out, K_in);
+    auto al16 = [](const void *p) { return ((uintptr_t)p & 15) == 0; };
+    XMA_REQUIRE(DY && X && DW && expert_offsets && al16(DY) && al16(X) && al16(DW), XMA_ROCM_EINVAL,
+                "group_bwd_W_few_rows: null or misaligned operand");
     XMA_REQUIRE(sorted_scattered_idxs || (dy_grouped && x_grouped && !dy_scale), XMA_ROCM_EINVAL,
                 "group_bwd_W_few_rows: sorted_scattered_idxs is required unless everything is grouped");
-    const int cpr = K_in / 8;
-    int groups = (cpr < FR_THREADS) ? FR_THREADS / cpr : 1;
-    if (groups > FR_GROUPS) groups = FR_GROUPS;
-    const int64_t rows_n = ((int64_t)N_out + FR_NB * groups - 1) / (FR_NB * groups);
-    XMA_REQUIRE(rows_n <= 65535, XMA_ROCM_EUNSUPPORTED, "group_bwd_W_few_rows: N_out=%d exceeds %d", N_out, 65535 * FR_NB);
+    XMA_REQUIRE((N_out + DT_TILE - 1) / DT_TILE <= 65535, XMA_ROCM_EUNSUPPORTED, "group_bwd_W_few_rows: N_out=%d exceeds %d", N_out,
+                65535 * DT_TILE);
     DwArgs a;
     a.DY = (const uint16_t *)DY;
     a.lddy = lddy;
@@ -134,13 +157,13 @@ extern "C" int xma_rocm_group_bwd_W_few_rows(const void *DY, int64_t lddy, int d
     a.x_fan_out = x_fan_out;
     a.dy_div = make_fastdiv((uint32_t)dy_fan_out);
     a.x_div = make_fastdiv((uint32_t)x_fan_out);
-    const dim3 grid(groups > 1 ? 1 : (cpr + FR_THREADS - 1) / FR_THREADS, (unsigned)rows_n, E);
     hipStream_t st = (hipStream_t)stream;
+    const dim3 grid((K_in + DT_TILE - 1) / DT_TILE, (N_out + DT_TILE - 1) / DT_TILE, E);
     if (dtype == XMA_ROCM_BF16)
-        dw_few_rows_kernel<__bf16><<<grid, FR_THREADS, 0, st>>>(a);
+        dw_tile_kernel<__bf16><<<grid, FR_THREADS, 0, st>>>(a);
     else
-        dw_few_rows_kernel<_Float16><<<grid, FR_THREADS, 0, st>>>(a);
-    return xma_check_launch("dw_few_rows_kernel");
+        dw_tile_kernel<_Float16><<<grid, FR_THREADS, 0, st>>>(a);
+    return xma_check_launch("dw_tile_kernel");
 }
 
 namespace {
@@ -420,26 +443,33 @@ __global__ __launch_bounds__(FR_THREADS) void fr_epilogue_kernel(const FwdArgs a
 // ------------------------------------------------------------------------------------------------
 // 5 to 32 rows per expert: too many for vector FMAs (one pass over the weights per 4 or 8 rows), too few for the
 // 256 x 256 tiles (one 32 KB stage of weights in flight per compute unit).  A small MFMA tile instead: 32 rows of the
-// expert x 128 output columns, K in steps of 64, operands through registers into two LDS stages of 20 KB, so that four
-// workgroups share a compute unit and keep 80 KB of loads in flight.  One v_mfma_f32_32x32x16 block per wave; lane l holds
-// 16 sums of row l % 32 in quads of 4 consecutive columns, so bias, row scale and the epilogues are lane-local, with the
-// arithmetic of tile_epilogue in grouped_gemm.hip.  An expert's rows are taken 32 at a time.
-//   WT = 0, W[e] as (N, K): the W tile is [128 n][64 k], read back with ds_read_b128 like the X tile.
-//   WT = 1, W[e] as (K, N): the W tile is [64 k][128 n] as it lies in memory; ds_read_b64_tr_b16 hands a lane 4
-//       consecutive k of one column (groups of 16 lanes: lane p addresses 4 columns of k-row p / 4 and receives column p).
+// expert x 128 output columns, operands through registers into 40 KB of LDS, so that four workgroups share a compute unit
+// and keep 80 KB of loads in flight.  One v_mfma_f32_32x32x16 block per wave; lane l holds 16 sums of row l % 32 in
+// quads of 4 consecutive columns, so bias, row scale and the epilogues are lane-local, with the arithmetic of
+// tile_epilogue in grouped_gemm.hip.  An expert's rows are taken 32 at a time.  Every load instruction of a workgroup
+// asks for 256 contiguous bytes per row of memory (128-byte pieces of 128 rows of W measured 4.4 TB/s, 256-byte pieces
+// the 5.6 TB/s of a copy):
+//   WT = 0, W[e] as (N, K): K in steps of 128; the W tile is [128 n][128 k] in one LDS stage, read back with ds_read_b128
+//       like the X tile; the next step waits in registers while this one is multiplied.
+//   WT = 1, W[e] as (K, N): K in steps of 64, two LDS stages of 20 KB; the W tile is [64 k][128 n] as it lies in memory;
+//       ds_read_b64_tr_b16 hands a lane 4 consecutive k of one column (groups of 16 lanes: lane p addresses 4 columns of
+//       k-row p / 4 and receives column p).
 // ------------------------------------------------------------------------------------------------
-constexpr int ST_M = 32, ST_N = 128, ST_K = 64;
+constexpr int ST_M = 32, ST_N = 128, ST_K = 64, ST_K_NT = 128;
 constexpr int ST_W_BYTES = ST_N * ST_K * 2, ST_X_BYTES = ST_M * ST_K * 2, ST_STAGE = ST_W_BYTES + ST_X_BYTES;
+constexpr int ST_W_BYTES_NT = ST_N * ST_K_NT * 2;
+__host__ __device__ constexpr int st_k(int wt) { return wt ? ST_K : ST_K_NT; } // K of a step
 
 // 16-byte slot of (row, chunk) in a tile of 128-byte rows: chunk ^ (row & 7) keeps 8 consecutive rows off each other's banks
 __device__ __forceinline__ int st_slot(int row, int chunk) { return row * 128 + ((chunk ^ (row & 7)) << 4); }
-// the same for the [64 k][128 n] tile of 256-byte rows: 16-byte chunk c of k-row kr sits at c ^ ((kr & 3) << 2)
-__device__ __forceinline__ int st_slot_kn(int kr, int chunk) { return kr * 256 + ((chunk ^ ((kr & 3) << 2)) << 4); }
+// (the [64 k][128 n] tile of 256-byte rows uses st_slot_kn above)
+// and for tiles of 256-byte rows read along the row (WT = 0): chunk 0..15, the same rotation inside each half
+__device__ __forceinline__ int st_slot_nt(int row, int chunk) { return row * 256 + ((chunk ^ (row & 7)) << 4); }
 
 // EPI = -1: the launch is cut along K (blockIdx.z takes `steps_per` steps) because N alone gives too few workgroups; the
 // fp32 sums go to part[blockIdx.z][M][N] and fr_epilogue_kernel finishes.
 template <typename T, int WT, int EPI>
-__global__ __launch_bounds__(FR_THREADS) void fr_tile_kernel(const FwdArgs a, float *__restrict__ part, int steps_per) {
+__global__ __launch_bounds__(FR_THREADS, 4) void fr_tile_kernel(const FwdArgs a, float *__restrict__ part, int steps_per) {
     __shared__ __attribute__((aligned(16))) unsigned char s_t[2 * ST_STAGE];
     typedef short v4s __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) v4s *lds_v4s;
@@ -448,90 +478,114 @@ __global__ __launch_bounds__(FR_THREADS) void fr_tile_kernel(const FwdArgs a, fl
     if (lo >= hi) return; // uniform
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
     const int n0 = blockIdx.x * ST_N;
-    const int steps_all = (a.K + ST_K - 1) / ST_K;
+    const int steps_all = (a.K + st_k(WT) - 1) / st_k(WT);
     const int s_begin = (EPI < 0) ? blockIdx.z * steps_per : 0;
     const int s_end = (EPI < 0 && s_begin + steps_per < steps_all) ? s_begin + steps_per : steps_all;
-    // X loader: thread = (row tid / 8, chunk tid % 8); W loader, WT = 0: the same with rows + 32 i; WT = 1: (k-row
-    // tid / 16 + 16 i, 16-byte chunk tid % 16 of the 128 columns)
+    // loaders.  WT = 0: thread = (row tid / 16 + 16 i, 16-byte chunk tid % 16 of the step's 128 k) for both tiles, rows of W
+    // past N clamped (computed, never stored).  WT = 1: W thread = (k-row tid / 16 + 16 i, 16-byte chunk tid % 16 of the 128
+    // columns), X thread = (row tid / 8, chunk tid % 8 of the step's 64 k)
     const int ld_row = tid >> 3, ld_chunk = tid & 7;
     const int kn_row = tid >> 4, kn_chunk = tid & 15;
     const bool kn_ok = n0 + 8 * kn_chunk < a.N; // N % 8 == 0: a chunk is inside or outside
+    // WT = 0 addresses its 8 rows as a uniform base + 32-bit byte offsets (the host checks that N * ldw * 2 fits)
+    const unsigned char *w_base = (const unsigned char *)(a.W + (int64_t)e * a.w_es);
+    uint32_t w_off[8];
     const uint16_t *w_src[4];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        if constexpr (WT == 0) {
-            int n = n0 + ld_row + 32 * i;
-            if (n >= a.N) n = a.N - 1; // clamped: computed, never stored
-            w_src[i] = a.W + (int64_t)e * a.w_es + (int64_t)n * a.ldw + 8 * ld_chunk;
-        } else {
-            w_src[i] = a.W + (int64_t)e * a.w_es + (int64_t)(kn_row + 16 * i) * a.ldw + n0 + 8 * kn_chunk;
-        }
+    for (int i = 0; i < 8; ++i) {
+        int n = n0 + kn_row + 16 * i;
+        if (n >= a.N) n = a.N - 1;
+        w_off[i] = ((uint32_t)n * (uint32_t)a.ldw + 8u * kn_chunk) * 2u;
     }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w_src[i] = a.W + (int64_t)e * a.w_es + (int64_t)(kn_row + 16 * i) * a.ldw + n0 + 8 * kn_chunk;
     // this lane's fragment of the W tile (byte offset inside a stage, k slice 0)
-    int w_frag;
-    if constexpr (WT == 0) {
-        w_frag = 0; // st_slot depends on kk: computed in the loop
-    } else {
+    int w_frag = 0;
+    if constexpr (WT == 1) {
         const int p = lane & 15, G = lane >> 4;
         const int m = wave * 32 + ((G & 1) << 4) + ((p & 3) << 2), kr = ((G >> 1) << 3) + (p >> 2);
         w_frag = kr * 256 + ((((m >> 3) ^ ((kr & 3) << 2))) << 4) + ((m & 7) << 1);
     }
     for (int64_t r0 = lo; r0 < hi; r0 += ST_M) {
-        int64_t xr = r0 + ld_row;
-        if (xr >= hi) xr = hi - 1;
-        const uint16_t *x_src = a.X + fr_src_row(a, xr) * a.ldx + 8 * ld_chunk;
-        u32x4 wv[4], xv;
-        auto fetch = [&](int s) {
-            const u32x4 zero = {0u, 0u, 0u, 0u};
-            const bool x_ok = s * ST_K + 8 * ld_chunk < a.K; // chunks past K are zeros
-            xv = x_ok ? *(const u32x4 *)(x_src + s * ST_K) : zero;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                if constexpr (WT == 0) {
-                    wv[i] = x_ok ? __builtin_nontemporal_load((const u32x4 *)(w_src[i] + s * ST_K)) : zero;
-                } else {
-                    const bool ok = kn_ok && s * ST_K + kn_row + 16 * i < a.K;
-                    wv[i] = ok ? __builtin_nontemporal_load((const u32x4 *)(w_src[i] + (int64_t)s * ST_K * a.ldw)) : zero;
-                }
-            }
-        };
-        auto stash = [&](int stage) {
-            unsigned char *base = s_t + stage * ST_STAGE;
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                if constexpr (WT == 0)
-                    *(u32x4 *)(base + st_slot(ld_row + 32 * i, ld_chunk)) = wv[i];
-                else
-                    *(u32x4 *)(base + st_slot_kn(kn_row + 16 * i, kn_chunk)) = wv[i];
-            }
-            *(u32x4 *)(base + ST_W_BYTES + st_slot(ld_row, ld_chunk)) = xv;
-        };
         f32x16 acc;
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[i] = 0.f;
-        __syncthreads(); // the pass before no longer reads the stages
-        fetch(s_begin);
-        stash(s_begin & 1);
-        __syncthreads();
-        for (int s = s_begin; s < s_end; ++s) {
-            if (s + 1 < s_end) fetch(s + 1); // in flight while this step computes
-            unsigned char *base = s_t + (s & 1) * ST_STAGE;
+        const u32x4 zero = {0u, 0u, 0u, 0u};
+        if constexpr (WT == 0) {
+            const uint16_t *x_src[2];
 #pragma unroll
-            for (int kk = 0; kk < 4; ++kk) {
-                u32x4 wa;
-                if constexpr (WT == 0) {
-                    wa = *(const u32x4 *)(base + st_slot(wave * 32 + l32, 2 * kk + half));
-                } else { // k-rows 16 kk + ..: the swizzle depends on kr & 3 only, so kk adds 16 rows = 4096 bytes
+            for (int i = 0; i < 2; ++i) {
+                int64_t xr = r0 + kn_row + 16 * i;
+                if (xr >= hi) xr = hi - 1;
+                x_src[i] = a.X + fr_src_row(a, xr) * a.ldx + 8 * kn_chunk;
+            }
+            u32x4 wv[8], xv[2];
+            auto fetch = [&](int s) {
+                const bool ok = s * ST_K_NT + 8 * kn_chunk < a.K; // chunks past K are zeros
+#pragma unroll
+                for (int i = 0; i < 2; ++i) xv[i] = ok ? *(const u32x4 *)(x_src[i] + s * ST_K_NT) : zero;
+#pragma unroll
+                for (int i = 0; i < 8; ++i) wv[i] = ok ? __builtin_nontemporal_load((const u32x4 *)(w_base + (size_t)s * (ST_K_NT * 2) + w_off[i])) : zero;
+            };
+            fetch(s_begin);
+            // the 26 LDS addresses of a step are recomputed in every step from two values the compiler cannot see through
+            // (the vector ALU is idle here, and kept in registers they would cost the fourth workgroup per compute unit)
+            int slot_st = st_slot_nt(kn_row, kn_chunk), row_rd = l32;
+            for (int s = s_begin; s < s_end; ++s) {
+                asm volatile("" : "+v"(slot_st), "+v"(row_rd));
+                __syncthreads(); // the step (or the pass) before no longer reads the stage
+#pragma unroll
+                for (int i = 0; i < 8; ++i) *(u32x4 *)(s_t + slot_st + 16 * 256 * i) = wv[i]; // rows + 16 i: the same rotation
+#pragma unroll
+                for (int i = 0; i < 2; ++i) *(u32x4 *)(s_t + ST_W_BYTES_NT + slot_st + 16 * 256 * i) = xv[i];
+                __syncthreads();
+                if (s + 1 < s_end) fetch(s + 1); // in flight while this step is multiplied
+#pragma unroll
+                for (int kk = 0; kk < 8; ++kk) {
+                    const int slot = st_slot_nt(row_rd, 2 * kk + half);
+                    const u32x4 wa = *(const u32x4 *)(s_t + wave * (32 * 256) + slot);
+                    const u32x4 xb = *(const u32x4 *)(s_t + ST_W_BYTES_NT + slot);
+                    acc = Elem<T>::mfma(wa, xb, acc);
+                }
+            }
+        } else {
+            int64_t xr = r0 + ld_row;
+            if (xr >= hi) xr = hi - 1;
+            const uint16_t *x_src = a.X + fr_src_row(a, xr) * a.ldx + 8 * ld_chunk;
+            u32x4 wv[4], xv;
+            auto fetch = [&](int s) {
+                xv = (s * ST_K + 8 * ld_chunk < a.K) ? *(const u32x4 *)(x_src + s * ST_K) : zero; // chunks past K are zeros
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const bool ok = kn_ok && s * ST_K + kn_row + 16 * i < a.K;
+                    wv[i] = ok ? __builtin_nontemporal_load((const u32x4 *)(w_src[i] + (int64_t)s * ST_K * a.ldw)) : zero;
+                }
+            };
+            auto stash = [&](int stage) {
+                unsigned char *base = s_t + stage * ST_STAGE;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) *(u32x4 *)(base + st_slot_kn(kn_row + 16 * i, kn_chunk)) = wv[i];
+                *(u32x4 *)(base + ST_W_BYTES + st_slot(ld_row, ld_chunk)) = xv;
+            };
+            __syncthreads(); // the pass before no longer reads the stages
+            fetch(s_begin);
+            stash(s_begin & 1);
+            __syncthreads();
+            for (int s = s_begin; s < s_end; ++s) {
+                if (s + 1 < s_end) fetch(s + 1); // in flight while this step computes
+                unsigned char *base = s_t + (s & 1) * ST_STAGE;
+#pragma unroll
+                for (int kk = 0; kk < 4; ++kk) { // k-rows 16 kk + ..: the swizzle depends on kr & 3 only, so kk adds 16 rows = 4096 bytes
                     const v4s k03 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(base + w_frag + kk * 4096));
                     const v4s k47 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(base + w_frag + kk * 4096 + 1024));
                     const u32x2 a01 = __builtin_bit_cast(u32x2, k03), a23 = __builtin_bit_cast(u32x2, k47);
-                    wa = u32x4{a01[0], a01[1], a23[0], a23[1]};
+                    const u32x4 wa = u32x4{a01[0], a01[1], a23[0], a23[1]};
+                    const u32x4 xb = *(const u32x4 *)(base + ST_W_BYTES + st_slot(l32, 2 * kk + half));
+                    acc = Elem<T>::mfma(wa, xb, acc);
                 }
-                const u32x4 xb = *(const u32x4 *)(base + ST_W_BYTES + st_slot(l32, 2 * kk + half));
-                acc = Elem<T>::mfma(wa, xb, acc);
+                if (s + 1 < s_end) stash((s + 1) & 1); // that stage was last read in step s - 1, behind a barrier
+                __syncthreads();
             }
-            if (s + 1 < s_end) stash((s + 1) & 1); // that stage was last read in step s - 1, behind a barrier
-            __syncthreads();
         }
         const int64_t r = r0 + l32;
         if (r >= hi) continue;
@@ -592,12 +646,12 @@ inline bool fr_takes_tile(int64_t M, int E, int w_is_kn) {
 }
 
 // K ranges of the small MFMA tile: enough workgroups for four per compute unit (twice as many measured slower: the
-// partial sums and their kernel cost more than the extra parallelism brings), ranges of at least 8 steps
-inline int fr_tile_splits(int N, int K, int E) {
+// partial sums and their kernel cost more than the extra parallelism brings), ranges of at least 512 columns of K
+inline int fr_tile_splits(int N, int K, int E, int w_is_kn) {
     const int64_t wgs = (int64_t)((N + ST_N - 1) / ST_N) * E;
-    const int steps = (K + ST_K - 1) / ST_K;
+    const int ks = st_k(w_is_kn), steps = (K + ks - 1) / ks, min_steps = 512 / ks;
     int S = (int)((1024 + wgs - 1) / wgs);
-    if (S > steps / 8) S = steps / 8;
+    if (S > steps / min_steps) S = steps / min_steps;
     return S < 1 ? 1 : S;
 }
 
@@ -608,8 +662,8 @@ template <typename T, int EPI> int fr_launch_epilogue(const FwdArgs &a, const fl
 }
 
 template <typename T, int WT, int EPI> int fr_launch_tile(const FwdArgs &a, float *part, hipStream_t st) {
-    const int S = fr_tile_splits(a.N, a.K, a.E);
-    const int steps_all = (a.K + ST_K - 1) / ST_K, steps_per = (steps_all + S - 1) / S;
+    const int S = fr_tile_splits(a.N, a.K, a.E, WT);
+    const int steps_all = (a.K + st_k(WT) - 1) / st_k(WT), steps_per = (steps_all + S - 1) / S;
     const dim3 grid((a.N + ST_N - 1) / ST_N, a.E, S);
     if (S == 1) {
         fr_tile_kernel<T, WT, EPI><<<grid, FR_THREADS, 0, st>>>(a, nullptr, steps_all);
@@ -657,7 +711,7 @@ extern "C" size_t xma_rocm_scatter2scatter_few_rows_workspace_bytes(int64_t M, i
     if (M <= 0 || N <= 0 || K <= 0 || E <= 0) return 0;
     int S;
     if (fr_takes_tile(M, E, w_is_kn)) { // the small MFMA tile, cut along K or not
-        S = fr_tile_splits(N, K, E);
+        S = fr_tile_splits(N, K, E, w_is_kn);
         if (S == 1) return 0;
     } else if (w_is_kn) { // partial sums of the K ranges
         const int kc = fr_nn_range(K);

@@ -86,11 +86,10 @@ CONTINUOUS_COUNT_SET_MAX_BINS = 8192
 # them 256 x 256 for the matrix pipes, up to FEW_ROWS_PER_EXPERT rows per expert on average.  The limits are measured
 # cross-overs (8 experts of H = 2048, I = 8192; 64 of H = 2048, I = 1408; 128 of H = 576, I = 256): the forward-type GEMMs
 # walk an expert's rows 32 at a time (small MFMA tile; vector FMAs up to 2 rows per expert and 64 rows in all, the library
-# decides), each pass streaming the weights again, so they lead while most experts need one pass; the weight gradient is
-# vector FMAs throughout and grows with the rows.
-FEW_ROWS_PER_EXPERT = {"x @ W^T": 24, "dy @ W": 24, "dW": 16}
-FEW_ROWS_MAX = 256  # weight gradient: beyond that its per-row work shows where the experts are small
-FEW_ROWS_MAX_MFMA = 4096  # forward-type GEMMs
+# decides), each pass streaming the weights again, so they lead while most experts need one pass; the weight gradient
+# holds a 128 x 128 tile of dW in registers while it walks the rows, so it leads as long as its stores outweigh its loads.
+FEW_ROWS_PER_EXPERT = {"x @ W^T": 24, "dy @ W": 24, "dW": 128}
+FEW_ROWS_MAX = 16384  # rows in all, every form (beyond the measured range; 0 switches the few-token entry points off)
 FEW_ROWS_MAX_WORKSPACE = 256 << 20  # bytes of fp32 partial sums a forward-type launch may ask for
 
 
@@ -170,8 +169,7 @@ FEW_ROWS_NN_MAX_K = 65536  # limit of the few-token entry point for W as (K, N)
 
 def _few_rows(M: int, E: int, dtype: torch.dtype, form: str) -> bool:
     """whether a grouped GEMM of M rows over E experts takes an entry point written for the few-token regime"""
-    cap = FEW_ROWS_MAX_MFMA if form != "dW" and FEW_ROWS_MAX > 0 else FEW_ROWS_MAX
-    return 0 < M <= min(cap, FEW_ROWS_PER_EXPERT[form] * E) and dtype in (torch.bfloat16, torch.float16)
+    return 0 < M <= min(FEW_ROWS_MAX, FEW_ROWS_PER_EXPERT[form] * E) and dtype in (torch.bfloat16, torch.float16)
 
 
 def _few_rows_fwd(lib, M: int, N: int, K: int, E: int, w_is_kn: int, dtype: torch.dtype, epilogue: int) -> bool:

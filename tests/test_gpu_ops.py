@@ -348,8 +348,8 @@ FEW_ROWS_CASES = [
 @pytest.mark.parametrize("case", FEW_ROWS_CASES)
 def test_forward_type_gemms_few_rows(dtype, case):
     """The six operand forms of the layer's forward-type GEMMs through the kernels written for a handful of rows (weights
-    streamed once, vector FMAs, sums through a workspace, one small epilogue kernel), each against the oracle and against
-    the MFMA kernels on the same operands: up-projection + SwiGLU with a bias (z and h), up-projection with a plain store,
+    streamed once per 32 rows of an expert; vector FMAs or a small MFMA tile, sums through a workspace and one small
+    epilogue kernel where K is cut), each against the oracle and against the 256 x 256 kernels on the same operands: up-projection + SwiGLU with a bias (z and h), up-projection with a plain store,
     down-projection with a bias, a row scale and scattered rows, dX1 (dz @ W1, scattered), dX2 + SwiGLU backward with and
     without the scaled activations."""
     from xma.rocm import ops
@@ -454,10 +454,12 @@ def test_forward_type_gemms_few_rows(dtype, case):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("case", [(7, 8, 2, 264, 136, ()), (3, 128, 8, 576, 512, ()), (16, 4, 4, 2048, 72, (2,)), (1, 8, 1, 64, 8, ()),
-                                  (9, 5, 3, 4104, 24, (0, 4))])
+                                  (9, 5, 3, 4104, 24, (0, 4)), (100, 3, 2, 200, 328, ())])
 def test_group_bwd_W_few_rows(dtype, case):
-    """The weight gradient written for a handful of rows (an outer product per row, streamed stores) against the oracle
-    and against the MFMA kernel on the same operands: every operand form of the layer, more than 2048 columns (two column blocks, the second partly filled), experts without rows (zeros), more experts than rows."""
+    """The weight gradient written for a handful of rows (a 128 x 128 tile of dW per workgroup, the expert's rows as the K
+    dimension of the MFMAs, 32 at a time, streamed stores) against the oracle and against the 256 x 256 kernel on the same
+    operands: every operand form of the layer, tiles partly outside dW in both directions, experts without rows (zeros),
+    more experts than rows, about 67 rows per expert (two full passes and a partial one)."""
     from xma.rocm import ops
 
     T, E, k, K, N, empty = case

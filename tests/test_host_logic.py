@@ -87,6 +87,7 @@ def test_argument_errors_are_reported_before_any_launch():
     dw = lib.xma_rocm_group_bwd_W_few_rows
     assert dw(p, 64, 1, 1, None, p, 64, 1, 1, p, p, p, 64 * 64, 64, 64, 64, 2, 2, None) == -2  # fp32
     assert dw(p, 64, 1, 1, None, p, 60, 1, 1, p, p, p, 64 * 64, 64, 64, 64, 2, 0, None) == -2  # ldx % 8
+    assert dw(p, 60, 1, 1, None, p, 64, 1, 1, p, p, p, 64 * 64, 64, 64, 64, 2, 0, None) == -2  # lddy % 8
     assert dw(None, 64, 1, 1, None, p, 64, 1, 1, p, p, p, 64 * 64, 64, 64, 64, 2, 0, None) == -1
     # empty problems are accepted without touching a pointer
     assert few(None, 64, None, 64 * 64, 64, 0, None, None, None, 64, None, 0, None, 0, None, None, 0, 0, 64, 64, 2, 1, 1, 1, 0, 0, None, 0, None) == 0
@@ -101,10 +102,10 @@ def test_few_token_dispatch_rule():
 
     bf = torch.bfloat16
     assert ops._few_rows(14, 8, bf, "x @ W^T") and ops._few_rows(192, 8, bf, "x @ W^T") and not ops._few_rows(193, 8, bf, "x @ W^T")
-    assert ops._few_rows(3072, 128, bf, "dy @ W") and not ops._few_rows(4097, 256, bf, "x @ W^T")  # their cap on the rows
+    assert ops._few_rows(3072, 128, bf, "dy @ W") and not ops._few_rows(16385, 1024, bf, "x @ W^T")  # the cap on the rows
     assert ops._few_rows(192, 8, bf, "dy @ W") and not ops._few_rows(193, 8, bf, "dy @ W")
-    assert ops._few_rows(128, 8, bf, "dW") and not ops._few_rows(129, 8, bf, "dW")
-    assert ops._few_rows(256, 128, bf, "dW") and not ops._few_rows(257, 128, bf, "dW")  # the weight gradient's cap
+    assert ops._few_rows(1024, 8, bf, "dW") and not ops._few_rows(1025, 8, bf, "dW")
+    assert ops._few_rows(16384, 128, bf, "dW") and not ops._few_rows(16385, 128, bf, "dW")
     assert not ops._few_rows(0, 8, bf, "dW") and not ops._few_rows(14, 8, torch.float32, "dW")
     assert ops._few_rows(14, 8, torch.float16, "dy @ W")
 
