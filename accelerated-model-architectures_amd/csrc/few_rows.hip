@@ -441,12 +441,12 @@ __global__ __launch_bounds__(FR_THREADS) void fr_epilogue_kernel(const FwdArgs a
 }
 
 // ------------------------------------------------------------------------------------------------
-// 5 to 32 rows per expert: too many for vector FMAs (one pass over the weights per 4 or 8 rows), too few for the
-// 256 x 256 tiles (one 32 KB stage of weights in flight per compute unit).  A small MFMA tile instead: 32 rows of the
-// expert x 128 output columns, operands through registers into 40 KB of LDS, so that four workgroups share a compute unit
-// and keep 80 KB of loads in flight.  One v_mfma_f32_32x32x16 block per wave; lane l holds 16 sums of row l % 32 in
+// 3 to 64 rows per expert: too many for vector FMAs (one pass over the weights per 4 or 8 rows), too few for the
+// 256 x 256 tiles (one 32 KB stage of weights in flight per compute unit).  A small MFMA tile instead: 32 (or 64) rows of
+// the expert x 128 output columns, operands through registers into 40 (48) KB of LDS, so that four (three) workgroups
+// share a compute unit and keep 80 KB of loads in flight.  One v_mfma_f32_32x32x16 block per wave; lane l holds 16 sums of row l % 32 in
 // quads of 4 consecutive columns, so bias, row scale and the epilogues are lane-local, with the arithmetic of
-// tile_epilogue in grouped_gemm.hip.  An expert's rows are taken 32 at a time.  Every load instruction of a workgroup
+// tile_epilogue in grouped_gemm.hip.  An expert's rows are taken 32 or 64 at a time.  Every load instruction of a workgroup
 // asks for 256 contiguous bytes per row of memory (128-byte pieces of 128 rows of W measured 4.4 TB/s, 256-byte pieces
 // the 5.6 TB/s of a copy):
 //   WT = 0, W[e] as (N, K): K in steps of 128; the W tile is [128 n][128 k] in one LDS stage, read back with ds_read_b128
@@ -468,9 +468,11 @@ __device__ __forceinline__ int st_slot_nt(int row, int chunk) { return row * 256
 
 // EPI = -1: the launch is cut along K (blockIdx.z takes `steps_per` steps) because N alone gives too few workgroups; the
 // fp32 sums go to part[blockIdx.z][M][N] and fr_epilogue_kernel finishes.
-template <typename T, int WT, int EPI>
-__global__ __launch_bounds__(FR_THREADS, 4) void fr_tile_kernel(const FwdArgs a, float *__restrict__ part, int steps_per) {
-    __shared__ __attribute__((aligned(16))) unsigned char s_t[2 * ST_STAGE];
+// MB = 32-row blocks of the expert per pass (1 or 2): the weights are streamed once per pass.
+template <typename T, int WT, int EPI, int MB>
+__global__ __launch_bounds__(FR_THREADS, MB == 1 ? 4 : 3) void fr_tile_kernel(const FwdArgs a, float *__restrict__ part, int steps_per) {
+    constexpr int X_BYTES = MB * ST_X_BYTES, STAGE = ST_W_BYTES + X_BYTES; // WT = 1, per stage
+    __shared__ __attribute__((aligned(16))) unsigned char s_t[WT == 0 ? ST_W_BYTES_NT + 2 * X_BYTES : 2 * STAGE];
     typedef short v4s __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) v4s *lds_v4s;
     const int e = blockIdx.y;
@@ -506,24 +508,26 @@ __global__ __launch_bounds__(FR_THREADS, 4) void fr_tile_kernel(const FwdArgs a,
         const int m = wave * 32 + ((G & 1) << 4) + ((p & 3) << 2), kr = ((G >> 1) << 3) + (p >> 2);
         w_frag = kr * 256 + ((((m >> 3) ^ ((kr & 3) << 2))) << 4) + ((m & 7) << 1);
     }
-    for (int64_t r0 = lo; r0 < hi; r0 += ST_M) {
-        f32x16 acc;
+    for (int64_t r0 = lo; r0 < hi; r0 += MB * ST_M) {
+        f32x16 acc[MB];
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[i] = 0.f;
+        for (int b = 0; b < MB; ++b)
+#pragma unroll
+            for (int i = 0; i < 16; ++i) acc[b][i] = 0.f;
         const u32x4 zero = {0u, 0u, 0u, 0u};
         if constexpr (WT == 0) {
-            const uint16_t *x_src[2];
+            const uint16_t *x_src[2 * MB];
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
+            for (int i = 0; i < 2 * MB; ++i) {
                 int64_t xr = r0 + kn_row + 16 * i;
                 if (xr >= hi) xr = hi - 1;
                 x_src[i] = a.X + fr_src_row(a, xr) * a.ldx + 8 * kn_chunk;
             }
-            u32x4 wv[8], xv[2];
+            u32x4 wv[8], xv[2 * MB];
             auto fetch = [&](int s) {
                 const bool ok = s * ST_K_NT + 8 * kn_chunk < a.K; // chunks past K are zeros
 #pragma unroll
-                for (int i = 0; i < 2; ++i) xv[i] = ok ? *(const u32x4 *)(x_src[i] + s * ST_K_NT) : zero;
+                for (int i = 0; i < 2 * MB; ++i) xv[i] = ok ? *(const u32x4 *)(x_src[i] + s * ST_K_NT) : zero;
 #pragma unroll
                 for (int i = 0; i < 8; ++i) wv[i] = ok ? __builtin_nontemporal_load((const u32x4 *)(w_base + (size_t)s * (ST_K_NT * 2) + w_off[i])) : zero;
             };
@@ -537,24 +541,29 @@ __global__ __launch_bounds__(FR_THREADS, 4) void fr_tile_kernel(const FwdArgs a,
 #pragma unroll
                 for (int i = 0; i < 8; ++i) *(u32x4 *)(s_t + slot_st + 16 * 256 * i) = wv[i]; // rows + 16 i: the same rotation
 #pragma unroll
-                for (int i = 0; i < 2; ++i) *(u32x4 *)(s_t + ST_W_BYTES_NT + slot_st + 16 * 256 * i) = xv[i];
+                for (int i = 0; i < 2 * MB; ++i) *(u32x4 *)(s_t + ST_W_BYTES_NT + slot_st + 16 * 256 * i) = xv[i];
                 __syncthreads();
                 if (s + 1 < s_end) fetch(s + 1); // in flight while this step is multiplied
 #pragma unroll
                 for (int kk = 0; kk < 8; ++kk) {
                     const int slot = st_slot_nt(row_rd, 2 * kk + half);
                     const u32x4 wa = *(const u32x4 *)(s_t + wave * (32 * 256) + slot);
-                    const u32x4 xb = *(const u32x4 *)(s_t + ST_W_BYTES_NT + slot);
-                    acc = Elem<T>::mfma(wa, xb, acc);
+#pragma unroll
+                    for (int b = 0; b < MB; ++b) acc[b] = Elem<T>::mfma(wa, *(const u32x4 *)(s_t + ST_W_BYTES_NT + b * (32 * 256) + slot), acc[b]);
                 }
             }
         } else {
-            int64_t xr = r0 + ld_row;
-            if (xr >= hi) xr = hi - 1;
-            const uint16_t *x_src = a.X + fr_src_row(a, xr) * a.ldx + 8 * ld_chunk;
-            u32x4 wv[4], xv;
+            const uint16_t *x_src[MB];
+#pragma unroll
+            for (int b = 0; b < MB; ++b) {
+                int64_t xr = r0 + ld_row + 32 * b;
+                if (xr >= hi) xr = hi - 1;
+                x_src[b] = a.X + fr_src_row(a, xr) * a.ldx + 8 * ld_chunk;
+            }
+            u32x4 wv[4], xv[MB];
             auto fetch = [&](int s) {
-                xv = (s * ST_K + 8 * ld_chunk < a.K) ? *(const u32x4 *)(x_src + s * ST_K) : zero; // chunks past K are zeros
+#pragma unroll
+                for (int b = 0; b < MB; ++b) xv[b] = (s * ST_K + 8 * ld_chunk < a.K) ? *(const u32x4 *)(x_src[b] + s * ST_K) : zero; // chunks past K are zeros
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const bool ok = kn_ok && s * ST_K + kn_row + 16 * i < a.K;
@@ -562,10 +571,11 @@ __global__ __launch_bounds__(FR_THREADS, 4) void fr_tile_kernel(const FwdArgs a,
                 }
             };
             auto stash = [&](int stage) {
-                unsigned char *base = s_t + stage * ST_STAGE;
+                unsigned char *base = s_t + stage * STAGE;
 #pragma unroll
                 for (int i = 0; i < 4; ++i) *(u32x4 *)(base + st_slot_kn(kn_row + 16 * i, kn_chunk)) = wv[i];
-                *(u32x4 *)(base + ST_W_BYTES + st_slot(ld_row, ld_chunk)) = xv;
+#pragma unroll
+                for (int b = 0; b < MB; ++b) *(u32x4 *)(base + ST_W_BYTES + st_slot(ld_row + 32 * b, ld_chunk)) = xv[b];
             };
             __syncthreads(); // the pass before no longer reads the stages
             fetch(s_begin);
@@ -573,66 +583,70 @@ __global__ __launch_bounds__(FR_THREADS, 4) void fr_tile_kernel(const FwdArgs a,
             __syncthreads();
             for (int s = s_begin; s < s_end; ++s) {
                 if (s + 1 < s_end) fetch(s + 1); // in flight while this step computes
-                unsigned char *base = s_t + (s & 1) * ST_STAGE;
+                unsigned char *base = s_t + (s & 1) * STAGE;
 #pragma unroll
                 for (int kk = 0; kk < 4; ++kk) { // k-rows 16 kk + ..: the swizzle depends on kr & 3 only, so kk adds 16 rows = 4096 bytes
                     const v4s k03 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(base + w_frag + kk * 4096));
                     const v4s k47 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(base + w_frag + kk * 4096 + 1024));
                     const u32x2 a01 = __builtin_bit_cast(u32x2, k03), a23 = __builtin_bit_cast(u32x2, k47);
                     const u32x4 wa = u32x4{a01[0], a01[1], a23[0], a23[1]};
-                    const u32x4 xb = *(const u32x4 *)(base + ST_W_BYTES + st_slot(l32, 2 * kk + half));
-                    acc = Elem<T>::mfma(wa, xb, acc);
+#pragma unroll
+                    for (int b = 0; b < MB; ++b)
+                        acc[b] = Elem<T>::mfma(wa, *(const u32x4 *)(base + ST_W_BYTES + st_slot(l32 + 32 * b, 2 * kk + half)), acc[b]);
                 }
                 if (s + 1 < s_end) stash((s + 1) & 1); // that stage was last read in step s - 1, behind a barrier
                 __syncthreads();
             }
         }
-        const int64_t r = r0 + l32;
-        if (r >= hi) continue;
-        if constexpr (EPI < 0) {
-            float *mine = part + ((int64_t)blockIdx.z * a.M + r) * a.N;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int n = n0 + wave * 32 + 8 * g + 4 * half;
-                if (n < a.N) *(float4 *)(mine + n) = make_float4(acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]);
+        for (int b = 0; b < MB; ++b) {
+            const int64_t r = r0 + 32 * b + l32;
+            if (r >= hi) continue;
+            if constexpr (EPI < 0) {
+                float *mine = part + ((int64_t)blockIdx.z * a.M + r) * a.N;
+    #pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int n = n0 + wave * 32 + 8 * g + 4 * half;
+                    if (n < a.N) *(float4 *)(mine + n) = make_float4(acc[b][4 * g], acc[b][4 * g + 1], acc[b][4 * g + 2], acc[b][4 * g + 3]);
+                }
+                continue;
             }
-            continue;
-        }
-        const int64_t s_idx = a.idx ? a.idx[r] : r;
-        const float sc = a.scale ? fr_scalar<T>(a.scale, s_idx) : 1.f;
-        const int64_t dst = a.y_grouped ? r : s_idx;
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const int n = n0 + wave * 32 + 8 * g + 4 * half; // acc[4 g + q] is column n + q of row r
-            if (n >= a.N) continue;
-            if constexpr (EPI == XMA_ROCM_EPI_SWIGLU_BWD) {
-                // d h of 4 columns -> (d gate, d up) of their 4 pairs; rows are grouped on both sides
-                const u32x4 z = *(const u32x4 *)(a.aux + r * a.ldaux + 2 * n);
-                u32x4 o;
-                float hv[4];
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const float dh = acc[4 * g + q] * sc;
-                    const float gg = Elem<T>::lo(z[q]), uu = Elem<T>::hi(z[q]);
-                    const float sg = sigmoidf_fast(gg), silu = gg * sg;
-                    o[q] = Elem<T>::pack(dh * uu * (sg + silu * (1.f - sg)), dh * silu);
-                    hv[q] = uu * silu * sc;
-                }
-                *(u32x4 *)(a.out + r * a.ldo + 2 * n) = o;
-                if (a.aux2) *(u32x2 *)(a.aux2 + r * a.ldaux2 + n) = u32x2{Elem<T>::pack(hv[0], hv[1]), Elem<T>::pack(hv[2], hv[3])};
-            } else {
-                float v[4];
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    v[q] = acc[4 * g + q];
-                    if (a.bias) v[q] += fr_scalar<T>(a.bias, (int64_t)e * a.bias_es + n + q);
-                    v[q] *= sc;
-                }
-                const uint32_t z0 = Elem<T>::pack(v[0], v[1]), z1 = Elem<T>::pack(v[2], v[3]);
-                if (a.out) *(u32x2 *)(a.out + dst * a.ldo + n) = u32x2{z0, z1};
-                if constexpr (EPI == XMA_ROCM_EPI_SWIGLU) {
-                    const float g0 = Elem<T>::lo(z0), u0 = Elem<T>::hi(z0), g1 = Elem<T>::lo(z1), u1 = Elem<T>::hi(z1);
-                    *(uint32_t *)(a.aux + dst * a.ldaux + (n >> 1)) = Elem<T>::pack(u0 * g0 * sigmoidf_fast(g0), u1 * g1 * sigmoidf_fast(g1));
+            const int64_t s_idx = a.idx ? a.idx[r] : r;
+            const float sc = a.scale ? fr_scalar<T>(a.scale, s_idx) : 1.f;
+            const int64_t dst = a.y_grouped ? r : s_idx;
+    #pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int n = n0 + wave * 32 + 8 * g + 4 * half; // acc[b][4 g + q] is column n + q of row r
+                if (n >= a.N) continue;
+                if constexpr (EPI == XMA_ROCM_EPI_SWIGLU_BWD) {
+                    // d h of 4 columns -> (d gate, d up) of their 4 pairs; rows are grouped on both sides
+                    const u32x4 z = *(const u32x4 *)(a.aux + r * a.ldaux + 2 * n);
+                    u32x4 o;
+                    float hv[4];
+    #pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const float dh = acc[b][4 * g + q] * sc;
+                        const float gg = Elem<T>::lo(z[q]), uu = Elem<T>::hi(z[q]);
+                        const float sg = sigmoidf_fast(gg), silu = gg * sg;
+                        o[q] = Elem<T>::pack(dh * uu * (sg + silu * (1.f - sg)), dh * silu);
+                        hv[q] = uu * silu * sc;
+                    }
+                    *(u32x4 *)(a.out + r * a.ldo + 2 * n) = o;
+                    if (a.aux2) *(u32x2 *)(a.aux2 + r * a.ldaux2 + n) = u32x2{Elem<T>::pack(hv[0], hv[1]), Elem<T>::pack(hv[2], hv[3])};
+                } else {
+                    float v[4];
+    #pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        v[q] = acc[b][4 * g + q];
+                        if (a.bias) v[q] += fr_scalar<T>(a.bias, (int64_t)e * a.bias_es + n + q);
+                        v[q] *= sc;
+                    }
+                    const uint32_t z0 = Elem<T>::pack(v[0], v[1]), z1 = Elem<T>::pack(v[2], v[3]);
+                    if (a.out) *(u32x2 *)(a.out + dst * a.ldo + n) = u32x2{z0, z1};
+                    if constexpr (EPI == XMA_ROCM_EPI_SWIGLU) {
+                        const float g0 = Elem<T>::lo(z0), u0 = Elem<T>::hi(z0), g1 = Elem<T>::lo(z1), u1 = Elem<T>::hi(z1);
+                        *(uint32_t *)(a.aux + dst * a.ldaux + (n >> 1)) = Elem<T>::pack(u0 * g0 * sigmoidf_fast(g0), u1 * g1 * sigmoidf_fast(g1));
+                    }
                 }
             }
         }
@@ -661,18 +675,26 @@ template <typename T, int EPI> int fr_launch_epilogue(const FwdArgs &a, const fl
     return xma_check_launch("fr_epilogue_kernel");
 }
 
-template <typename T, int WT, int EPI> int fr_launch_tile(const FwdArgs &a, float *part, hipStream_t st) {
+// passes of 64 rows once many experts have more than 32 (below that they are 3-15 % slower than passes of 32: three
+// workgroups per compute unit instead of four, by registers and LDS)
+inline int fr_tile_row_blocks(int64_t M, int E) { return M > (int64_t)24 * E ? 2 : 1; }
+
+template <typename T, int WT, int EPI, int MB> int fr_launch_tile_mb(const FwdArgs &a, float *part, hipStream_t st) {
     const int S = fr_tile_splits(a.N, a.K, a.E, WT);
     const int steps_all = (a.K + st_k(WT) - 1) / st_k(WT), steps_per = (steps_all + S - 1) / S;
     const dim3 grid((a.N + ST_N - 1) / ST_N, a.E, S);
     if (S == 1) {
-        fr_tile_kernel<T, WT, EPI><<<grid, FR_THREADS, 0, st>>>(a, nullptr, steps_all);
+        fr_tile_kernel<T, WT, EPI, MB><<<grid, FR_THREADS, 0, st>>>(a, nullptr, steps_all);
         return xma_check_launch("fr_tile_kernel");
     }
-    fr_tile_kernel<T, WT, -1><<<grid, FR_THREADS, 0, st>>>(a, part, steps_per);
+    fr_tile_kernel<T, WT, -1, MB><<<grid, FR_THREADS, 0, st>>>(a, part, steps_per);
     int rc = xma_check_launch("fr_tile_kernel");
     if (rc) return rc;
     return fr_launch_epilogue<T, EPI>(a, part, (steps_all + steps_per - 1) / steps_per, st);
+}
+
+template <typename T, int WT, int EPI> int fr_launch_tile(const FwdArgs &a, float *part, hipStream_t st) {
+    return fr_tile_row_blocks(a.M, a.E) == 2 ? fr_launch_tile_mb<T, WT, EPI, 2>(a, part, st) : fr_launch_tile_mb<T, WT, EPI, 1>(a, part, st);
 }
 
 template <typename T, int EPI> int fr_launch_epi(const FwdArgs &a, int w_is_kn, float *part, hipStream_t st) {
