@@ -201,14 +201,15 @@ XMA_API int xma_rocm_down_projection_dx_swiglu(const void *dY, int64_t lddy, con
  * only.  With a handful of rows per expert the product is a stream over the weights.  Up to 2 rows per expert on average
  * (and 64 in all) vector FMAs do the work: for W[e] as (N, K) a wave reads two rows of W with its lanes along K, for W[e]
  * as (K, N) threads own 8 columns each and walk a K range.  Beyond that a small MFMA tile (32 rows of the expert x 128
- * output columns, four workgroups per compute unit) takes over, cut along K where N alone gives too few workgroups.
+ * output columns and four workgroups per compute unit, or 64 rows and three from 24 rows per expert on average) takes
+ * over, cut along K where N alone gives too few workgroups.
  * Whatever does not finish in one kernel sums through the workspace (xma_rocm_scatter2scatter_few_rows_workspace_bytes
  * bytes for the same M, N, K, num_experts, w_is_kn and epilogue; 0 = none needed, pass NULL) to a small kernel that
  * applies the bias and the epilogue with the arithmetic of the MFMA kernels.  Limits: M and E at most 65535, K at most
- * 65536 for W as (K, N).  Correct for any M, but an expert's rows are walked 4 or 8 (vector kernels) or 32 (small tile)
- * at a time, each pass streaming its weights again: meant for launches of a few rows per expert (the torch ops of this
- * package take it up to 24 on average and 4096 in all).  No counterpart in the reference (its
- * kernel is the same for every size).
+ * 65536 for W as (K, N).  Correct for any M, but an expert's rows are walked 4 or 8 (vector kernels), 32 or 64 (small
+ * tile) at a time, each pass streaming its weights again: meant for launches of a few rows per expert (the torch ops of
+ * this package take it up to 48 on average and 16384 in all).  No counterpart in the reference (its kernel is the same
+ * for every size).
  */
 XMA_API size_t xma_rocm_scatter2scatter_few_rows_workspace_bytes(int64_t M, int32_t N, int32_t K, int32_t num_experts,
                                                          int w_is_kn, int epilogue);
@@ -239,12 +240,14 @@ XMA_API int xma_rocm_group_bwd_W(const void *DY, int64_t lddy, int dy_grouped, i
                          int dtype, void *stream);
 
 /*
- * xma_rocm_group_bwd_W for the few-token regime (same arguments, same result up to the order of the fp32 sums; bf16 /
- * fp16 only; DY needs no 16-byte alignment and N_out no multiple of 8).  One workgroup per 8 rows of DW[e] streams its
- * stores and adds one outer product per row of the expert with vector FMAs: with a handful of rows per expert the launch
- * runs at the rate of a fill of DW, where the MFMA tiles of xma_rocm_group_bwd_W spend a prologue, one K step and an
- * epilogue per 256 x 256 tile.  Correct for any number of rows, but its time grows with (rows per expert) x |DW|: meant
- * for launches of a few rows per expert (the torch ops take it up to 16 on average).  No counterpart in the reference (its kernel is the same for every size).
+ * xma_rocm_group_bwd_W for the few-token regime (same arguments and limits, same result up to the order of the fp32
+ * sums; bf16 / fp16 only; a scaled row of DY is rounded to the operand type before it is multiplied, as a scaled grouped
+ * copy would hold it).  One workgroup per 128 x 128 tile of DW[e]; the expert's rows are the K dimension of its MFMAs,
+ * 32 at a time: with a handful of rows per expert the launch runs at the rate of a fill of DW, where
+ * xma_rocm_group_bwd_W spends a prologue, one K step and an epilogue per 256 x 256 tile.  Correct for any number of rows;
+ * more rows are more passes over two 8 KB operand tiles, so it leads until the loads outweigh the stores (the torch ops
+ * take it up to 128 rows per expert on average).  No counterpart in the reference (its kernel is the same for every
+ * size).
  */
 XMA_API int xma_rocm_group_bwd_W_few_rows(const void *DY, int64_t lddy, int dy_grouped, int32_t dy_fan_out,
                                   const void *dy_scale, const void *X, int64_t ldx, int x_grouped, int32_t x_fan_out,
