@@ -763,6 +763,8 @@ extern "C" int xma_rocm_scatter2scatter_few_rows(const void *X, int64_t ldx, con
                 XMA_ROCM_EUNSUPPORTED, "scatter2scatter_few_rows: N=%d K=%d and the leading dimensions must be multiples of 8", N, K);
     XMA_REQUIRE(!w_is_kn || fr_nn_range(K) <= FR_NN_KC_MAX, XMA_ROCM_EUNSUPPORTED,
                 "scatter2scatter_few_rows: K=%d exceeds %d for W as (K, N)", K, FR_NN_KC_MAX * FR_NN_SPLITS);
+    XMA_REQUIRE(w_is_kn || (int64_t)N * ldw < ((int64_t)1 << 31) - 128, XMA_ROCM_EUNSUPPORTED,
+                "scatter2scatter_few_rows: N * ldw = %lld exceeds 2^31 - 128 elements for W as (N, K)", (long long)N * (long long)ldw);
     if (M == 0) return XMA_ROCM_OK;
     auto al16 = [](const void *p) { return ((uintptr_t)p & 15) == 0; };
     XMA_REQUIRE(X && W && expert_offsets && al16(X) && al16(W), XMA_ROCM_EINVAL, "scatter2scatter_few_rows: null or misaligned operand");

@@ -166,6 +166,7 @@ def scatter2scatter_workspace_bytes(M: int, N: int, K: int, E: int, device_index
 
 
 FEW_ROWS_NN_MAX_K = 65536  # limit of the few-token entry point for W as (K, N)
+FEW_ROWS_NT_MAX_ELEMENTS = (1 << 31) - 128  # and for W as (N, K): N * ldw
 
 
 def _few_rows(M: int, E: int, dtype: torch.dtype, form: str) -> bool:
@@ -173,9 +174,11 @@ def _few_rows(M: int, E: int, dtype: torch.dtype, form: str) -> bool:
     return 0 < M <= min(FEW_ROWS_MAX, FEW_ROWS_PER_EXPERT[form] * E) and dtype in (torch.bfloat16, torch.float16)
 
 
-def _few_rows_fwd(lib, M: int, N: int, K: int, E: int, w_is_kn: int, dtype: torch.dtype, epilogue: int) -> bool:
+def _few_rows_fwd(lib, M: int, N: int, K: int, E: int, w_is_kn: int, ldw: int, dtype: torch.dtype, epilogue: int) -> bool:
     """the same for a forward-type GEMM, whose few-token entry point has limits of its own"""
     if not _few_rows(M, E, dtype, "dy @ W" if w_is_kn else "x @ W^T") or (w_is_kn and K > FEW_ROWS_NN_MAX_K):
+        return False
+    if not w_is_kn and N * ldw >= FEW_ROWS_NT_MAX_ELEMENTS:  # it addresses the rows of W[e] with 32-bit byte offsets
         return False
     return lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes(M, N, K, E, w_is_kn, epilogue) <= FEW_ROWS_MAX_WORKSPACE
 
@@ -209,7 +212,7 @@ def _scatter2scatter(X, W, idx, offs, out, aux, scale, fan_out, x_grouped, y_gro
     if scale is not None:
         assert scale.dtype == X.dtype and scale.is_contiguous()
     lib = get_library()
-    if _few_rows_fwd(lib, M, N, K, W.size(0), w_is_kn, X.dtype, epilogue):
+    if _few_rows_fwd(lib, M, N, K, W.size(0), w_is_kn, ldw, X.dtype, epilogue):
         _scatter2scatter_few_rows(lib, X, W, w_is_kn, w_es, ldw, idx, offs, out, aux, None, scale, bias, fan_out, x_grouped,
                                   y_grouped, epilogue, M, N, K)
         return
@@ -314,7 +317,7 @@ def down_projection_dx_swiglu_scaled_act_rocm(
     w_is_kn, w_es, ldw = _weight_layout(W)
     assert w_is_kn == 1, "W should be the down-projection parameter as stored, (E, H, I) with I contiguous"
     lib = get_library()
-    if _few_rows_fwd(lib, M, N, K, E, 1, dY.dtype, EPI_SWIGLU_BWD):
+    if _few_rows_fwd(lib, M, N, K, E, 1, ldw, dY.dtype, EPI_SWIGLU_BWD):
         _scatter2scatter_few_rows(lib, dY, W, 1, w_es, ldw, sorted_scattered_idxs, expert_offsets, dz, z, scaled_act,
                                   row_scale, None, FAN_OUT, False, True, EPI_SWIGLU_BWD, M, N, K)
         return

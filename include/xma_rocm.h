@@ -206,7 +206,7 @@ XMA_API int xma_rocm_down_projection_dx_swiglu(const void *dY, int64_t lddy, con
  * Whatever does not finish in one kernel sums through the workspace (xma_rocm_scatter2scatter_few_rows_workspace_bytes
  * bytes for the same M, N, K, num_experts, w_is_kn and epilogue; 0 = none needed, pass NULL) to a small kernel that
  * applies the bias and the epilogue with the arithmetic of the MFMA kernels.  Limits: M and E at most 65535, K at most
- * 65536 for W as (K, N).  Correct for any M, but an expert's rows are walked 4 or 8 (vector kernels), 32 or 64 (small
+ * 65536 for W as (K, N), N * ldw below 2^31 - 128 elements for W as (N, K) (32-bit byte offsets inside an expert).  Correct for any M, but an expert's rows are walked 4 or 8 (vector kernels), 32 or 64 (small
  * tile) at a time, each pass streaming its weights again: meant for launches of a few rows per expert (the torch ops of
  * this package take it up to 48 on average and 16384 in all).  No counterpart in the reference (its kernel is the same
  * for every size).

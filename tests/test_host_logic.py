@@ -76,6 +76,9 @@ def test_argument_errors_are_reported_before_any_launch():
     assert b"workspace" in lib.xma_rocm_last_error()
     assert few(None, 64, None, 64 * 64, 64, 0, p, p, p, 64, None, 0, None, 0, None, None, 0, 4, 64, 64, 2, 1, 1, 1, 0, 0, None, 0, None) == -1
     assert b"null or misaligned" in lib.xma_rocm_last_error()
+    # W as (N, K) is addressed with 32-bit byte offsets inside an expert
+    assert few(p, 64, p, 64 << 26, 1 << 26, 0, p, p, p, 64, None, 0, None, 0, None, None, 0, 4, 64, 64, 2, 1, 1, 1, 0, 0, None, 0, None) == -2
+    assert b"N * ldw" in lib.xma_rocm_last_error()
     ws = lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes  # (M, N, K, E, w_is_kn, epilogue)
     assert ws(4, 64, 64, 2, 0, 0) == 0 and ws(4, 64, 64, 2, 0, 1) == 0  # the vector kernel finishes the job itself (2 rows per expert)
     assert ws(4, 64, 64, 2, 0, 2) == 4 * 64 * 4  # SwiGLU backward: through the epilogue kernel
