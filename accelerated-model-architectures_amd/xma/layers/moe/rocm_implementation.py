@@ -346,10 +346,15 @@ class _FusedSwiGLUExperts(torch.autograd.Function):
             ops.down_projection_dx_swiglu_rocm(
                 grad_out, w_proj.permute(0, 2, 1), sorted_scattered_idxs, expert_offsets, z, dz, flat_w, top_k
             )
-            grouped_dy = _scaled_grouped_dy(grad_out, sorted_scattered_idxs, flat_w, top_k)
-            ops.group_bwd_W_rocm(grouped_dy, h, sorted_scattered_idxs, expert_offsets, d_w_proj, None, 0, 0)
-            if b_proj is not None:
-                d_b_proj = _bias_grad(grouped_dy, None, expert_offsets, b_proj)
+            if b_proj is None and ops._few_rows(z.size(0), w_proj.size(0), z.dtype, "dW"):
+                # a handful of rows per expert: the weight gradient's loader gathers and scales the rows of dy itself (and
+                # rounds them like the copy would), one launch less
+                ops.group_bwd_W_rocm(grad_out, h, sorted_scattered_idxs, expert_offsets, d_w_proj, flat_w, top_k, 0)
+            else:
+                grouped_dy = _scaled_grouped_dy(grad_out, sorted_scattered_idxs, flat_w, top_k)
+                ops.group_bwd_W_rocm(grouped_dy, h, sorted_scattered_idxs, expert_offsets, d_w_proj, None, 0, 0)
+                if b_proj is not None:
+                    d_b_proj = _bias_grad(grouped_dy, None, expert_offsets, b_proj)
         d_w_fc = _empty_dw_like(w_fc)
         ops.group_bwd_W_rocm(dz, x, sorted_scattered_idxs, expert_offsets, d_w_fc, None, 0, top_k)
         d_b_fc = None if b_fc is None else _bias_grad(dz, None, expert_offsets, b_fc)
