@@ -213,10 +213,13 @@ __global__ __launch_bounds__(ROUTE_THREADS) void route_scan_kernel(uint32_t *__r
     if (tid == ROUTE_THREADS - 1) counts[e] = incl;
 }
 
-template <typename IdT, int BALLOT>
+// SINGLE = 1: the whole problem is one unit (n <= ROUTE_CHUNK, the few-token regime) and this kernel is the whole call:
+// the local sorted order is the global one, and the counts and offsets come out of the per-wave counters (no unit
+// histogram, no scan kernel; unit_base is not read and counts is written instead).
+template <typename IdT, int BALLOT, int SINGLE>
 __global__ __launch_bounds__(ROUTE_THREADS) void route_scatter_kernel(
     const IdT *__restrict__ ids, int64_t n, int E, int nbits, const uint32_t *__restrict__ unit_base,
-    const uint32_t *__restrict__ counts, int64_t *__restrict__ offs_incl, int64_t *__restrict__ offs_excl,
+    uint32_t *__restrict__ counts, int64_t *__restrict__ offs_incl, int64_t *__restrict__ offs_excl,
     IdT *__restrict__ sorted_ids, int64_t *__restrict__ sorted_pos) {
     // LDS: [E] global start of each expert's local run minus its local start, [WAVES][E] per-wave counters,
     //      [256] scan scratch, then the staged unit: local index and expert id of every sorted position
@@ -241,7 +244,7 @@ __global__ __launch_bounds__(ROUTE_THREADS) void route_scatter_kernel(
     }
 
     // global exclusive scan of counts over experts (wave 0, 64 experts per step) -> s_gbase; block 0 writes the offsets
-    if (wave == 0) {
+    if (SINGLE == 0 && wave == 0) {
         uint32_t carry = 0;
         for (int b = 0; b < E; b += WAVE) {
             const int e = b + lane;
@@ -296,11 +299,19 @@ __global__ __launch_bounds__(ROUTE_THREADS) void route_scatter_kernel(
     if (tid == ROUTE_THREADS - 1) s_scan[ROUTE_WAVES] = incl;
     uint32_t run = incl - mine;
     for (int e = e0; e < e1; ++e) {
-        s_gbase[e] -= run; // destination of local sorted position j of expert e = s_gbase[e] + j
+        const uint32_t start = run;
         for (int w = 0; w < ROUTE_WAVES; ++w) {
             const uint32_t c = s_ctr[w * E + e];
             s_ctr[w * E + e] = run;
             run += c;
+        }
+        if constexpr (SINGLE != 0) {
+            s_gbase[e] = 0; // local sorted position = global sorted position
+            counts[e] = run - start;
+            offs_incl[e] = (int64_t)run;
+            if (offs_excl) offs_excl[e] = (int64_t)start;
+        } else {
+            s_gbase[e] -= start; // destination of local sorted position j of expert e = s_gbase[e] + j
         }
     }
     __syncthreads();
@@ -370,8 +381,19 @@ int route_launch(const IdT *ids, int64_t n, int E, uint32_t *counts, int64_t *in
     while ((1 << nbits) < E) ++nbits;
     const size_t lds3 = route_scatter_lds(E);
     const bool ballot = g_route_rank_method.load(std::memory_order_relaxed) == 1;
-    const void *scatter = ballot ? (const void *)route_scatter_kernel<IdT, 1> : (const void *)route_scatter_kernel<IdT, 0>;
+    // both size classes get their LDS limit on the first call, whatever its size: a caller that warms up with one size
+    // and captures another into a graph makes no attribute call under capture
+    const void *single = ballot ? (const void *)route_scatter_kernel<IdT, 1, 1> : (const void *)route_scatter_kernel<IdT, 0, 1>;
+    const void *scatter = ballot ? (const void *)route_scatter_kernel<IdT, 1, 0> : (const void *)route_scatter_kernel<IdT, 0, 0>;
+    if (xma_set_max_lds_once(single, (int)route_scatter_lds(ROUTE_MAX_E))) return XMA_ROCM_ELAUNCH;
     if (xma_set_max_lds_once(scatter, (int)route_scatter_lds(ROUTE_MAX_E))) return XMA_ROCM_ELAUNCH;
+    if (units == 1) { // a single unit: one kernel counts, scans and sorts
+        if (ballot)
+            route_scatter_kernel<IdT, 1, 1><<<1, ROUTE_THREADS, lds3, st>>>(ids, n, E, nbits, nullptr, counts, incl, excl, sorted_ids, sorted_pos);
+        else
+            route_scatter_kernel<IdT, 0, 1><<<1, ROUTE_THREADS, lds3, st>>>(ids, n, E, nbits, nullptr, counts, incl, excl, sorted_ids, sorted_pos);
+        return xma_check_launch("route_scatter_kernel (single unit)");
+    }
     int rc, copies, stride;
     hist_lds_layout(E, copies, stride);
     histogram_kernel<IdT, 1><<<(int)units, HIST_THREADS, (size_t)copies * stride * sizeof(uint32_t), st>>>(
@@ -380,11 +402,11 @@ int route_launch(const IdT *ids, int64_t n, int E, uint32_t *counts, int64_t *in
     route_scan_kernel<<<E, ROUTE_THREADS, 0, st>>>(unit_hist, (int)units, counts);
     if ((rc = xma_check_launch("route_scan_kernel"))) return rc;
     if (ballot)
-        route_scatter_kernel<IdT, 1><<<(int)units, ROUTE_THREADS, lds3, st>>>(ids, n, E, nbits, unit_hist, counts, incl,
-                                                                              excl, sorted_ids, sorted_pos);
+        route_scatter_kernel<IdT, 1, 0><<<(int)units, ROUTE_THREADS, lds3, st>>>(ids, n, E, nbits, unit_hist, counts, incl,
+                                                                                 excl, sorted_ids, sorted_pos);
     else
-        route_scatter_kernel<IdT, 0><<<(int)units, ROUTE_THREADS, lds3, st>>>(ids, n, E, nbits, unit_hist, counts, incl,
-                                                                              excl, sorted_ids, sorted_pos);
+        route_scatter_kernel<IdT, 0, 0><<<(int)units, ROUTE_THREADS, lds3, st>>>(ids, n, E, nbits, unit_hist, counts, incl,
+                                                                                 excl, sorted_ids, sorted_pos);
     return xma_check_launch("route_scatter_kernel");
 }
 
