@@ -531,11 +531,18 @@ __global__ __launch_bounds__(FR_THREADS, MB == 1 ? 4 : 3) void fr_tile_kernel(co
 #pragma unroll
                 for (int i = 0; i < 8; ++i) wv[i] = ok ? __builtin_nontemporal_load((const u32x4 *)(w_base + (size_t)s * (ST_K_NT * 2) + w_off[i])) : zero;
             };
-            fetch(s_begin);
+            // Workgroups that run at the same time are at about the same step, and with every one walking K from the front
+            // all their requests of a moment would fall on the same 256 bytes of every 4 KB of a row, a fraction of the
+            // memory channels: each workgroup starts at a step of its own and wraps around (the fp32 sums of different
+            // column blocks are added in different orders).
+            const int n_steps = s_end - s_begin;
+            int s_at = s_begin + (int)((blockIdx.x + 3u * blockIdx.y) % (unsigned)n_steps);
+            auto next_step = [&](int s) { return s + 1 < s_end ? s + 1 : s_begin; };
+            fetch(s_at);
             // the 26 LDS addresses of a step are recomputed in every step from two values the compiler cannot see through
             // (the vector ALU is idle here, and kept in registers they would cost the fourth workgroup per compute unit)
             int slot_st = st_slot_nt(kn_row, kn_chunk), row_rd = l32;
-            for (int s = s_begin; s < s_end; ++s) {
+            for (int done = 0; done < n_steps; ++done) {
                 asm volatile("" : "+v"(slot_st), "+v"(row_rd));
                 __syncthreads(); // the step (or the pass) before no longer reads the stage
 #pragma unroll
@@ -543,7 +550,8 @@ __global__ __launch_bounds__(FR_THREADS, MB == 1 ? 4 : 3) void fr_tile_kernel(co
 #pragma unroll
                 for (int i = 0; i < 2 * MB; ++i) *(u32x4 *)(s_t + ST_W_BYTES_NT + slot_st + 16 * 256 * i) = xv[i];
                 __syncthreads();
-                if (s + 1 < s_end) fetch(s + 1); // in flight while this step is multiplied
+                s_at = next_step(s_at);
+                if (done + 1 < n_steps) fetch(s_at); // in flight while this step is multiplied
 #pragma unroll
                 for (int kk = 0; kk < 8; ++kk) {
                     const int slot = st_slot_nt(row_rd, 2 * kk + half);
