@@ -441,12 +441,12 @@ __global__ __launch_bounds__(FR_THREADS) void fr_epilogue_kernel(const FwdArgs a
 }
 
 // ------------------------------------------------------------------------------------------------
-// 3 to 64 rows per expert: too many for vector FMAs (one pass over the weights per 4 or 8 rows), too few for the
-// 256 x 256 tiles (one 32 KB stage of weights in flight per compute unit).  A small MFMA tile instead: 32 (or 64) rows of
-// the expert x 128 output columns, operands through registers into 40 (48) KB of LDS, so that four (three) workgroups
-// share a compute unit and keep 80 KB of loads in flight.  One v_mfma_f32_32x32x16 block per wave; lane l holds 16 sums of row l % 32 in
+// 3 to 128 rows per expert: too many for vector FMAs (one pass over the weights per 4 or 8 rows), too few for the
+// 256 x 256 tiles (one 32 KB stage of weights in flight per compute unit).  A small MFMA tile instead: 32 (or 128) rows of
+// the expert x 128 output columns, operands through registers into 40 (64) KB of LDS, so that four (two) workgroups
+// share a compute unit and keep 80 (128) KB of loads in flight.  One v_mfma_f32_32x32x16 block per wave; lane l holds 16 sums of row l % 32 in
 // quads of 4 consecutive columns, so bias, row scale and the epilogues are lane-local, with the arithmetic of
-// tile_epilogue in grouped_gemm.hip.  An expert's rows are taken 32 or 64 at a time.  Every load instruction of a workgroup
+// tile_epilogue in grouped_gemm.hip.  An expert's rows are taken 32 or 128 at a time.  Every load instruction of a workgroup
 // asks for 256 contiguous bytes per row of memory (128-byte pieces of 128 rows of W measured 4.4 TB/s, 256-byte pieces
 // the 5.6 TB/s of a copy):
 //   WT = 0, W[e] as (N, K): K in steps of 128; the W tile is [128 n][128 k] in one LDS stage, read back with ds_read_b128
@@ -468,9 +468,9 @@ __device__ __forceinline__ int st_slot_nt(int row, int chunk) { return row * 256
 
 // EPI = -1: the launch is cut along K (blockIdx.z takes `steps_per` steps) because N alone gives too few workgroups; the
 // fp32 sums go to part[blockIdx.z][M][N] and fr_epilogue_kernel finishes.
-// MB = 32-row blocks of the expert per pass (1 or 2): the weights are streamed once per pass.
+// MB = 32-row blocks of the expert per pass (1 or 4): the weights are streamed once per pass.
 template <typename T, int WT, int EPI, int MB>
-__global__ __launch_bounds__(FR_THREADS, MB == 1 ? 4 : 3) void fr_tile_kernel(const FwdArgs a, float *__restrict__ part, int steps_per) {
+__global__ __launch_bounds__(FR_THREADS, MB == 1 ? 4 : 2) void fr_tile_kernel(const FwdArgs a, float *__restrict__ part, int steps_per) {
     constexpr int X_BYTES = MB * ST_X_BYTES, STAGE = ST_W_BYTES + X_BYTES; // WT = 1, per stage
     __shared__ __attribute__((aligned(16))) unsigned char s_t[WT == 0 ? ST_W_BYTES_NT + 2 * X_BYTES : 2 * STAGE];
     typedef short v4s __attribute__((ext_vector_type(4)));
@@ -683,9 +683,10 @@ template <typename T, int EPI> int fr_launch_epilogue(const FwdArgs &a, const fl
     return xma_check_launch("fr_epilogue_kernel");
 }
 
-// passes of 64 rows once many experts have more than 32 (below that they are 3-15 % slower than passes of 32: three
-// workgroups per compute unit instead of four, by registers and LDS)
-inline int fr_tile_row_blocks(int64_t M, int E) { return M > (int64_t)24 * E ? 2 : 1; }
+// passes of 128 rows once many experts have more than 32: two workgroups per compute unit instead of four (registers
+// and 64 KB of LDS), 3-10 % slower than passes of 32 rows where those suffice; passes of 64 rows and three workgroups were
+// no faster than these anywhere
+inline int fr_tile_row_blocks(int64_t M, int E) { return M > (int64_t)24 * E ? 4 : 1; }
 
 template <typename T, int WT, int EPI, int MB> int fr_launch_tile_mb(const FwdArgs &a, float *part, hipStream_t st) {
     const int S = fr_tile_splits(a.N, a.K, a.E, WT);
@@ -702,7 +703,7 @@ template <typename T, int WT, int EPI, int MB> int fr_launch_tile_mb(const FwdAr
 }
 
 template <typename T, int WT, int EPI> int fr_launch_tile(const FwdArgs &a, float *part, hipStream_t st) {
-    return fr_tile_row_blocks(a.M, a.E) == 2 ? fr_launch_tile_mb<T, WT, EPI, 2>(a, part, st) : fr_launch_tile_mb<T, WT, EPI, 1>(a, part, st);
+    return fr_tile_row_blocks(a.M, a.E) == 4 ? fr_launch_tile_mb<T, WT, EPI, 4>(a, part, st) : fr_launch_tile_mb<T, WT, EPI, 1>(a, part, st);
 }
 
 template <typename T, int EPI> int fr_launch_epi(const FwdArgs &a, int w_is_kn, float *part, hipStream_t st) {

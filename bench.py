@@ -541,8 +541,8 @@ def _other_configs(args) -> dict:
 
 def run_small_t(args):
     """Latency of one forward + backward of the expert computation with a handful of tokens, the case the reference's
-    own test runs (7 tokens, tests/layers/moe_test.py:107) at its two size points (moe_test.py:26-53), and with 64 and
-    192 tokens (decoding batches): eager, and replayed from a HIP graph (no host launch overhead), beside the time the weights touched by the
+    own test runs (7 tokens, tests/layers/moe_test.py:107) at its two size points (moe_test.py:26-53), and with 64,
+    192 and 384 tokens (decoding batches): eager, and replayed from a HIP graph (no host launch overhead), beside the time the weights touched by the
     step need to stream through HBM once per use at 8 TB/s (forward, dX and the dW store: three uses); and the forward
     alone (router, routing, both projections, combine) from a graph, the step of a decoding loop."""
     from xma import KernelBackend, set_seed
@@ -555,7 +555,7 @@ def run_small_t(args):
     for E, k, H, I in ((8, 2, 2048, 8192), (128, 8, 576, 256)):
         set_seed(0)
         moe = MoE(E, k, H, I, swiglu_packed, True, add_bias=False, std=0.02).to(torch.bfloat16).cuda()
-        for T in (7, 64, 192):
+        for T in (7, 64, 192, 384):
             if args.only not in f"E{E}_k{k}_H{H}_I{I}_T{T}":
                 continue
             x = torch.randn(T, H, device="cuda").to(torch.bfloat16).requires_grad_()
@@ -614,7 +614,7 @@ def run_small_t(args):
                       "steps": args.steps, "warmup": args.warmup, "ms_per_step": first["graph_ms"], "higher_is_better": False,
                       "dtype": "bf16", "data": "synthetic",
                       "config": {"workload": "small_t: expert computation fwd+bwd (router top-k from given logits, routing, "
-                                             "experts, combine and all gradients) at T = 7, 64 and 192 on the reference test's two "
+                                             "experts, combine and all gradients) at T = 7, 64, 192 and 384 on the reference test's two "
                                              "size points, bf16 packed SwiGLU"},
                       "results": res}))
 

@@ -104,9 +104,10 @@ def test_few_token_dispatch_rule():
     from xma.rocm import ops
 
     bf = torch.bfloat16
-    assert ops._few_rows(14, 8, bf, "x @ W^T") and ops._few_rows(384, 8, bf, "x @ W^T") and not ops._few_rows(385, 8, bf, "x @ W^T")
+    assert ops._few_rows(14, 8, bf, "x @ W^T") and ops._few_rows(768, 8, bf, "x @ W^T") and not ops._few_rows(769, 8, bf, "x @ W^T")
     assert ops._few_rows(3072, 128, bf, "dy @ W") and not ops._few_rows(16385, 1024, bf, "x @ W^T")  # the cap on the rows
-    assert ops._few_rows(384, 8, bf, "dy @ W") and not ops._few_rows(385, 8, bf, "dy @ W")
+    assert ops._few_rows(768, 8, bf, "dy @ W") and not ops._few_rows(769, 8, bf, "dy @ W")
+    assert ops._few_rows(384, 8, bf, "dy @ W, SwiGLU'") and not ops._few_rows(385, 8, bf, "dy @ W, SwiGLU'")
     assert ops._few_rows(1024, 8, bf, "dW") and not ops._few_rows(1025, 8, bf, "dW")
     assert ops._few_rows(16384, 128, bf, "dW") and not ops._few_rows(16385, 128, bf, "dW")
     assert not ops._few_rows(0, 8, bf, "dW") and not ops._few_rows(14, 8, torch.float32, "dW")
