@@ -373,14 +373,21 @@ __global__ __launch_bounds__(RG_THREADS) void router_gate_topk_kernel(const uint
             for (int b = 0; b < NB; ++b) acc[b] = Elem<T>::mfma(st.xa[q], st.wb[b][q], acc[b]);
     };
     // two stages of operands in registers: the loads of step s + 1 are in flight while step s multiplies
+    // (every workgroup starts its wave's K range at a step of its own and wraps around: workgroups that run together are
+    // at about the same step, and walking from the front they would all ask for the same 128 bytes of every row of x)
     Stage s0, s1;
     const int f_end = s_end < steps_full ? s_end : steps_full;
-    if (s_begin < f_end) fetch(s0, s_begin);
-    for (int step = s_begin; step < f_end; step += 2) {
-        if (step + 1 < f_end) fetch(s1, step + 1);
+    const int cnt = f_end - s_begin, rot = cnt > 0 ? (int)((blockIdx.x * 3u) % (unsigned)cnt) : 0;
+    auto step_of = [&](int i) {
+        const int j = i + rot;
+        return s_begin + (j < cnt ? j : j - cnt);
+    };
+    if (cnt > 0) fetch(s0, step_of(0));
+    for (int i = 0; i < cnt; i += 2) {
+        if (i + 1 < cnt) fetch(s1, step_of(i + 1));
         multiply(s0);
-        if (step + 1 < f_end) {
-            if (step + 2 < f_end) fetch(s0, step + 2);
+        if (i + 1 < cnt) {
+            if (i + 2 < cnt) fetch(s0, step_of(i + 2));
             multiply(s1);
         }
     }
@@ -417,7 +424,8 @@ __global__ __launch_bounds__(RG_THREADS) void router_gate_topk_kernel(const uint
 // The accumulators pass through LDS; the pairs share out the 16 accumulator slots for the selection, which adds the
 // KS partial sums as it reads them.
 constexpr int RL_TOKENS = 64, RL_ROW = 72;
-constexpr int64_t RL_SPLIT_K_BELOW = 24576; // tokens: fewer leave SIMDs of a 256-CU device idle at one wave per 32 tokens
+constexpr int64_t RL_SPLIT_K_BELOW = 98304; // tokens: fewer leave a 256-CU device less than three waves per SIMD at one wave per 32 tokens
+                                            // (with two, one wave's selection tail runs beside the other's K loop)
 
 template <int NB, int KS> constexpr int rl_lds_bytes() { return 2 * KS * NB * 32 * RL_ROW * 2; }
 
@@ -452,14 +460,22 @@ __global__ __launch_bounds__(128 * KS) void router_gate_topk_lds_kernel(const ui
     // used.  Rows of the slice past E re-read row E - 1: their accumulator columns are never looked at.
     const int steps_full = H / 64, per = (steps_full + KS - 1) / KS; // every pair runs `per` rounds of barriers
     const int s_lo = kh * per, my_steps = steps_full - s_lo < per ? (steps_full - s_lo > 0 ? steps_full - s_lo : 0) : per;
+    // Workgroups that run together are at about the same step; with all of them walking K from the front, the requests of
+    // a moment fall on the same 128 bytes of every row of x, a fraction of the memory channels.  Every workgroup starts
+    // at a step of its own and wraps around inside its pair's K range.
+    const int rot = my_steps > 0 ? (int)((blockIdx.x * 3u) % (unsigned)my_steps) : 0;
+    auto step_of = [&](int i) {
+        const int j = i + rot;
+        return s_lo + (j < my_steps ? j : j - my_steps);
+    };
     auto fetch_x = [&](u32x4(&d)[4], int i) {
-        const int k0 = (i < my_steps ? s_lo + i : 0) * 64;
+        const int k0 = (i < my_steps ? step_of(i) : 0) * 64;
 #pragma unroll
         for (int q = 0; q < 4; ++q) d[q] = *(const u32x4 *)(xrow + k0 + 8 * q);
     };
     // chunk c of a slice: expert row c / 8, k offset 8 (c % 8)
     auto fetch_w = [&](u32x4(&d)[W_CHUNKS], int i) {
-        const int k0 = (s_lo + i) * 64;
+        const int k0 = step_of(i) * 64;
 #pragma unroll
         for (int j = 0; j < W_CHUNKS; ++j) {
             const int c = ptid + 128 * j, e = c >> 3;

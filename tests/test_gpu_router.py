@@ -155,11 +155,11 @@ GATE_CASES = [  # T, H, E, k
     (8192, 4096, 8, 2),
     (4133, 1032, 96, 4),
     (2085, 2048, 128, 8),
-    (24613, 136, 40, 3),  # enough tokens for the variant without a K split
+    (98333, 136, 40, 3),  # enough tokens for the variant without a K split
     (8192, 256, 64, 4),  # the gate's weight gradient as a batched GEMM over slices of the tokens
-    (24577, 64, 128, 8),
+    (98305, 64, 128, 8),
     (16384, 2048, 64, 6),  # the two benchmark layers with more than 32 experts, at their exact shapes: two pairs of waves
-    (32768, 2048, 128, 8),  # per workgroup with a K split (below 24576 tokens) and without; 32 K steps through the LDS ring
+    (32768, 2048, 128, 8),  # per workgroup with a K split (below 98304 tokens); 16 K steps per pair through the LDS ring
 ]
 
 
