@@ -667,12 +667,19 @@ inline bool fr_takes_tile(int64_t M, int E, int w_is_kn) {
     return M > (int64_t)(w_is_kn ? FR_NN_VALU_ROWS_PER_EXPERT : FR_NT_VALU_ROWS_PER_EXPERT) * E || M > FR_NT_VALU_ROWS;
 }
 
-// K ranges of the small MFMA tile: enough workgroups for four per compute unit (twice as many measured slower: the
-// partial sums and their kernel cost more than the extra parallelism brings), ranges of at least 512 columns of K
+// passes of 128 rows once many experts have more than 32: two workgroups per compute unit instead of four (registers
+// and 64 KB of LDS), 3-10 % slower than passes of 32 rows where those suffice; passes of 64 rows and three workgroups were
+// no faster than these anywhere
+inline int fr_tile_row_blocks(int64_t M, int E) { return M > (int64_t)24 * E ? 4 : 1; }
+
+// K ranges of the small MFMA tile: enough workgroups for two per compute unit of a 256-CU device, ranges of at least 512
+// columns of K.  Measured (8 experts, 16 rows each, down-projection / dX1 / dX2): 1024 workgroups 61 / 99 / 57 us, 512
+// 52 / 91 / 46, 256 55 / 137 / 46: beyond two per compute unit the partial sums and their kernel cost more than the
+// parallelism brings.
 inline int fr_tile_splits(int N, int K, int E, int w_is_kn) {
     const int64_t wgs = (int64_t)((N + ST_N - 1) / ST_N) * E;
     const int ks = st_k(w_is_kn), steps = (K + ks - 1) / ks, min_steps = 512 / ks;
-    int S = (int)((1024 + wgs - 1) / wgs);
+    int S = (int)((512 + wgs - 1) / wgs);
     if (S > steps / min_steps) S = steps / min_steps;
     return S < 1 ? 1 : S;
 }
@@ -682,11 +689,6 @@ template <typename T, int EPI> int fr_launch_epilogue(const FwdArgs &a, const fl
     fr_epilogue_kernel<T, EPI><<<egrid, FR_THREADS, 0, st>>>(a, part, S);
     return xma_check_launch("fr_epilogue_kernel");
 }
-
-// passes of 128 rows once many experts have more than 32: two workgroups per compute unit instead of four (registers
-// and 64 KB of LDS), 3-10 % slower than passes of 32 rows where those suffice; passes of 64 rows and three workgroups were
-// no faster than these anywhere
-inline int fr_tile_row_blocks(int64_t M, int E) { return M > (int64_t)24 * E ? 4 : 1; }
 
 template <typename T, int WT, int EPI, int MB> int fr_launch_tile_mb(const FwdArgs &a, float *part, hipStream_t st) {
     const int S = fr_tile_splits(a.N, a.K, a.E, WT);

@@ -87,10 +87,9 @@ CONTINUOUS_COUNT_SET_MAX_BINS = 8192
 # cross-overs (8 experts of H = 2048, I = 8192; 64 of H = 2048, I = 1408; 128 of H = 576, I = 256): the forward-type GEMMs
 # walk an expert's rows 32 or 128 at a time (small MFMA tile; vector FMAs up to 2 rows per expert and 64 rows in all, the
 # library decides), each pass streaming the weights again, so they lead while most experts need one pass (at 128 rows
-# per expert on average uneven routing gives enough experts a second pass; dX2 with the SwiGLU backward in its epilogue
-# crosses over earlier); the weight gradient holds a 128 x 128 tile of dW in registers while it walks the rows, so it
-# leads as long as its stores outweigh its loads.
-FEW_ROWS_PER_EXPERT = {"x @ W^T": 96, "dy @ W": 96, "dy @ W, SwiGLU'": 48, "dW": 128}
+# per expert on average uneven routing gives enough experts a second pass); the weight gradient holds a 128 x 128 tile of
+# dW in registers while it walks the rows, so it leads as long as its stores outweigh its loads.
+FEW_ROWS_PER_EXPERT = {"x @ W^T": 96, "dy @ W": 96, "dW": 128}
 FEW_ROWS_MAX = 16384  # rows in all, every form (beyond the measured range; 0 switches the few-token entry points off)
 FEW_ROWS_MAX_WORKSPACE = 256 << 20  # bytes of fp32 partial sums a forward-type launch may ask for
 
@@ -177,8 +176,7 @@ def _few_rows(M: int, E: int, dtype: torch.dtype, form: str) -> bool:
 
 def _few_rows_fwd(lib, M: int, N: int, K: int, E: int, w_is_kn: int, ldw: int, dtype: torch.dtype, epilogue: int) -> bool:
     """the same for a forward-type GEMM, whose few-token entry point has limits of its own"""
-    form = ("dy @ W, SwiGLU'" if epilogue == EPI_SWIGLU_BWD else "dy @ W") if w_is_kn else "x @ W^T"
-    if not _few_rows(M, E, dtype, form) or (w_is_kn and K > FEW_ROWS_NN_MAX_K):
+    if not _few_rows(M, E, dtype, "dy @ W" if w_is_kn else "x @ W^T") or (w_is_kn and K > FEW_ROWS_NN_MAX_K):
         return False
     if not w_is_kn and N * ldw >= FEW_ROWS_NT_MAX_ELEMENTS:  # it addresses the rows of W[e] with 32-bit byte offsets
         return False
