@@ -169,17 +169,17 @@ extern "C" int xma_rocm_group_bwd_W_few_rows(const void *DY, int64_t lddy, int d
 namespace {
 
 // ------------------------------------------------------------------------------------------------
-// Forward-type product for a handful of rows: acc[r][n] = sum_k X[src(r)][k] * B_e[k][n] in fp32, written to a workspace
-// part[S][M][N] as S partial sums over K ranges, then one small kernel that adds the parts in order and runs the epilogue.
-//   W[e] as (N, K), K contiguous (x @ W^T): a wave takes two rows of W at a time, its lanes split K in 16-byte pieces,
-//       the expert's rows of X wait in LDS (2048 columns at a time), and the lanes' partial dot products meet in a butterfly.  S = 1, and for the
-//       STORE and SWIGLU epilogues the wave finishes the job itself: no workspace, no second kernel.
-//   W[e] as (K, N), N contiguous (dy @ W): a thread owns 8 columns n and walks the rows k of its workgroup's K range;
-//       the X values of the range sit in LDS as floats.  S = K / range.
+// Forward-type product for one or two rows per expert, W[e] as (N, K), K contiguous (x @ W^T): acc[r][n] = sum_k
+// X[src(r)][k] * W_e[n][k] in fp32 with vector FMAs.  A wave takes two rows of W at a time, its lanes split K in 16-byte
+// pieces, the expert's rows of X wait in LDS (2048 columns at a time), and the lanes' partial dot products meet in a
+// butterfly.  For the STORE and SWIGLU epilogues the wave finishes the job itself: no workspace, no second kernel;
+// SWIGLU_BWD writes its sums to the workspace part[1][M][N] for fr_epilogue_kernel.  (W[e] as (K, N) had a vector kernel
+// of its own, a thread owning 8 columns and walking the rows k of a K range; the small MFMA tile below beat it at every
+// number of rows once its K ranges were few enough, 82 against 90 us for dX1 with one row per expert.)
 // ------------------------------------------------------------------------------------------------
 constexpr int FR_NT_ROWS = 32;  // rows of W per workgroup (8 per wave, two at a time); 8 when the rows are short
 constexpr int FR_NT_VALU_ROWS_PER_EXPERT = 2; // on average; beyond that x @ W^T takes the small MFMA tile,
-constexpr int FR_NT_VALU_ROWS = 64;             // and beyond this many rows in all (the vector kernels' work per row)
+constexpr int FR_NT_VALU_ROWS = 64;             // and beyond this many rows in all (the vector kernel's work per row)
 constexpr int FR_NT_PIECE = 2048; // elements of K whose X values are staged in LDS at a time (4 rows: 16 KB)
 constexpr int FR_NT_PAIRS = FR_NT_ROWS / 8; // pairs of rows of W per wave
 
@@ -298,85 +298,6 @@ __global__ __launch_bounds__(FR_THREADS, 4) void fr_nt_kernel(const FwdArgs a, f
         fr_nt_rows<T, 2, EPI>(a, part, s_x_nt, e, lo, hi, n_first, n_count);
     else
         fr_nt_rows<T, 4, EPI>(a, part, s_x_nt, e, lo, hi, n_first, n_count);
-}
-
-constexpr int FR_NN_KC_MIN = 32;  // rows k of W per workgroup, at least (four rounds of eight loads per thread)
-constexpr int FR_NN_SPLITS = 64;  // K ranges, at most
-constexpr int FR_NN_KC_MAX = 1024; // 8 rows x range floats in LDS: 32 KB
-
-inline int fr_nn_range(int K) {
-    int kc = (K + FR_NN_SPLITS - 1) / FR_NN_SPLITS;
-    if (kc < FR_NN_KC_MIN) kc = FR_NN_KC_MIN;
-    return kc;
-}
-
-template <typename T, int RC>
-__device__ __forceinline__ void fr_nn_rows(const FwdArgs &a, float *__restrict__ part, float *s_x, int e, int64_t lo,
-                                           int64_t hi, int k_lo, int k_hi, int n_t, bool n_ok) {
-    const int tid = threadIdx.x;
-    const int kc = k_hi - k_lo;
-    const uint16_t *w = a.W + (int64_t)e * a.w_es + (int64_t)k_lo * a.ldw + n_t;
-    for (int64_t r0 = lo; r0 < hi; r0 += RC) {
-        __syncthreads();
-        for (int i = tid; i < RC * kc; i += FR_THREADS) {
-            const int u = i / kc, k = i - u * kc;
-            s_x[i] = (r0 + u < hi) ? fr_scalar<T>(a.X, fr_src_row(a, r0 + u) * a.ldx + k_lo + k) : 0.f;
-        }
-        __syncthreads();
-        float acc[RC][8];
-#pragma unroll
-        for (int u = 0; u < RC; ++u)
-#pragma unroll
-            for (int i = 0; i < 8; ++i) acc[u][i] = 0.f;
-        if (n_ok) {
-            for (int k0 = 0; k0 < kc; k0 += 8) { // eight rows of W in flight per thread
-                u32x4 wv[8];
-#pragma unroll
-                for (int q = 0; q < 8; ++q) {
-                    wv[q] = u32x4{0u, 0u, 0u, 0u};
-                    if (k0 + q < kc) wv[q] = __builtin_nontemporal_load((const u32x4 *)(w + (int64_t)(k0 + q) * a.ldw));
-                }
-#pragma unroll
-                for (int q = 0; q < 8; ++q) {
-                    if (k0 + q < kc) {
-                        float fw[8];
-                        fr_unpack<T>(wv[q], fw);
-#pragma unroll
-                        for (int u = 0; u < RC; ++u) {
-                            const float xv = s_x[u * kc + k0 + q];
-#pragma unroll
-                            for (int i = 0; i < 8; ++i) acc[u][i] = __builtin_fmaf(xv, fw[i], acc[u][i]);
-                        }
-                    }
-                }
-            }
-#pragma unroll
-            for (int u = 0; u < RC; ++u) {
-                if (r0 + u < hi) {
-                    float4 *o = (float4 *)(part + (r0 + u) * a.N + n_t);
-                    o[0] = make_float4(acc[u][0], acc[u][1], acc[u][2], acc[u][3]);
-                    o[1] = make_float4(acc[u][4], acc[u][5], acc[u][6], acc[u][7]);
-                }
-            }
-        }
-    }
-}
-
-template <typename T>
-__global__ __launch_bounds__(FR_THREADS) void fr_nn_kernel(const FwdArgs a, float *__restrict__ part, int kc) {
-    extern __shared__ __attribute__((aligned(16))) float s_x_nn[];
-    const int e = blockIdx.z, split = blockIdx.y;
-    const int64_t lo = e ? a.offs[e - 1] : 0, hi = a.offs[e];
-    if (lo >= hi) return; // uniform
-    const int k_lo = split * kc, k_hi = (k_lo + kc < a.K) ? k_lo + kc : a.K;
-    const int n_t = (blockIdx.x * FR_THREADS + threadIdx.x) * 8;
-    float *mine = part + (int64_t)split * a.M * a.N;
-    if (hi - lo <= 2)
-        fr_nn_rows<T, 2>(a, mine, s_x_nn, e, lo, hi, k_lo, k_hi, n_t, n_t < a.N);
-    else if (hi - lo <= 4)
-        fr_nn_rows<T, 4>(a, mine, s_x_nn, e, lo, hi, k_lo, k_hi, n_t, n_t < a.N);
-    else
-        fr_nn_rows<T, 8>(a, mine, s_x_nn, e, lo, hi, k_lo, k_hi, n_t, n_t < a.N);
 }
 
 // One workgroup per row and 512 columns: the S parts are added in order, the bias joins, and the epilogue of the MFMA kernels is applied
@@ -661,10 +582,9 @@ __global__ __launch_bounds__(FR_THREADS, MB == 1 ? 4 : 2) void fr_tile_kernel(co
     }
 }
 
-// more than a pass or two of the vector kernels per expert -> the small MFMA tile
-constexpr int FR_NN_VALU_ROWS_PER_EXPERT = 2;
+// W[e] as (K, N), or more than a pass or two of the vector kernel per expert -> the small MFMA tile
 inline bool fr_takes_tile(int64_t M, int E, int w_is_kn) {
-    return M > (int64_t)(w_is_kn ? FR_NN_VALU_ROWS_PER_EXPERT : FR_NT_VALU_ROWS_PER_EXPERT) * E || M > FR_NT_VALU_ROWS;
+    return w_is_kn || M > (int64_t)FR_NT_VALU_ROWS_PER_EXPERT * E || M > FR_NT_VALU_ROWS;
 }
 
 // passes of 128 rows once many experts have more than 32: two workgroups per compute unit instead of four (registers
@@ -711,13 +631,6 @@ template <typename T, int WT, int EPI> int fr_launch_tile(const FwdArgs &a, floa
 template <typename T, int EPI> int fr_launch_epi(const FwdArgs &a, int w_is_kn, float *part, hipStream_t st) {
     int rc;
     if (fr_takes_tile(a.M, a.E, w_is_kn)) return w_is_kn ? fr_launch_tile<T, 1, EPI>(a, part, st) : fr_launch_tile<T, 0, EPI>(a, part, st);
-    if (w_is_kn) {
-        const int kc = fr_nn_range(a.K), S = (a.K + kc - 1) / kc;
-        const dim3 grid((a.N / 8 + FR_THREADS - 1) / FR_THREADS, S, a.E);
-        fr_nn_kernel<T><<<grid, FR_THREADS, (size_t)8 * kc * sizeof(float), st>>>(a, part, kc);
-        if ((rc = xma_check_launch("fr_nn_kernel"))) return rc;
-        return fr_launch_epilogue<T, EPI>(a, part, S, st);
-    }
     // one pair of rows per wave instead of four where the rows are short or the launch would have few workgroups
     const int rows_per_wg = (a.K >= 2048 && (int64_t)(a.N / FR_NT_ROWS) * a.E >= 2048) ? FR_NT_ROWS : 8;
     const dim3 grid((a.N + rows_per_wg - 1) / rows_per_wg, a.E);
@@ -746,9 +659,6 @@ extern "C" size_t xma_rocm_scatter2scatter_few_rows_workspace_bytes(int64_t M, i
     if (fr_takes_tile(M, E, w_is_kn)) { // the small MFMA tile, cut along K or not
         S = fr_tile_splits(N, K, E, w_is_kn);
         if (S == 1) return 0;
-    } else if (w_is_kn) { // partial sums of the K ranges
-        const int kc = fr_nn_range(K);
-        S = (K + kc - 1) / kc;
     } else if (epilogue == XMA_ROCM_EPI_SWIGLU_BWD) {
         S = 1; // the vector kernel's sums go to the epilogue kernel
     } else {
@@ -772,8 +682,6 @@ extern "C" int xma_rocm_scatter2scatter_few_rows(const void *X, int64_t ldx, con
                 "scatter2scatter_few_rows: M=%lld N=%d K=%d E=%d fan_out=%d (M and E at most 65535)", (long long)M, N, K, E, fan_out);
     XMA_REQUIRE(N % 8 == 0 && K % 8 == 0 && ldx % 8 == 0 && ldw % 8 == 0 && ldo % 8 == 0 && w_expert_stride % 8 == 0,
                 XMA_ROCM_EUNSUPPORTED, "scatter2scatter_few_rows: N=%d K=%d and the leading dimensions must be multiples of 8", N, K);
-    XMA_REQUIRE(!w_is_kn || fr_nn_range(K) <= FR_NN_KC_MAX, XMA_ROCM_EUNSUPPORTED,
-                "scatter2scatter_few_rows: K=%d exceeds %d for W as (K, N)", K, FR_NN_KC_MAX * FR_NN_SPLITS);
     XMA_REQUIRE(w_is_kn || (int64_t)N * ldw < ((int64_t)1 << 31) - 128, XMA_ROCM_EUNSUPPORTED,
                 "scatter2scatter_few_rows: N * ldw = %lld exceeds 2^31 - 128 elements for W as (N, K)", (long long)N * (long long)ldw);
     if (M == 0) return XMA_ROCM_OK;

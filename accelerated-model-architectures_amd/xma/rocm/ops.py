@@ -165,8 +165,7 @@ def scatter2scatter_workspace_bytes(M: int, N: int, K: int, E: int, device_index
     return _S2S_WORKSPACE_BYTES[key]
 
 
-FEW_ROWS_NN_MAX_K = 65536  # limit of the few-token entry point for W as (K, N)
-FEW_ROWS_NT_MAX_ELEMENTS = (1 << 31) - 128  # and for W as (N, K): N * ldw
+FEW_ROWS_NT_MAX_ELEMENTS = (1 << 31) - 128  # limit of the few-token entry point for W as (N, K): N * ldw
 
 
 def _few_rows(M: int, E: int, dtype: torch.dtype, form: str) -> bool:
@@ -176,7 +175,7 @@ def _few_rows(M: int, E: int, dtype: torch.dtype, form: str) -> bool:
 
 def _few_rows_fwd(lib, M: int, N: int, K: int, E: int, w_is_kn: int, ldw: int, dtype: torch.dtype, epilogue: int) -> bool:
     """the same for a forward-type GEMM, whose few-token entry point has limits of its own"""
-    if not _few_rows(M, E, dtype, "dy @ W" if w_is_kn else "x @ W^T") or (w_is_kn and K > FEW_ROWS_NN_MAX_K):
+    if not _few_rows(M, E, dtype, "dy @ W" if w_is_kn else "x @ W^T"):
         return False
     if not w_is_kn and N * ldw >= FEW_ROWS_NT_MAX_ELEMENTS:  # it addresses the rows of W[e] with 32-bit byte offsets
         return False

@@ -67,12 +67,12 @@ def test_argument_errors_are_reported_before_any_launch():
     assert lib.xma_rocm_router_topk_bwd(None, 8, 4, 8, 2, 0, None, 1, None, None, 4, None) == -1  # ldd < E
     assert lib.xma_rocm_router_topk(None, 8, 0, 8, 2, 0, None, None, 1, None) == 0
     # the few-token entry points: dtype (no fp32), M beyond the epilogue's grid, a missing workspace where sums go through
-    # one (W as (K, N)), none needed for W as (N, K) with a plain store (fails later, on the null operands), dW shapes
+    # one (few column blocks and a long K: the launch is cut along K), none needed for W as (N, K) with a plain store (fails later, on the null operands), dW shapes
     p = ctypes.c_void_p(256)
     few = lib.xma_rocm_scatter2scatter_few_rows
     assert few(p, 64, p, 64 * 64, 64, 0, p, p, p, 64, None, 0, None, 0, None, None, 0, 4, 64, 64, 2, 1, 1, 1, 0, 2, None, 0, None) == -2
     assert few(p, 64, p, 64 * 64, 64, 0, p, p, p, 64, None, 0, None, 0, None, None, 0, 70000, 64, 64, 2, 1, 1, 1, 0, 0, None, 0, None) == -1
-    assert few(p, 64, p, 64 * 64, 64, 1, p, p, p, 64, None, 0, None, 0, None, None, 0, 4, 64, 64, 2, 1, 1, 1, 0, 0, None, 0, None) == -3
+    assert few(p, 16384, p, 16384 * 64, 64, 1, p, p, p, 64, None, 0, None, 0, None, None, 0, 4, 64, 16384, 2, 1, 1, 1, 0, 0, None, 0, None) == -3
     assert b"workspace" in lib.xma_rocm_last_error()
     assert few(None, 64, None, 64 * 64, 64, 0, p, p, p, 64, None, 0, None, 0, None, None, 0, 4, 64, 64, 2, 1, 1, 1, 0, 0, None, 0, None) == -1
     assert b"null or misaligned" in lib.xma_rocm_last_error()
@@ -82,7 +82,7 @@ def test_argument_errors_are_reported_before_any_launch():
     ws = lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes  # (M, N, K, E, w_is_kn, epilogue)
     assert ws(4, 64, 64, 2, 0, 0) == 0 and ws(4, 64, 64, 2, 0, 1) == 0  # the vector kernel finishes the job itself (2 rows per expert)
     assert ws(4, 64, 64, 2, 0, 2) == 4 * 64 * 4  # SwiGLU backward: through the epilogue kernel
-    assert ws(4, 64, 16384, 2, 1, 0) == 64 * 4 * 64 * 4  # W as (K, N): 64 ranges of K
+    assert ws(4, 64, 16384, 2, 1, 0) == 32 * 4 * 64 * 4  # W as (K, N): the small tile at any number of rows, 32 ranges of K
     assert ws(64, 2048, 16384, 8, 1, 0) == 4 * 64 * 2048 * 4 and ws(64, 8192, 2048, 8, 1, 2) == 0  # small tile: 4 ranges of K; none
     assert ws(64, 16384, 2048, 8, 0, 1) == 0  # small MFMA tile, enough workgroups from N alone
     assert ws(64, 2048, 8192, 8, 0, 0) == 4 * 64 * 2048 * 4  # small MFMA tile cut into 4 ranges of K
