@@ -404,6 +404,7 @@ __global__ __launch_bounds__(FR_THREADS, MB == 1 ? 4 : 2) void fr_tile_kernel(co
     const int steps_all = (a.K + st_k(WT) - 1) / st_k(WT);
     const int s_begin = (EPI < 0) ? blockIdx.z * steps_per : 0;
     const int s_end = (EPI < 0 && s_begin + steps_per < steps_all) ? s_begin + steps_per : steps_all;
+    if (s_begin >= s_end) return; // uniform; the host launches no empty range
     // loaders.  WT = 0: thread = (row tid / 16 + 16 i, 16-byte chunk tid % 16 of the step's 128 k) for both tiles, rows of W
     // past N clamped (computed, never stored).  WT = 1: W thread = (k-row tid / 16 + 16 i, 16-byte chunk tid % 16 of the 128
     // columns), X thread = (row tid / 8, chunk tid % 8 of the step's 64 k)
@@ -611,8 +612,9 @@ template <typename T, int EPI> int fr_launch_epilogue(const FwdArgs &a, const fl
 }
 
 template <typename T, int WT, int EPI, int MB> int fr_launch_tile_mb(const FwdArgs &a, float *part, hipStream_t st) {
-    const int S = fr_tile_splits(a.N, a.K, a.E, WT);
-    const int steps_all = (a.K + st_k(WT) - 1) / st_k(WT), steps_per = (steps_all + S - 1) / S;
+    const int S_max = fr_tile_splits(a.N, a.K, a.E, WT);
+    const int steps_all = (a.K + st_k(WT) - 1) / st_k(WT), steps_per = (steps_all + S_max - 1) / S_max;
+    const int S = (steps_all + steps_per - 1) / steps_per; // ranges that hold a step (25 steps in 6 ranges of 5: only 5 do)
     const dim3 grid((a.N + ST_N - 1) / ST_N, a.E, S);
     if (S == 1) {
         fr_tile_kernel<T, WT, EPI, MB><<<grid, FR_THREADS, 0, st>>>(a, nullptr, steps_all);
@@ -621,7 +623,7 @@ template <typename T, int WT, int EPI, int MB> int fr_launch_tile_mb(const FwdAr
     fr_tile_kernel<T, WT, -1, MB><<<grid, FR_THREADS, 0, st>>>(a, part, steps_per);
     int rc = xma_check_launch("fr_tile_kernel");
     if (rc) return rc;
-    return fr_launch_epilogue<T, EPI>(a, part, (steps_all + steps_per - 1) / steps_per, st);
+    return fr_launch_epilogue<T, EPI>(a, part, S, st);
 }
 
 template <typename T, int WT, int EPI> int fr_launch_tile(const FwdArgs &a, float *part, hipStream_t st) {

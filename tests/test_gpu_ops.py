@@ -340,7 +340,8 @@ FEW_ROWS_CASES = [
     (16, 4, 4, 2048, 72, (2,)),  # about twenty rows per expert: several passes of 4 or 8 rows over the weights
     (1, 8, 1, 64, 8, ()),
     (9, 5, 3, 4104, 24, (0, 4)),  # a row of W as (N, K) is 513 pieces of 16 bytes: two passes of a wave and one lane more
-    (7, 8, 2, 512, 8192, ()),  # K = 8192 for the down-projection (64 KB of LDS), 128 K ranges of 128 for dX1
+    (7, 8, 2, 512, 8192, ()),  # long K for the down-projection and dX1: both cut into ranges of K
+    (5, 2, 2, 64, 3200, ()),  # down-projection: 25 K steps in 6 ranges of 5, of which only 5 hold a step
 ]
 
 
