@@ -20,35 +20,43 @@ template <typename T> __device__ __forceinline__ void fr_unpack(const u32x4 v, f
 
 // DW[e][n][k] = sum over the rows r of expert e of DY[dsrc(r)][n] * scale[idx[r]] * X[xsrc(r)][k]: MFMAs whose K dimension is
 // the expert's rows, 32 at a time, zeros beyond the last.  With few rows the launch is its stores (a vector-FMA version, a
-// thread owning 8 k of 8 rows n, was as fast up to 8 rows per expert and three times slower at 32).  Workgroup = a 128 x 128 tile of DW[e] (32 KB of stores) for (k block, n block, expert); both operand tiles are [32 rows][128
-// columns] as they lie in memory, and ds_read_b64_tr_b16 hands a lane 4 consecutive rows of one column (st_slot_kn and the
-// fragment offsets of fr_tile_kernel below).  Wave w owns the 32 rows n of block w and all 128 columns k: 4 accumulator blocks,
-// where lane l holds row n = l % 32 and quads of 4 consecutive k.  The tile leaves through LDS as whole 256-byte rows,
-// 16 bytes per lane.  Any number of rows (more passes), every element written exactly once, zeros for an expert without rows.
-constexpr int DT_TILE = 128, DT_ROWS = 32, DT_OPERAND = DT_ROWS * DT_TILE * 2;
+// thread owning 8 k of 8 rows n, was as fast up to 8 rows per expert and three times slower at 32).  Workgroup = a TN x TK
+// tile of DW[e] (32 KB of stores) for (k block, n block, expert); the operand tiles are [32 rows][columns] as they lie in
+// memory, and ds_read_b64_tr_b16 hands a lane 4 consecutive rows of one column (st_slot_kn and the fragment offsets of
+// fr_tile_kernel below).  A wave owns one block of 32 rows n and four blocks of 32 columns k: 4 accumulator blocks, where
+// lane l holds row n = l % 32 and quads of 4 consecutive k.  The tile leaves through LDS as whole rows, 16 bytes per lane.
+// Any number of rows (more passes), every element written exactly once, zeros for an expert without rows.
+constexpr int DT_ROWS = 32, DT_OPERAND = DT_ROWS * 128 * 2; // rows of a pass; bytes of the dY tile [32][128]
+constexpr int DW_WIDE_ROWS_PER_EXPERT = 24;              // on average: up to here the 64 x 256 tile
 // 16-byte slot of (k-row, chunk) in a tile of 256-byte rows that is read down its columns: chunk c of k-row kr sits at
 // c ^ ((kr & 3) << 2)
 __device__ __forceinline__ int st_slot_kn(int kr, int chunk) { return kr * 256 + ((chunk ^ ((kr & 3) << 2)) << 4); }
 
-template <typename T> __global__ __launch_bounds__(FR_THREADS, 4) void dw_tile_kernel(const DwArgs a) {
-    __shared__ __attribute__((aligned(16))) unsigned char s_t[DT_TILE * DT_TILE * 2]; // the operand tiles (2 x 8 KB), then the output tile
+template <typename T, int TN, int TK> __global__ __launch_bounds__(FR_THREADS, 4) void dw_tile_kernel(const DwArgs a) {
+    // TN x TK = 16384: TN rows n of DW[e] x TK columns k per workgroup; dY tile [32 rows][128 columns, TN used], X tile
+    // [32 rows][TK columns], then the output tile [TN][TK] in their place
+    static_assert(TN * TK == 16384 && TN >= 32 && TK >= 128, "a wave owns 4 blocks of 32 x 32");
+    // 64 x 256 (512-byte rows out: 87 / 45 instead of 98 / 50 us for dW1 / dW2 of 8 experts of H = 2048, I = 8192) while a
+    // pass or two cover an expert; 128 x 128 beyond, whose pass reads 16 KB of operands instead of 20 (32 x 512: the eight
+    // gathered rows per thread spill, twice the time)
+    constexpr int XROW = 2 * TK, XCH = TK / 8, DYCH = TN / 8, NBN = TN / 32; // bytes and 16-byte chunks per tile row, n blocks
+    constexpr int OPERANDS = DT_OPERAND + DT_ROWS * XROW, OUT = TN * TK * 2;
+    __shared__ __attribute__((aligned(16))) unsigned char s_t[OPERANDS > OUT ? OPERANDS : OUT];
     typedef short v4s __attribute__((ext_vector_type(4)));
     typedef __attribute__((address_space(3))) v4s *lds_v4s;
     const int e = blockIdx.z, tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, half = lane >> 5, l32 = lane & 31;
-    const int k0 = blockIdx.x * DT_TILE, n0 = blockIdx.y * DT_TILE;
+    const int k0 = blockIdx.x * TK, n0 = blockIdx.y * TN;
     const int64_t lo = e ? a.offs[e - 1] : 0, hi = a.offs[e];
-    // loader and storer: thread = (row tid / 16 + 16 i, 16-byte chunk tid % 16 of the 128 columns)
-    const int ld_row = tid >> 4, ld_chunk = tid & 15;
-    const bool dy_ok = n0 + 8 * ld_chunk < a.N_out, x_ok = k0 + 8 * ld_chunk < a.K_in; // multiples of 8: a chunk is inside or outside
-    // this lane's fragment of column block `blk` of an operand tile, rows 0-3 of its 8 (the other 4: + 1024, rows + 16: + 4096)
+    const int nb = wave % NBN, kb0 = (wave / NBN) * 4; // this wave's n block and its four k blocks
+    // this lane's fragment of column block `blk` of an operand tile, rows 0-3 of its 8 (the other 4: 4 rows on, rows + 16: 16 rows on)
     const int p = lane & 15, G = lane >> 4, kr = ((G >> 1) << 3) + (p >> 2), m_in = ((G & 1) << 4) + ((p & 3) << 2);
-    auto frag_off = [&](int blk) {
+    auto frag_off = [&](int blk, int row_bytes) {
         const int m = blk * 32 + m_in;
-        return kr * 256 + (((m >> 3) ^ ((kr & 3) << 2)) << 4) + ((m & 7) << 1);
+        return kr * row_bytes + (((m >> 3) ^ ((kr & 3) << 2)) << 4) + ((m & 7) << 1);
     };
-    auto frag = [&](const unsigned char *at) {
+    auto frag = [&](const unsigned char *at, int row_bytes) {
         const v4s r03 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)at);
-        const v4s r47 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(at + 1024));
+        const v4s r47 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_v4s)(at + 4 * row_bytes));
         const u32x2 a01 = __builtin_bit_cast(u32x2, r03), a23 = __builtin_bit_cast(u32x2, r47);
         return u32x4{a01[0], a01[1], a23[0], a23[1]};
     };
@@ -57,63 +65,74 @@ template <typename T> __global__ __launch_bounds__(FR_THREADS, 4) void dw_tile_k
     for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int i = 0; i < 16; ++i) acc[j][i] = 0.f;
+    constexpr int DY_IT = (DT_ROWS * DYCH + FR_THREADS - 1) / FR_THREADS, X_IT = DT_ROWS * XCH / FR_THREADS;
     for (int64_t r0 = lo; r0 < hi; r0 += DT_ROWS) {
-        u32x4 dyv[2], xv[2];
+        u32x4 dyv[DY_IT], xv[X_IT];
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const int64_t r = r0 + ld_row + 16 * i;
-            dyv[i] = xv[i] = u32x4{0u, 0u, 0u, 0u}; // rows past the expert's last add nothing
-            if (r < hi) {
+        for (int i = 0; i < DY_IT; ++i) { // chunk c of the dY tile: row c / DYCH, 16-byte chunk c % DYCH
+            const int c = tid + FR_THREADS * i, row = c / DYCH, ch = c % DYCH;
+            const int64_t r = r0 + row;
+            dyv[i] = u32x4{0u, 0u, 0u, 0u}; // rows past the expert's last add nothing
+            if (row < DT_ROWS && r < hi && n0 + 8 * ch < a.N_out) {
                 const int64_t s = a.idx ? a.idx[r] : r;
-                if (dy_ok) {
-                    const int64_t src = a.dy_grouped ? r : (int64_t)fastdiv((uint32_t)s, a.dy_div);
-                    dyv[i] = *(const u32x4 *)(a.DY + src * a.lddy + n0 + 8 * ld_chunk);
-                    if (a.scale) { // the scaled row rounded to the operand type, as a scaled grouped copy of dY would hold it
-                        const float sc = fr_scalar<T>(a.scale, s);
-                        float f[8];
-                        fr_unpack<T>(dyv[i], f);
+                const int64_t src = a.dy_grouped ? r : (int64_t)fastdiv((uint32_t)s, a.dy_div);
+                dyv[i] = *(const u32x4 *)(a.DY + src * a.lddy + n0 + 8 * ch);
+                if (a.scale) { // the scaled row rounded to the operand type, as a scaled grouped copy of dY would hold it
+                    const float sc = fr_scalar<T>(a.scale, s);
+                    float f[8];
+                    fr_unpack<T>(dyv[i], f);
 #pragma unroll
-                        for (int q = 0; q < 4; ++q) dyv[i][q] = Elem<T>::pack(f[2 * q] * sc, f[2 * q + 1] * sc);
-                    }
+                    for (int q = 0; q < 4; ++q) dyv[i][q] = Elem<T>::pack(f[2 * q] * sc, f[2 * q + 1] * sc);
                 }
-                if (x_ok) {
-                    const int64_t src = a.x_grouped ? r : (int64_t)fastdiv((uint32_t)s, a.x_div);
-                    xv[i] = *(const u32x4 *)(a.X + src * a.ldx + k0 + 8 * ld_chunk);
-                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < X_IT; ++i) {
+            const int c = tid + FR_THREADS * i, row = c / XCH, ch = c % XCH;
+            const int64_t r = r0 + row;
+            xv[i] = u32x4{0u, 0u, 0u, 0u};
+            if (r < hi && k0 + 8 * ch < a.K_in) {
+                const int64_t src = a.x_grouped ? r : (int64_t)fastdiv((uint32_t)a.idx[r], a.x_div);
+                xv[i] = *(const u32x4 *)(a.X + src * a.ldx + k0 + 8 * ch);
             }
         }
         __syncthreads(); // the pass before no longer reads the tiles
 #pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            *(u32x4 *)(s_t + st_slot_kn(ld_row + 16 * i, ld_chunk)) = dyv[i];
-            *(u32x4 *)(s_t + DT_OPERAND + st_slot_kn(ld_row + 16 * i, ld_chunk)) = xv[i];
+        for (int i = 0; i < DY_IT; ++i) {
+            const int c = tid + FR_THREADS * i, row = c / DYCH, ch = c % DYCH;
+            if (row < DT_ROWS) *(u32x4 *)(s_t + st_slot_kn(row, ch)) = dyv[i];
+        }
+#pragma unroll
+        for (int i = 0; i < X_IT; ++i) {
+            const int c = tid + FR_THREADS * i, row = c / XCH, ch = c % XCH;
+            *(u32x4 *)(s_t + DT_OPERAND + row * XROW + ((ch ^ ((row & 3) << 2)) << 4)) = xv[i];
         }
         __syncthreads();
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
-            const u32x4 dy_f = frag(s_t + frag_off(wave) + kk * 4096);
+            const u32x4 dy_f = frag(s_t + frag_off(nb, 256) + kk * 16 * 256, 256);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) acc[j] = Elem<T>::mfma(frag(s_t + DT_OPERAND + frag_off(j) + kk * 4096), dy_f, acc[j]);
+            for (int j = 0; j < 4; ++j)
+                acc[j] = Elem<T>::mfma(frag(s_t + DT_OPERAND + frag_off(kb0 + j, XROW) + kk * 16 * XROW, XROW), dy_f, acc[j]);
         }
     }
     __syncthreads(); // the operand tiles are done with: the output tile takes their place
-    // acc[j][4 g + q] = DW[n0 + 32 wave + l32][k0 + 32 j + 8 g + 4 half + q]; the 16-byte chunk c of row n sits at c ^ (n % 16)
-    const int n_l = wave * 32 + l32;
+    // acc[j][4 g + q] = DW[n0 + 32 nb + l32][k0 + 32 (kb0 + j) + 8 g + 4 half + q]; the 16-byte chunk c of row n sits at c ^ (n % 16)
+    const int n_l = nb * 32 + l32;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
         for (int g = 0; g < 4; ++g)
-            *(u32x2 *)(s_t + n_l * 256 + (((4 * j + g) ^ (n_l & 15)) << 4) + 8 * half) =
+            *(u32x2 *)(s_t + n_l * XROW + (((4 * (kb0 + j) + g) ^ (n_l & 15)) << 4) + 8 * half) =
                 u32x2{Elem<T>::pack(acc[j][4 * g], acc[j][4 * g + 1]), Elem<T>::pack(acc[j][4 * g + 2], acc[j][4 * g + 3])};
     __syncthreads();
-    if (!x_ok) return;
-    uint16_t *out = a.DW + (int64_t)e * a.dw_es + k0 + 8 * ld_chunk;
+    uint16_t *out = a.DW + (int64_t)e * a.dw_es + k0;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int row = ld_row + 16 * i;
-        if (n0 + row < a.N_out)
-            __builtin_nontemporal_store(*(const u32x4 *)(s_t + row * 256 + ((ld_chunk ^ (row & 15)) << 4)),
-                                        (u32x4 *)(out + (int64_t)(n0 + row) * a.lddw));
+    for (int i = 0; i < 8; ++i) { // whole rows of the tile out: XCH lanes side by side per row
+        const int c = tid + FR_THREADS * i, row = c / XCH, ch = c % XCH;
+        if (n0 + row < a.N_out && k0 + 8 * ch < a.K_in)
+            __builtin_nontemporal_store(*(const u32x4 *)(s_t + row * XROW + ((ch ^ (row & 15)) << 4)),
+                                        (u32x4 *)(out + (int64_t)(n0 + row) * a.lddw + 8 * ch));
     }
 }
 
@@ -123,7 +142,7 @@ extern "C" int xma_rocm_group_bwd_W_few_rows(const void *DY, int64_t lddy, int d
                                              const void *dy_scale, const void *X, int64_t ldx, int x_grouped,
                                              int32_t x_fan_out, const int64_t *sorted_scattered_idxs,
                                              const int64_t *expert_offsets, void *DW, int64_t dw_expert_stride, int64_t lddw,
-                                             int32_t N_out, int32_t K_in, int32_t E, int dtype, void *stream) {
+                                             int32_t N_out, int32_t K_in, int32_t E, int64_t M, int dtype, void *stream) {
     XMA_REQUIRE(dtype == XMA_ROCM_BF16 || dtype == XMA_ROCM_F16, XMA_ROCM_EUNSUPPORTED, "group_bwd_W_few_rows: dtype %d", dtype);
     XMA_REQUIRE(N_out >= 8 && K_in >= 8 && E >= 1 && E <= 65535 && dy_fan_out >= 1 && x_fan_out >= 1, XMA_ROCM_EINVAL,
                 "group_bwd_W_few_rows: N_out=%d K_in=%d E=%d", N_out, K_in, E);
@@ -135,8 +154,7 @@ extern "C" int xma_rocm_group_bwd_W_few_rows(const void *DY, int64_t lddy, int d
                 "group_bwd_W_few_rows: null or misaligned operand");
     XMA_REQUIRE(sorted_scattered_idxs || (dy_grouped && x_grouped && !dy_scale), XMA_ROCM_EINVAL,
                 "group_bwd_W_few_rows: sorted_scattered_idxs is required unless everything is grouped");
-    XMA_REQUIRE((N_out + DT_TILE - 1) / DT_TILE <= 65535, XMA_ROCM_EUNSUPPORTED, "group_bwd_W_few_rows: N_out=%d exceeds %d", N_out,
-                65535 * DT_TILE);
+    XMA_REQUIRE((N_out + 31) / 32 <= 65535, XMA_ROCM_EUNSUPPORTED, "group_bwd_W_few_rows: N_out=%d exceeds %d", N_out, 65535 * 32);
     DwArgs a;
     a.DY = (const uint16_t *)DY;
     a.lddy = lddy;
@@ -158,11 +176,20 @@ extern "C" int xma_rocm_group_bwd_W_few_rows(const void *DY, int64_t lddy, int d
     a.dy_div = make_fastdiv((uint32_t)dy_fan_out);
     a.x_div = make_fastdiv((uint32_t)x_fan_out);
     hipStream_t st = (hipStream_t)stream;
-    const dim3 grid((K_in + DT_TILE - 1) / DT_TILE, (N_out + DT_TILE - 1) / DT_TILE, E);
-    if (dtype == XMA_ROCM_BF16)
-        dw_tile_kernel<__bf16><<<grid, FR_THREADS, 0, st>>>(a);
-    else
-        dw_tile_kernel<_Float16><<<grid, FR_THREADS, 0, st>>>(a);
+    const bool wide = M > 0 && M <= (int64_t)DW_WIDE_ROWS_PER_EXPERT * E;
+    const int TN = wide ? 64 : 128, TK = 16384 / TN;
+    const dim3 grid((K_in + TK - 1) / TK, (N_out + TN - 1) / TN, E);
+    if (dtype == XMA_ROCM_BF16) {
+        if (wide)
+            dw_tile_kernel<__bf16, 64, 256><<<grid, FR_THREADS, 0, st>>>(a);
+        else
+            dw_tile_kernel<__bf16, 128, 128><<<grid, FR_THREADS, 0, st>>>(a);
+    } else {
+        if (wide)
+            dw_tile_kernel<_Float16, 64, 256><<<grid, FR_THREADS, 0, st>>>(a);
+        else
+            dw_tile_kernel<_Float16, 128, 128><<<grid, FR_THREADS, 0, st>>>(a);
+    }
     return xma_check_launch("dw_tile_kernel");
 }
 

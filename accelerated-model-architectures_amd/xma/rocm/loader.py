@@ -67,7 +67,7 @@ SIGNATURES = {
     ),
     "xma_rocm_group_bwd_W_few_rows": (
         _int,
-        [_p, _i64, _int, _i32, _p, _p, _i64, _int, _i32, _p, _p, _p, _i64, _i64, _i32, _i32, _i32, _int, _p],
+        [_p, _i64, _int, _i32, _p, _p, _i64, _int, _i32, _p, _p, _p, _i64, _i64, _i32, _i32, _i32, _i64, _int, _p],
     ),
     "xma_rocm_group": (_int, [_p, _i64, _p, _p, _i64, _p, _i64, _i32, _i32, _int, _p]),
     "xma_rocm_combine": (_int, [_p, _i64, _p, _p, _i64, _i64, _i32, _i32, _int, _p]),

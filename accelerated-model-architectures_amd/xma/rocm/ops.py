@@ -355,17 +355,16 @@ def group_bwd_W_rocm(
         assert dy_scale.dtype == DY.dtype and dy_scale.is_contiguous()
     lib = get_library()
     # a handful of rows per expert (the index has one entry per row): the launch is a stream of stores, not arithmetic
-    few = _few_rows(sorted_scattered_idxs.numel(), E, DW.dtype, "dW")
+    M = sorted_scattered_idxs.numel()
+    few = _few_rows(M, E, DW.dtype, "dW")
     name = "xma_rocm_group_bwd_W_few_rows" if few else "xma_rocm_group_bwd_W"
-    check(
-        getattr(lib, name)(
-            _ptr(DY), _rows(DY, "DY"), int(dy_fan_out == 0), max(dy_fan_out, 1), _ptr(dy_scale),
-            _ptr(X), _rows(X, "X"), int(x_fan_out == 0), max(x_fan_out, 1),
-            _ptr(sorted_scattered_idxs), _ptr(expert_offsets), _ptr(DW), DW.stride(0), DW.stride(2),
-            N_out, K_in, E, _code(X), _stream(X),
-        ),
-        name,
+    operands = (
+        _ptr(DY), _rows(DY, "DY"), int(dy_fan_out == 0), max(dy_fan_out, 1), _ptr(dy_scale),
+        _ptr(X), _rows(X, "X"), int(x_fan_out == 0), max(x_fan_out, 1),
+        _ptr(sorted_scattered_idxs), _ptr(expert_offsets), _ptr(DW), DW.stride(0), DW.stride(2), N_out, K_in, E,
     )
+    # the few-token entry point also takes the number of rows: it picks the shape of a workgroup's tile of dW by it
+    check(getattr(lib, name)(*operands, *((M,) if few else ()), _code(X), _stream(X)), name)
 
 
 @torch.library.custom_op("xma_rocm::expert_column_sums", mutates_args={"out"})

@@ -240,20 +240,21 @@ XMA_API int xma_rocm_group_bwd_W(const void *DY, int64_t lddy, int dy_grouped, i
                          int dtype, void *stream);
 
 /*
- * xma_rocm_group_bwd_W for the few-token regime (same arguments and limits, same result up to the order of the fp32
- * sums; bf16 / fp16 only; a scaled row of DY is rounded to the operand type before it is multiplied, as a scaled grouped
- * copy would hold it).  One workgroup per 128 x 128 tile of DW[e]; the expert's rows are the K dimension of its MFMAs,
- * 32 at a time: with a handful of rows per expert the launch runs at the rate of a fill of DW, where
- * xma_rocm_group_bwd_W spends a prologue, one K step and an epilogue per 256 x 256 tile.  Correct for any number of rows;
- * more rows are more passes over two 8 KB operand tiles, so it leads until the loads outweigh the stores (the torch ops
- * take it up to 128 rows per expert on average).  No counterpart in the reference (its kernel is the same for every
- * size).
+ * xma_rocm_group_bwd_W for the few-token regime (same arguments and limits plus M, same result up to the order of the
+ * fp32 sums; bf16 / fp16 only; a scaled row of DY is rounded to the operand type before it is multiplied, as a scaled
+ * grouped copy would hold it).  M = rows in all (the length of the grouped order), which picks the shape of a
+ * workgroup's tile of DW[e]: 64 x 256 up to 24 rows per expert on average, 128 x 128 beyond or when M <= 0 (not known).
+ * The expert's rows are the K dimension of the tile's MFMAs, 32 at a time: with a handful of rows per expert the launch
+ * runs at the rate of a fill of DW, where xma_rocm_group_bwd_W spends a prologue, one K step and an epilogue per
+ * 256 x 256 tile.  Correct for any number of rows; more rows are more passes over two small operand tiles, so it leads
+ * until the loads outweigh the stores (the torch ops take it up to 128 rows per expert on average).  No counterpart in
+ * the reference (its kernel is the same for every size).
  */
 XMA_API int xma_rocm_group_bwd_W_few_rows(const void *DY, int64_t lddy, int dy_grouped, int32_t dy_fan_out,
                                   const void *dy_scale, const void *X, int64_t ldx, int x_grouped, int32_t x_fan_out,
                                   const int64_t *sorted_scattered_idxs, const int64_t *expert_offsets, void *DW,
                                   int64_t dw_expert_stride, int64_t lddw, int32_t N_out, int32_t K_in,
-                                  int32_t num_experts, int dtype, void *stream);
+                                  int32_t num_experts, int64_t M, int dtype, void *stream);
 
 /*
  * Gather copy: out[n, :] = A[idx[n] / fan_out, :] * (coeff ? coeff[idx[n]] : 1), n < M.

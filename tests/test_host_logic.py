@@ -88,10 +88,10 @@ def test_argument_errors_are_reported_before_any_launch():
     assert ws(64, 2048, 8192, 8, 0, 0) == 4 * 64 * 2048 * 4  # small MFMA tile cut into 4 ranges of K
     assert ws(0, 64, 64, 2, 1, 0) == 0
     dw = lib.xma_rocm_group_bwd_W_few_rows
-    assert dw(p, 64, 1, 1, None, p, 64, 1, 1, p, p, p, 64 * 64, 64, 64, 64, 2, 2, None) == -2  # fp32
-    assert dw(p, 64, 1, 1, None, p, 60, 1, 1, p, p, p, 64 * 64, 64, 64, 64, 2, 0, None) == -2  # ldx % 8
-    assert dw(p, 60, 1, 1, None, p, 64, 1, 1, p, p, p, 64 * 64, 64, 64, 64, 2, 0, None) == -2  # lddy % 8
-    assert dw(None, 64, 1, 1, None, p, 64, 1, 1, p, p, p, 64 * 64, 64, 64, 64, 2, 0, None) == -1
+    assert dw(p, 64, 1, 1, None, p, 64, 1, 1, p, p, p, 64 * 64, 64, 64, 64, 2, 4, 2, None) == -2  # fp32
+    assert dw(p, 64, 1, 1, None, p, 60, 1, 1, p, p, p, 64 * 64, 64, 64, 64, 2, 4, 0, None) == -2  # ldx % 8
+    assert dw(p, 60, 1, 1, None, p, 64, 1, 1, p, p, p, 64 * 64, 64, 64, 64, 2, 4, 0, None) == -2  # lddy % 8
+    assert dw(None, 64, 1, 1, None, p, 64, 1, 1, p, p, p, 64 * 64, 64, 64, 64, 2, 4, 0, None) == -1
     # empty problems are accepted without touching a pointer
     assert few(None, 64, None, 64 * 64, 64, 0, None, None, None, 64, None, 0, None, 0, None, None, 0, 0, 64, 64, 2, 1, 1, 1, 0, 0, None, 0, None) == 0
     assert lib.xma_rocm_combine(None, 8, None, None, 8, 0, 2, 16, 0, None) == 0
