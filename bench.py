@@ -1,6 +1,6 @@
 """MoE hot-path benchmark on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c5|c2|small_t|copy|mfma_peak|library_gemm]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload c3|c4|c5|c2|small_t|few_rows|copy|mfma_peak|library_gemm]
 
 Default workload: the Mixtral-shaped layer (T=8192, H=4096, I=14336, E=8, top-2, packed SwiGLU, bf16).
 A step is one forward + backward of the layer behind the gate: router (top-k + softmax + expert ids from the
@@ -541,10 +541,11 @@ def _other_configs(args) -> dict:
 
 def run_small_t(args):
     """Latency of one forward + backward of the expert computation with a handful of tokens, the case the reference's
-    own test runs (7 tokens, tests/layers/moe_test.py:107) at its two size points (moe_test.py:26-53), and with 64,
-    192 and 384 tokens (decoding batches): eager, and replayed from a HIP graph (no host launch overhead), beside the time the weights touched by the
-    step need to stream through HBM once per use at 8 TB/s (forward, dX and the dW store: three uses); and the forward
-    alone (router, routing, both projections, combine) from a graph, the step of a decoding loop."""
+    own test runs (7 tokens, tests/layers/moe_test.py:107) at its two size points (moe_test.py:26-53), with 64, 192 and
+    384 tokens (decoding batches), and C4's layer (64 experts) at 64, 512 and 1024 tokens: eager, replayed from a HIP
+    graph (no host launch overhead), and the same graph with the 256 x 256 kernels only, beside the time the weights
+    touched by the step need to stream through HBM once per use at 8 TB/s (forward, dX and the dW store: three uses);
+    and the forward alone (router, routing, both projections, combine) from a graph, the step of a decoding loop."""
     from xma import KernelBackend, set_seed
     from xma.functional import swiglu_packed
     from xma.layers import MoE
@@ -552,10 +553,12 @@ def run_small_t(args):
     from xma.rocm import ops as _ops
 
     res = {}
-    for E, k, H, I in ((8, 2, 2048, 8192), (128, 8, 576, 256)):
+    # the reference test's two size points at 7 tokens and at decoding batches; C4's layer at three batch sizes
+    for E, k, H, I, Ts in ((8, 2, 2048, 8192, (7, 64, 192, 384)), (128, 8, 576, 256, (7, 64, 192, 384)),
+                           (64, 6, 2048, 1408, (64, 512, 1024))):
         set_seed(0)
         moe = MoE(E, k, H, I, swiglu_packed, True, add_bias=False, std=0.02).to(torch.bfloat16).cuda()
-        for T in (7, 64, 192, 384):
+        for T in Ts:
             if args.only not in f"E{E}_k{k}_H{H}_I{I}_T{T}":
                 continue
             x = torch.randn(T, H, device="cuda").to(torch.bfloat16).requires_grad_()
@@ -582,6 +585,18 @@ def run_small_t(args):
             with torch.cuda.graph(g_):
                 step()
             graph_ms = _time_gpu(g_.replay, max(args.steps, 20), warmup=5)
+            few_rows_max, _ops.FEW_ROWS_MAX = _ops.FEW_ROWS_MAX, 0  # the same step through the 256 x 256 kernels only
+            try:
+                step()
+                torch.cuda.synchronize()
+                gt = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(gt):
+                    step()
+                tiles_only_ms = _time_gpu(gt.replay, max(args.steps, 20), warmup=5)
+            finally:
+                _ops.FEW_ROWS_MAX = few_rows_max
+            del gt
+
             def forward_only():
                 with torch.no_grad():
                     w, ids = R.router_topk(lg, k, ids_dtype=torch.int32)
@@ -598,7 +613,8 @@ def run_small_t(args):
             wbytes = (2 * I * H + H * I) * 2  # both matrices of one expert
             stream_bytes = 2 * touched * wbytes + E * wbytes  # forward and dX read the touched experts, dW writes all
             res[f"E{E}_k{k}_H{H}_I{I}_T{T}"] = {
-                "eager_ms": round(eager_ms, 4), "graph_ms": round(graph_ms, 4), "experts_touched": touched,
+                "eager_ms": round(eager_ms, 4), "graph_ms": round(graph_ms, 4),
+                "mfma_tiles_only_graph_ms": round(tiles_only_ms, 4), "experts_touched": touched,
                 "gemm_kernels": {form: ("few_rows" if _ops._few_rows(T * k, E, torch.bfloat16, form) else "mfma tiles") for form in _ops.FEW_ROWS_PER_EXPERT},
                 "forward_only_graph_ms": round(fwd_graph_ms, 4),
                 "forward_only_weight_stream_ms_at_8TBs": round(touched * wbytes / PEAK_HBM_GBS / 1e6, 4),
@@ -617,6 +633,71 @@ def run_small_t(args):
                                              "experts, combine and all gradients) at T = 7, 64, 192 and 384 on the reference test's two "
                                              "size points, bf16 packed SwiGLU"},
                       "results": res}))
+
+
+def run_few_rows(args):
+    """The six grouped GEMMs of one layer (E = 8, H = 2048, I = 8192, bf16) with R rows in every expert, R from 1 to 192:
+    microseconds per launch from a graph of five launches, through the 256 x 256 MFMA kernels and through the kernels of
+    the few-token regime (csrc/few_rows.hip), whatever the dispatch rule of the ops would pick.  Where the two columns
+    cross is where the rule's limits come from (with routed, uneven tokens they sit lower: --workload small_t)."""
+    from xma.rocm import ops
+
+    E, H, I, dt = 8, 2048, 8192, torch.bfloat16
+    g = torch.Generator(device="cuda").manual_seed(0)
+    W1 = (torch.randn(E, 2 * I, H, device="cuda", generator=g) * 0.02).to(dt)
+    W2 = (torch.randn(E, H, I, device="cuda", generator=g) * 0.02).to(dt)
+    dW1, dW2 = torch.empty_like(W1), torch.empty_like(W2)
+
+    def graph_us(fn):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        gr = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(gr):
+            for _ in range(5):
+                fn()
+        return _time_gpu(gr.replay, 4, warmup=1) / 5 * 1e3
+
+    res = {}
+    for R in (1, 2, 4, 8, 16, 32, 64, 96, 128, 192):
+        M = R * E
+        ids = torch.arange(E, device="cuda").repeat_interleave(R)[torch.randperm(M, device="cuda", generator=g)]
+        se, ss = ids.sort(stable=True)
+        offs = torch.bincount(se, minlength=E).cumsum(0)
+        x, dy = (torch.randn(M, H, device="cuda", generator=g).to(dt) for _ in range(2))
+        hg = torch.randn(M, I, device="cuda", generator=g).to(dt)
+        dzg, zg = (torch.randn(M, 2 * I, device="cuda", generator=g).to(dt) for _ in range(2))
+        w = torch.rand(M, device="cuda", generator=g).to(dt)
+        z, dz = torch.empty(M, 2 * I, device="cuda", dtype=dt), torch.empty(M, 2 * I, device="cuda", dtype=dt)
+        h, out = torch.empty(M, I, device="cuda", dtype=dt), torch.empty(M, H, device="cuda", dtype=dt)
+        gemms = {
+            "up_swiglu": lambda: ops.up_projection_swiglu_rocm(x, W1.permute(0, 2, 1), ss, offs, z, h, 1, None),
+            "down": lambda: ops.scatter2scatter_rocm(hg, W2.permute(0, 2, 1), ss, offs, out, w, 1, True, False),
+            "dx1": lambda: ops.scatter2scatter_rocm(dzg, W1, ss, offs, out, None, 1, True, False),
+            "dx2_swiglu_bwd": lambda: ops.down_projection_dx_swiglu_rocm(dy, W2, ss, offs, zg, dz, w, 1),
+            "dw1": lambda: ops.group_bwd_W_rocm(dzg, x, ss, offs, dW1.permute(0, 2, 1), None, 0, 1),
+            "dw2": lambda: ops.group_bwd_W_rocm(dy, hg, ss, offs, dW2.permute(0, 2, 1), None, 1, 0),
+        }
+        row = {}
+        for name, fn in gemms.items():
+            saved = (ops.FEW_ROWS_MAX, ops.FEW_ROWS_PER_EXPERT)
+            try:
+                ops.FEW_ROWS_MAX = 0  # the 256 x 256 kernels
+                tiles = graph_us(fn)
+                ops.FEW_ROWS_MAX, ops.FEW_ROWS_PER_EXPERT = 1 << 20, dict.fromkeys(saved[1], 1 << 20)  # the few-token kernels
+                few = graph_us(fn)
+            finally:
+                ops.FEW_ROWS_MAX, ops.FEW_ROWS_PER_EXPERT = saved
+            row[name] = {"mfma_tiles_us": round(tiles, 1), "few_rows_us": round(few, 1)}
+        res[f"R{R}"] = row
+        print(f"R={R}: " + "  ".join(f"{n} {v['mfma_tiles_us']:.0f}/{v['few_rows_us']:.0f}" for n, v in row.items()), file=sys.stderr, flush=True)
+    first = res["R1"]["up_swiglu"]["few_rows_us"]
+    print(json.dumps({"metric": "few_rows_up_projection_us", "value": first, "unit": "us", "n_gpus": 1, "steps": args.steps,
+                      "warmup": args.warmup, "ms_per_step": first / 1e3, "higher_is_better": False, "dtype": "bf16",
+                      "data": "synthetic",
+                      "config": {"workload": "few_rows: the six grouped GEMMs of a layer of 8 experts, H = 2048, I = 8192, with R "
+                                             "rows in every expert, 256 x 256 MFMA kernels beside the few-token kernels"},
+                      "rules": {"rows_per_expert": dict(ops.FEW_ROWS_PER_EXPERT), "rows": ops.FEW_ROWS_MAX}, "results": res}))
 
 
 def run_copy(args):
@@ -702,7 +783,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=10)
     ap.add_argument("--warmup", type=int, default=3)
-    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "small_t", "copy", "mfma_peak", "library_gemm"])
+    ap.add_argument("--workload", default="c3", choices=["c2", "c3", "c4", "c5", "small_t", "few_rows", "copy", "mfma_peak", "library_gemm"])
     ap.add_argument("--zipf", action="store_true", help="c2 only: Zipf(s=1.1) ids instead of uniform")
     ap.add_argument("--kernel-iters", type=int, default=5)
     ap.add_argument("--cpu-fraction", type=int, default=1, help="CPU baseline runs on T / this many tokens")
@@ -725,6 +806,8 @@ def main():
         run_library_gemm(args)
     elif args.workload == "small_t":
         run_small_t(args)
+    elif args.workload == "few_rows":
+        run_few_rows(args)
     elif args.workload == "c2":
         print(json.dumps(measure_routing(args, args.zipf)))
     else:
