@@ -610,9 +610,11 @@ __global__ __launch_bounds__(FR_THREADS, MB == 1 ? 4 : 2) void fr_tile_kernel(co
     }
 }
 
-// W[e] as (K, N), or more than a pass or two of the vector kernel per expert -> the small MFMA tile
-inline bool fr_takes_tile(int64_t M, int E, int w_is_kn) {
-    return w_is_kn || M > (int64_t)FR_NT_VALU_ROWS_PER_EXPERT * E || M > FR_NT_VALU_ROWS;
+// W[e] as (K, N), more than a pass or two of the vector kernel per expert, or rows of W shorter than the 4 KB a wave of
+// the vector kernel takes at a time -> the small MFMA tile (128 experts of H = 576, I = 256, 7 tokens: forward 0.036
+// instead of 0.045 ms with it; 8 experts of H = 2048, I = 8192: 0.161 instead of 0.155)
+inline bool fr_takes_tile(int64_t M, int K, int E, int w_is_kn) {
+    return w_is_kn || M > (int64_t)FR_NT_VALU_ROWS_PER_EXPERT * E || M > FR_NT_VALU_ROWS || K < FR_NT_PIECE;
 }
 
 // passes of 128 rows once many experts have more than 32: two workgroups per compute unit instead of four (registers
@@ -659,7 +661,7 @@ template <typename T, int WT, int EPI> int fr_launch_tile(const FwdArgs &a, floa
 
 template <typename T, int EPI> int fr_launch_epi(const FwdArgs &a, int w_is_kn, float *part, hipStream_t st) {
     int rc;
-    if (fr_takes_tile(a.M, a.E, w_is_kn)) return w_is_kn ? fr_launch_tile<T, 1, EPI>(a, part, st) : fr_launch_tile<T, 0, EPI>(a, part, st);
+    if (fr_takes_tile(a.M, a.K, a.E, w_is_kn)) return w_is_kn ? fr_launch_tile<T, 1, EPI>(a, part, st) : fr_launch_tile<T, 0, EPI>(a, part, st);
     // one pair of rows per wave instead of four where the rows are short or the launch would have few workgroups
     const int rows_per_wg = (a.K >= 2048 && (int64_t)(a.N / FR_NT_ROWS) * a.E >= 2048) ? FR_NT_ROWS : 8;
     const dim3 grid((a.N + rows_per_wg - 1) / rows_per_wg, a.E);
@@ -685,7 +687,7 @@ extern "C" size_t xma_rocm_scatter2scatter_few_rows_workspace_bytes(int64_t M, i
                                                                     int epilogue) {
     if (M <= 0 || N <= 0 || K <= 0 || E <= 0) return 0;
     int S;
-    if (fr_takes_tile(M, E, w_is_kn)) { // the small MFMA tile, cut along K or not
+    if (fr_takes_tile(M, K, E, w_is_kn)) { // the small MFMA tile, cut along K or not
         S = fr_tile_splits(N, K, E, w_is_kn);
         if (S == 1) return 0;
     } else if (epilogue == XMA_ROCM_EPI_SWIGLU_BWD) {

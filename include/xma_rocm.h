@@ -199,9 +199,9 @@ XMA_API int xma_rocm_down_projection_dx_swiglu(const void *dY, int64_t lddy, con
  * xma_rocm_scatter2scatter_bias / xma_rocm_down_projection_dx_swiglu for the few-token regime: the same arguments
  * (aux2 = the scaled activations of the latter, or NULL), the same results up to the order of the fp32 sums, bf16 / fp16
  * only.  With a handful of rows per expert the product is a stream over the weights.  W[e] as (N, K), up to 2 rows per
- * expert on average (and 64 in all): vector FMAs, a wave reads two rows of W with its lanes along K.  Everything else: a
- * small MFMA tile (32 rows of the expert x 128 output columns and four workgroups per compute unit, or 128 rows and two
- * from 24 rows per expert on average), cut along K where N alone gives too few workgroups.
+ * expert on average (and 64 in all), K at least 2048: vector FMAs, a wave reads two rows of W with its lanes along K.
+ * Everything else: a small MFMA tile (32 rows of the expert x 128 output columns and four workgroups per compute unit,
+ * or 128 rows and two from 24 rows per expert on average), cut along K where N alone gives too few workgroups.
  * Whatever does not finish in one kernel sums through the workspace (xma_rocm_scatter2scatter_few_rows_workspace_bytes
  * bytes for the same M, N, K, num_experts, w_is_kn and epilogue; 0 = none needed, pass NULL) to a small kernel that
  * applies the bias and the epilogue with the arithmetic of the MFMA kernels.  Limits: M and E at most 65535, N * ldw

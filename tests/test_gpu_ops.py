@@ -342,6 +342,7 @@ FEW_ROWS_CASES = [
     (9, 5, 3, 4104, 24, (0, 4)),  # a row of W as (N, K) is 513 pieces of 16 bytes: two passes of a wave and one lane more
     (7, 8, 2, 512, 8192, ()),  # long K for the down-projection and dX1: both cut into ranges of K
     (5, 2, 2, 64, 3200, ()),  # down-projection: 25 K steps in 6 ranges of 5, of which only 5 hold a step
+    (5, 8, 2, 2056, 40, (3,)),  # one or two rows per expert and rows of W longer than 4 KB: the vector kernel for the up-projection
 ]
 
 

@@ -80,8 +80,9 @@ def test_argument_errors_are_reported_before_any_launch():
     assert few(p, 64, p, 64 << 26, 1 << 26, 0, p, p, p, 64, None, 0, None, 0, None, None, 0, 4, 64, 64, 2, 1, 1, 1, 0, 0, None, 0, None) == -2
     assert b"N * ldw" in lib.xma_rocm_last_error()
     ws = lib.xma_rocm_scatter2scatter_few_rows_workspace_bytes  # (M, N, K, E, w_is_kn, epilogue)
-    assert ws(4, 64, 64, 2, 0, 0) == 0 and ws(4, 64, 64, 2, 0, 1) == 0  # the vector kernel finishes the job itself (2 rows per expert)
-    assert ws(4, 64, 64, 2, 0, 2) == 4 * 64 * 4  # SwiGLU backward: through the epilogue kernel
+    assert ws(4, 64, 2048, 2, 0, 0) == 0 and ws(4, 64, 2048, 2, 0, 1) == 0  # the vector kernel finishes the job itself (2 rows per expert)
+    assert ws(4, 64, 2048, 2, 0, 2) == 4 * 64 * 4  # SwiGLU backward: through the epilogue kernel
+    assert ws(4, 64, 64, 2, 0, 2) == 0  # short rows of W: the small tile, one K range, epilogue in the kernel
     assert ws(4, 64, 16384, 2, 1, 0) == 32 * 4 * 64 * 4  # W as (K, N): the small tile at any number of rows, 32 ranges of K
     assert ws(64, 2048, 16384, 8, 1, 0) == 4 * 64 * 2048 * 4 and ws(64, 8192, 2048, 8, 1, 2) == 0  # small tile: 4 ranges of K; none
     assert ws(64, 16384, 2048, 8, 0, 1) == 0  # small MFMA tile, enough workgroups from N alone
